@@ -1,0 +1,78 @@
+// In-place paged append of new K/V rows, rotary applied to K.
+//
+// Semantics are those the reference documents for flash_attn_with_kvcache
+// (flash_attn_npu/flash_attn_npu_interface.py:1460-1474,1508-1513,1527-1530) and its host code
+// accepts but drops (csrc/ascend910/flash_attn_npu/flash_api.cpp:422-427):
+//   p = cache_seqlens[b] + t;  k_cache[block_table[b][p / page]][p % page][h] = rope(k_new[b][t][h], p)
+//   v_cache[...] = v_new[b][t][h].
+// Rotary arithmetic: operands widened to fp32, two separately rounded products and one separately
+// rounded add/sub (never a fused multiply-add), result rounded to nearest-even in the cache dtype,
+// so the written bytes can be compared bit-for-bit with a host computation.
+#include "fa_device.h"
+#include "fa_kernels.h"
+
+namespace fa {
+
+// grid: (Hk, Snew, B); block: 64 threads striding over the element pairs of one head row
+template <typename T>
+__global__ void __launch_bounds__(64) append_kv_kernel(const AppendParams p) {
+    const int h = blockIdx.x;
+    const int t = blockIdx.y;
+    const int b = blockIdx.z;
+    const int pos = p.cache_seqlens[b] + t;
+    if (pos < 0) return;
+    const int page = pos / p.page_size;
+    if (page >= p.max_blocks) return;   // no capacity: nothing is written
+    const int blk = p.block_table[(int64_t)b * p.bt_stride_b + page];
+    if (blk < 0 || blk >= p.num_blocks) return;
+    const int inpage = pos - page * p.page_size;
+
+    uint16_t *kdst = reinterpret_cast<uint16_t *>(p.k_cache) + (int64_t)blk * p.k_stride_block +
+                     (int64_t)inpage * p.k_stride_row + (int64_t)h * p.k_stride_h;
+    uint16_t *vdst = reinterpret_cast<uint16_t *>(p.v_cache) + (int64_t)blk * p.v_stride_block +
+                     (int64_t)inpage * p.v_stride_row + (int64_t)h * p.v_stride_h;
+    const uint16_t *ksrc = reinterpret_cast<const uint16_t *>(p.k_new) + (int64_t)b * p.kn_stride_b +
+                           (int64_t)t * p.kn_stride_s + (int64_t)h * p.kn_stride_h;
+    const uint16_t *vsrc = reinterpret_cast<const uint16_t *>(p.v_new) + (int64_t)b * p.vn_stride_b +
+                           (int64_t)t * p.vn_stride_s + (int64_t)h * p.vn_stride_h;
+
+    const uint16_t *cosT = reinterpret_cast<const uint16_t *>(p.rotary_cos);
+    const uint16_t *sinT = reinterpret_cast<const uint16_t *>(p.rotary_sin);
+    const int rot = (cosT != nullptr) ? p.rotary_dim : 0;
+    const int half = rot >> 1;
+    const int rpos = min(pos, p.seqlen_ro - 1);
+
+    for (int c = threadIdx.x; c < p.headdim_qk / 2; c += 64) {
+        int d1, d2;
+        if (c < half) {
+            d1 = p.rotary_interleaved ? 2 * c : c;
+            d2 = p.rotary_interleaved ? 2 * c + 1 : c + half;
+        } else {
+            d1 = rot + 2 * (c - half);
+            d2 = d1 + 1;
+        }
+        uint16_t o1 = ksrc[d1], o2 = ksrc[d2];
+        if (c < half) {
+            const float cs = to_float<T>(cosT[(int64_t)rpos * half + c]);
+            const float sn = to_float<T>(sinT[(int64_t)rpos * half + c]);
+            const float x1 = to_float<T>(o1), x2 = to_float<T>(o2);
+            o1 = from_float<T>(__fsub_rn(__fmul_rn(x1, cs), __fmul_rn(x2, sn)));
+            o2 = from_float<T>(__fadd_rn(__fmul_rn(x1, sn), __fmul_rn(x2, cs)));
+        }
+        kdst[d1] = o1;
+        kdst[d2] = o2;
+    }
+    if ((p.headdim_qk & 1) && threadIdx.x == 0) kdst[p.headdim_qk - 1] = ksrc[p.headdim_qk - 1];
+    for (int d = threadIdx.x; d < p.headdim_v; d += 64) vdst[d] = vsrc[d];
+}
+
+hipError_t launch_append_kv(const AppendParams &p, int dtype, hipStream_t stream) {
+    dim3 grid(p.nheads_k, p.seqlen_new, p.batch);
+    if (dtype == 0)
+        hipLaunchKernelGGL(append_kv_kernel<BF16>, grid, dim3(64), 0, stream, p);
+    else
+        hipLaunchKernelGGL(append_kv_kernel<FP16>, grid, dim3(64), 0, stream, p);
+    return hipGetLastError();
+}
+
+}  // namespace fa

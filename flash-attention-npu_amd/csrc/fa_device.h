@@ -1,0 +1,104 @@
+// Device-side helpers shared by the gfx950 attention kernels: 16-bit element traits,
+// MFMA wrappers for the two I/O dtypes, packing, wave-level exchanges.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace fa {
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
+typedef __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16 half8_t;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float float4_t;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float float16_t;
+typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4_t;
+
+struct BF16 {};
+struct FP16 {};
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+// ---- scalar conversions (round-to-nearest-even) ------------------------------------------
+template <typename T> __device__ __forceinline__ float to_float(uint16_t bits);
+template <> __device__ __forceinline__ float to_float<BF16>(uint16_t bits) {
+    return __uint_as_float(static_cast<uint32_t>(bits) << 16);
+}
+template <> __device__ __forceinline__ float to_float<FP16>(uint16_t bits) {
+    _Float16 h;
+    __builtin_memcpy(&h, &bits, 2);
+    return static_cast<float>(h);
+}
+
+template <typename T> __device__ __forceinline__ uint16_t from_float(float f);
+template <> __device__ __forceinline__ uint16_t from_float<BF16>(float f) {
+    __bf16 h = static_cast<__bf16>(f);   // RNE on gfx950 (v_cvt_pk_bf16_f32)
+    uint16_t b;
+    __builtin_memcpy(&b, &h, 2);
+    return b;
+}
+template <> __device__ __forceinline__ uint16_t from_float<FP16>(float f) {
+    _Float16 h = static_cast<_Float16>(f);
+    uint16_t b;
+    __builtin_memcpy(&b, &h, 2);
+    return b;
+}
+
+// two floats -> one dword holding (lo = a, hi = b) in the 16-bit type
+template <typename T> __device__ __forceinline__ uint32_t pack2(float a, float b) {
+    return static_cast<uint32_t>(from_float<T>(a)) | (static_cast<uint32_t>(from_float<T>(b)) << 16);
+}
+
+// ---- MFMA 16x16x32: D(16x16) += A(16x32) * B(32x16), 16-bit inputs, fp32 accumulate -------
+// Lane l holds A[l%16][8*(l/16) .. +7], B[8*(l/16) .. +7][l%16], D[4*(l/16) + r][l%16], r = 0..3.
+template <typename T>
+__device__ __forceinline__ float4_t mfma16(const u32x4_t &a, const u32x4_t &b, const float4_t &c);
+template <>
+__device__ __forceinline__ float4_t mfma16<BF16>(const u32x4_t &a, const u32x4_t &b, const float4_t &c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c,
+                                                   0, 0, 0);
+}
+template <>
+__device__ __forceinline__ float4_t mfma16<FP16>(const u32x4_t &a, const u32x4_t &b, const float4_t &c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a), __builtin_bit_cast(half8_t, b), c, 0,
+                                                  0, 0);
+}
+
+// ---- MFMA 32x32x16: D(32x32) += A(32x16) * B(16x32) ---------------------------------------
+// Lane l holds A[l%32][8*(l/32) .. +7], B[8*(l/32) .. +7][l%32],
+// D[8*(r/4) + 4*(l/32) + r%4][l%32], r = 0..15.
+template <typename T>
+__device__ __forceinline__ float16_t mfma32(const u32x4_t &a, const u32x4_t &b, const float16_t &c);
+template <>
+__device__ __forceinline__ float16_t mfma32<BF16>(const u32x4_t &a, const u32x4_t &b, const float16_t &c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c,
+                                                   0, 0, 0);
+}
+template <>
+__device__ __forceinline__ float16_t mfma32<FP16>(const u32x4_t &a, const u32x4_t &b, const float16_t &c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, a), __builtin_bit_cast(half8_t, b), c, 0,
+                                                  0, 0);
+}
+
+// ---- wave-level exchanges -------------------------------------------------------------------
+__device__ __forceinline__ float xor_shuffle(float v, int lane_mask) { return __shfl_xor(v, lane_mask, 64); }
+
+// max / sum over the four lanes {n, n+16, n+32, n+48}
+__device__ __forceinline__ float quad_rows_max(float v) {
+    v = fmaxf(v, xor_shuffle(v, 16));
+    v = fmaxf(v, xor_shuffle(v, 32));
+    return v;
+}
+__device__ __forceinline__ float quad_rows_sum(float v) {
+    v += xor_shuffle(v, 16);
+    v += xor_shuffle(v, 32);
+    return v;
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+
+// 16-byte global load / store through plain vector types
+__device__ __forceinline__ u32x4_t load16(const void *p) { return *reinterpret_cast<const u32x4_t *>(p); }
+__device__ __forceinline__ void store16(void *p, const u32x4_t &v) { *reinterpret_cast<u32x4_t *>(p) = v; }
+
+}  // namespace fa

@@ -1,0 +1,98 @@
+// Kernel parameter blocks and host-side launchers of the gfx950 attention kernels.
+// The C ABI (fa_rocm_api.cpp) fills these from fa_kvcache_args / fa_varlen_args.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace fa {
+
+// Parameters of the paged decode kernel and of the split-KV combine kernel.  Passed by value
+// (the counterpart of FAInferTilingData, csrc/ascend910/flash_attn_npu/tilingdata.h:34-62,
+// which the reference uploads with a host-to-device copy on every call).
+struct DecodeParams {
+    const void *q;
+    void *out;
+    float *lse;
+    const void *k_cache;
+    const void *v_cache;
+    const float *k_scale;
+    const float *v_scale;
+    const void *rotary_cos;
+    const void *rotary_sin;
+    const int32_t *cache_seqlens;
+    const int32_t *block_table;
+    float *o_partial;    // (B, Hk, nsplits, rows, Dv) fp32, each normalised by its own sum
+    float *lse_partial;  // (B, Hk, nsplits, rows)     fp32, base-2 log-sum-exp, -inf when empty
+    int32_t batch, seqlen_q, nheads, nheads_k, group, rows;  // rows = seqlen_q * group
+    int32_t seqlen_new, num_blocks, page_size, max_blocks;
+    int32_t rotary_dim, seqlen_ro, rotary_interleaved, rotary_per_token;
+    int64_t q_stride_b, q_stride_s, q_stride_h;
+    int64_t o_stride_b, o_stride_s, o_stride_h;
+    int64_t k_stride_block, k_stride_row, k_stride_h;
+    int64_t v_stride_block, v_stride_row, v_stride_h;
+    int64_t ks_stride_block, ks_stride_row;
+    int64_t bt_stride_b;
+    float scale_log2;      // softmax_scale * log2(e)            (softcap off)
+    float softcap_pre;     // softmax_scale / softcap            (softcap on)
+    float softcap_post;    // softcap * log2(e)
+    int32_t causal, window_left, window_right;
+    int32_t nsplits, split_keys;
+};
+
+struct AppendParams {
+    void *k_cache;
+    void *v_cache;
+    const void *k_new;
+    const void *v_new;
+    const void *rotary_cos;
+    const void *rotary_sin;
+    const int32_t *cache_seqlens;
+    const int32_t *block_table;
+    int32_t batch, seqlen_new, nheads_k, headdim_qk, headdim_v;
+    int32_t num_blocks, page_size, max_blocks;
+    int32_t rotary_dim, seqlen_ro, rotary_interleaved;
+    int64_t k_stride_block, k_stride_row, k_stride_h;
+    int64_t v_stride_block, v_stride_row, v_stride_h;
+    int64_t kn_stride_b, kn_stride_s, kn_stride_h;
+    int64_t vn_stride_b, vn_stride_s, vn_stride_h;
+    int64_t bt_stride_b;
+};
+
+// Parameters of the tiled (MFMA) forward used for varlen prefill and for kvcache calls whose
+// query block does not fit the decode kernel.
+struct PrefillParams {
+    const void *q;
+    const void *k;
+    const void *v;
+    void *out;
+    float *lse;
+    const int32_t *cu_seqlens_q;   // NULL: fixed seqlen_q per batch row (kvcache layout)
+    const int32_t *cu_seqlens_k;   // dense K/V only
+    const int32_t *seqused_k;      // paged: keys per row (cache_seqlens)
+    const int32_t *block_table;    // NULL: dense K/V
+    int32_t batch, nheads, nheads_k, group;
+    int32_t seqlen_q_fixed, seqlen_k_add;   // kvcache layout: Sq per row, keys appended this call
+    int32_t max_seqlen_q, total_q;
+    int32_t page_size, max_blocks, num_blocks;
+    int64_t q_stride_b, q_stride_t, q_stride_h;
+    int64_t o_stride_b, o_stride_t, o_stride_h;
+    int64_t k_stride_t, k_stride_h, k_stride_block;
+    int64_t v_stride_t, v_stride_h, v_stride_block;
+    int64_t bt_stride_b;
+    int64_t lse_stride_b, lse_stride_h;     // lse index = b*stride_b + h*stride_h + token
+    float scale_log2, softcap_pre, softcap_post;
+    int32_t causal, window_left, window_right;
+    int32_t num_m_blocks;                   // q tiles per sequence (grid.x)
+};
+
+// dtype: 0 = bf16, 1 = fp16 (enum fa_dtype).  All return hipError_t of the launch.
+hipError_t launch_append_kv(const AppendParams &p, int dtype, hipStream_t stream);
+hipError_t launch_decode_paged(const DecodeParams &p, int dtype, int headdim, hipStream_t stream);
+hipError_t launch_splitkv_combine(const DecodeParams &p, int dtype, int headdim_v, hipStream_t stream);
+hipError_t launch_decode_mla_i8(const DecodeParams &p, int dtype, hipStream_t stream);
+hipError_t launch_prefill(const PrefillParams &p, int dtype, int headdim, hipStream_t stream);
+
+// Largest query block (seqlen_q * group) the decode kernel packs into one workgroup.
+constexpr int kDecodeMaxRows = 64;
+
+}  // namespace fa

@@ -1,0 +1,431 @@
+// C ABI of the library: argument validation, split planning, workspace sizing and kernel
+// sequencing for one flash_attn_with_kvcache / flash_attn_varlen_func forward call.
+//
+// Host-side counterpart of the reference's mha_fwd_kvcache and mha_varlen_fwd
+// (csrc/ascend910/flash_attn_npu/flash_api.cpp:356-637 and :848-1089).  Unlike those it never
+// copies cache_seqlens to the host, uploads no mask and no tiling block: every decision made here
+// depends on shapes only, per-row lengths are read by the kernels.
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "../../include/fa_rocm.h"
+#include "fa_kernels.h"
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+constexpr float kLog2e = 1.4426950408889634f;
+
+int device_cus() {
+    // cached per host thread and device; a property query, not an allocation
+    thread_local int cached_dev = -1;
+    thread_local int cached_cus = 0;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return -1;
+    if (dev != cached_dev) {
+        int cus = 0;
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return -1;
+        cached_dev = dev;
+        cached_cus = cus;
+    }
+    return cached_cus;
+}
+
+bool is_mla_i8(const fa_kvcache_args *a) { return a->kv_dtype == FA_INT8; }
+
+// Upper bound of the live key range any row can have, from shapes alone.
+int64_t live_keys_bound(const fa_kvcache_args *a) {
+    int64_t cap = (int64_t)a->max_blocks_per_seq * a->page_size;
+    const int wr = a->causal ? 0 : a->window_right;
+    if (a->window_left >= 0) {
+        // keys in [off - wl, Sq-1 + off + max(wr, 0)] plus alignment slack of one 32-key chunk
+        int64_t span = (int64_t)a->window_left + a->seqlen_q + (wr > 0 ? wr : 0) + 32;
+        if (span < cap) cap = span;
+    }
+    return cap > 0 ? cap : 1;
+}
+
+}  // namespace
+
+extern "C" {
+
+int fa_rocm_abi_version(void) { return FA_ROCM_ABI_VERSION; }
+
+const char *fa_rocm_last_error(void) { return g_err; }
+
+size_t fa_rocm_sizeof_kvcache_args(void) { return sizeof(fa_kvcache_args); }
+
+size_t fa_rocm_sizeof_varlen_args(void) { return sizeof(fa_varlen_args); }
+
+int fa_rocm_num_cus(void) { return device_cus(); }
+
+int fa_rocm_kvcache_validate(const fa_kvcache_args *a) {
+    if (!a) return fail(FA_ERR_NULL, "args is NULL");
+    if (a->io_dtype != FA_BF16 && a->io_dtype != FA_FP16)
+        return fail(FA_ERR_DTYPE, "FlashAttention only supports FP16 and BF16 data types");
+    if (a->kv_dtype != a->io_dtype && a->kv_dtype != FA_INT8)
+        return fail(FA_ERR_DTYPE, "query and key_cache must have the same dtype");
+    if (!a->q || !a->out || !a->softmax_lse || !a->k_cache || !a->v_cache)
+        return fail(FA_ERR_NULL, "q, out, softmax_lse, k_cache and v_cache must be non-NULL");
+    if (!a->block_table) return fail(FA_ERR_UNSUPPORTED, "only the paged KV cache (block_table) is supported");
+    if (!a->cache_seqlens) return fail(FA_ERR_NULL, "cache_seqlens must be given with a paged KV cache");
+    if (a->batch <= 0) return fail(FA_ERR_SHAPE, "batch size must be positive");
+    if (a->seqlen_q <= 0 || a->nheads <= 0 || a->nheads_k <= 0) return fail(FA_ERR_SHAPE, "empty query");
+    if (a->nheads % a->nheads_k != 0)
+        return fail(FA_ERR_SHAPE, "Number of heads in key/value must divide number of heads in query");
+    if (a->page_size <= 0 || a->page_size % 32 != 0)
+        return fail(FA_ERR_SHAPE, "page_block_size must be a positive multiple of 32");
+    if (a->num_blocks <= 0 || a->max_blocks_per_seq <= 0) return fail(FA_ERR_SHAPE, "empty block_table or cache");
+    if (a->softcap < 0.f) return fail(FA_ERR_SHAPE, "softcap must be non-negative (0.0 disables softcap)");
+    if (a->num_splits < 0) return fail(FA_ERR_SHAPE, "num_splits must be non-negative");
+    if (is_mla_i8(a)) {
+        if (!a->k_scale_cache) return fail(FA_ERR_NULL, "int8 KV cache needs k_scale_cache");
+        if (a->headdim_qk != 576 || a->headdim_v != 512 || a->nheads_k != 1)
+            return fail(FA_ERR_SHAPE, "int8 KV cache supports the latent layout only (1 kv head, 576/512 dims)");
+        if (a->k_new) return fail(FA_ERR_UNSUPPORTED, "append into an int8 KV cache is not supported");
+    } else {
+        if (a->headdim_qk > 256) return fail(FA_ERR_SHAPE, "FlashAttention only supports head dimension at most 256");
+        if (a->headdim_qk != a->headdim_v) return fail(FA_ERR_SHAPE, "k and v head dimensions must match");
+        if (a->headdim_qk != 64 && a->headdim_qk != 128 && a->headdim_qk != 256)
+            return fail(FA_ERR_SHAPE, "head dimension must be 64, 128 or 256");
+    }
+    if ((a->k_new == nullptr) != (a->v_new == nullptr)) return fail(FA_ERR_NULL, "k and v must be passed together");
+    if (a->k_new && a->seqlen_new <= 0) return fail(FA_ERR_SHAPE, "seqlen_new must be positive when k is given");
+    if (!a->k_new && a->seqlen_new != 0) return fail(FA_ERR_SHAPE, "seqlen_new must be 0 without k");
+    if ((a->rotary_cos == nullptr) != (a->rotary_sin == nullptr))
+        return fail(FA_ERR_NULL, "rotary_cos and rotary_sin must be passed together");
+    if (a->rotary_cos) {
+        if (!a->k_new) return fail(FA_ERR_UNSUPPORTED, "rotary embedding is only applied when k and v are passed");
+        if (a->rotary_dim <= 0 || a->rotary_dim > a->headdim_qk || a->rotary_dim % 16 != 0)
+            return fail(FA_ERR_SHAPE, "rotary_dim must be divisible by 16 and at most headdim");
+        if (a->seqlen_ro <= 0) return fail(FA_ERR_SHAPE, "rotary tables are empty");
+    }
+    // strides the kernels turn into 32-bit byte offsets inside a page / 16-byte accesses
+    if (a->k_stride_row % 8 || a->k_stride_h % 8 || a->k_stride_block % 8 || a->v_stride_row % 8 ||
+        a->v_stride_h % 8 || a->v_stride_block % 8 || a->q_stride_h % 8 || a->q_stride_s % 8 || a->q_stride_b % 8 ||
+        a->o_stride_h % 8 || a->o_stride_s % 8 || a->o_stride_b % 8)
+        if (!is_mla_i8(a)) return fail(FA_ERR_SHAPE, "tensor strides must be multiples of 8 elements (16 bytes)");
+    if ((int64_t)a->page_size * a->k_stride_row * 2 >= (1ll << 31) || (int64_t)a->page_size * a->v_stride_row * 2 >= (1ll << 31))
+        return fail(FA_ERR_SHAPE, "a cache page must span less than 2 GiB");
+    return FA_OK;
+}
+
+int fa_rocm_choose_splits(const fa_kvcache_args *a, int num_cus, int32_t *split_keys) {
+    if (!a) return fail(FA_ERR_NULL, "args is NULL");
+    if (num_cus <= 0) num_cus = 256;
+    const int64_t bound = live_keys_bound(a);
+    const int64_t granule = 256;
+    int64_t sk;
+    if (a->num_splits == 1) {
+        sk = (bound + granule - 1) / granule * granule;
+    } else if (a->num_splits > 1) {
+        // forced mode (flash_attn_npu_3/fa_split.h:345-350): blocks per split = ceil(nblk / num_splits)
+        const int64_t nblk = (bound + granule - 1) / granule;
+        const int64_t per = (nblk + a->num_splits - 1) / a->num_splits;
+        sk = per * granule;
+    } else {
+        // heuristic: enough workgroups to give every CU several, but at least 1024 keys per split
+        // so that the per-split prologue/merge stays small next to the stream
+        const int64_t units = (int64_t)a->batch * a->nheads_k;
+        const int64_t target_wgs = (int64_t)num_cus * 8;
+        int64_t want = (target_wgs + units - 1) / units;  // splits per unit
+        if (want < 1) want = 1;
+        sk = (bound + want - 1) / want;
+        sk = (sk + granule - 1) / granule * granule;
+        if (sk < 1024) sk = 1024;
+    }
+    if (sk > (1 << 30)) sk = 1 << 30;
+    int64_t n = (bound + sk - 1) / sk;
+    if (n < 1) n = 1;
+    if (split_keys) *split_keys = (int32_t)sk;
+    return (int)n;
+}
+
+size_t fa_rocm_kvcache_workspace_bytes(const fa_kvcache_args *a, int num_cus) {
+    if (!a) return 0;
+    int32_t sk = 0;
+    const int n = fa_rocm_choose_splits(a, num_cus, &sk);
+    if (n <= 1) return 0;
+    const int group = a->nheads / (a->nheads_k > 0 ? a->nheads_k : 1);
+    const size_t rows = (size_t)a->seqlen_q * group;
+    const size_t slots = (size_t)a->batch * a->nheads_k * n * rows;
+    return slots * ((size_t)a->headdim_v + 1) * sizeof(float);
+}
+
+static void fill_append(const fa_kvcache_args *a, fa::AppendParams &p) {
+    std::memset(&p, 0, sizeof(p));
+    p.k_cache = a->k_cache;
+    p.v_cache = a->v_cache;
+    p.k_new = a->k_new;
+    p.v_new = a->v_new;
+    p.rotary_cos = a->rotary_cos;
+    p.rotary_sin = a->rotary_sin;
+    p.cache_seqlens = a->cache_seqlens;
+    p.block_table = a->block_table;
+    p.batch = a->batch;
+    p.seqlen_new = a->seqlen_new;
+    p.nheads_k = a->nheads_k;
+    p.headdim_qk = a->headdim_qk;
+    p.headdim_v = a->headdim_v;
+    p.num_blocks = a->num_blocks;
+    p.page_size = a->page_size;
+    p.max_blocks = a->max_blocks_per_seq;
+    p.rotary_dim = a->rotary_dim;
+    p.seqlen_ro = a->seqlen_ro;
+    p.rotary_interleaved = a->rotary_interleaved;
+    p.k_stride_block = a->k_stride_block;
+    p.k_stride_row = a->k_stride_row;
+    p.k_stride_h = a->k_stride_h;
+    p.v_stride_block = a->v_stride_block;
+    p.v_stride_row = a->v_stride_row;
+    p.v_stride_h = a->v_stride_h;
+    p.kn_stride_b = a->kn_stride_b;
+    p.kn_stride_s = a->kn_stride_s;
+    p.kn_stride_h = a->kn_stride_h;
+    p.vn_stride_b = a->vn_stride_b;
+    p.vn_stride_s = a->vn_stride_s;
+    p.vn_stride_h = a->vn_stride_h;
+    p.bt_stride_b = a->bt_stride_b;
+}
+
+int fa_rocm_append_kv(const fa_kvcache_args *a, void *stream) {
+    const int rc = fa_rocm_kvcache_validate(a);
+    if (rc != FA_OK) return rc;
+    if (!a->k_new) return FA_OK;
+    fa::AppendParams p;
+    fill_append(a, p);
+    const hipError_t e = fa::launch_append_kv(p, a->io_dtype, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return fail(FA_ERR_LAUNCH, "append_kv launch failed: %s", hipGetErrorString(e));
+    return FA_OK;
+}
+
+int fa_rocm_fwd_kvcache(const fa_kvcache_args *a, void *stream_) {
+    int rc = fa_rocm_kvcache_validate(a);
+    if (rc != FA_OK) return rc;
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const int group = a->nheads / a->nheads_k;
+    const int rows = a->seqlen_q * group;
+
+    if (a->k_new) {
+        rc = fa_rocm_append_kv(a, stream_);
+        if (rc != FA_OK) return rc;
+    }
+
+    const bool local = a->window_left >= 0 || a->window_right >= 0;
+
+    if (!is_mla_i8(a) && rows > fa::kDecodeMaxRows) {
+        // query block too tall for the decode kernel: tiled forward over the paged cache
+        fa::PrefillParams pp;
+        std::memset(&pp, 0, sizeof(pp));
+        pp.q = a->q;
+        pp.k = a->k_cache;
+        pp.v = a->v_cache;
+        pp.out = a->out;
+        pp.lse = a->softmax_lse;
+        pp.seqused_k = a->cache_seqlens;
+        pp.block_table = a->block_table;
+        pp.batch = a->batch;
+        pp.nheads = a->nheads;
+        pp.nheads_k = a->nheads_k;
+        pp.group = group;
+        pp.seqlen_q_fixed = a->seqlen_q;
+        pp.seqlen_k_add = a->seqlen_new;
+        pp.max_seqlen_q = a->seqlen_q;
+        pp.total_q = a->batch * a->seqlen_q;
+        pp.page_size = a->page_size;
+        pp.max_blocks = a->max_blocks_per_seq;
+        pp.num_blocks = a->num_blocks;
+        pp.q_stride_b = a->q_stride_b;
+        pp.q_stride_t = a->q_stride_s;
+        pp.q_stride_h = a->q_stride_h;
+        pp.o_stride_b = a->o_stride_b;
+        pp.o_stride_t = a->o_stride_s;
+        pp.o_stride_h = a->o_stride_h;
+        pp.k_stride_t = a->k_stride_row;
+        pp.k_stride_h = a->k_stride_h;
+        pp.k_stride_block = a->k_stride_block;
+        pp.v_stride_t = a->v_stride_row;
+        pp.v_stride_h = a->v_stride_h;
+        pp.v_stride_block = a->v_stride_block;
+        pp.bt_stride_b = a->bt_stride_b;
+        pp.lse_stride_b = (int64_t)a->nheads * a->seqlen_q;
+        pp.lse_stride_h = a->seqlen_q;
+        pp.scale_log2 = a->softmax_scale * kLog2e;
+        if (a->softcap > 0.f) {
+            pp.softcap_pre = a->softmax_scale / a->softcap;
+            pp.softcap_post = a->softcap * kLog2e;
+        }
+        pp.causal = a->causal;
+        pp.window_left = a->window_left;
+        pp.window_right = a->window_right;
+        if (a->rotary_cos)
+            return fail(FA_ERR_UNSUPPORTED, "rotary embedding needs seqlen_q * (nheads / nheads_k) <= %d", fa::kDecodeMaxRows);
+        const hipError_t e = fa::launch_prefill(pp, a->io_dtype, a->headdim_qk, stream);
+        if (e != hipSuccess) return fail(FA_ERR_LAUNCH, "prefill launch failed: %s", hipGetErrorString(e));
+        return FA_OK;
+    }
+
+    int cus = device_cus();
+    if (cus <= 0) cus = 256;
+    int32_t split_keys = 0;
+    const int nsplits = fa_rocm_choose_splits(a, cus, &split_keys);
+    const size_t need = fa_rocm_kvcache_workspace_bytes(a, cus);
+    if (need > 0 && (!a->workspace || a->workspace_bytes < need))
+        return fail(FA_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", need, a->workspace ? a->workspace_bytes : (size_t)0);
+
+    fa::DecodeParams p;
+    std::memset(&p, 0, sizeof(p));
+    p.q = a->q;
+    p.out = a->out;
+    p.lse = a->softmax_lse;
+    p.k_cache = a->k_cache;
+    p.v_cache = a->v_cache;
+    p.k_scale = a->k_scale_cache;
+    p.v_scale = a->v_scale_cache ? a->v_scale_cache : a->k_scale_cache;
+    p.rotary_cos = a->k_new ? a->rotary_cos : nullptr;
+    p.rotary_sin = a->k_new ? a->rotary_sin : nullptr;
+    p.cache_seqlens = a->cache_seqlens;
+    p.block_table = a->block_table;
+    p.batch = a->batch;
+    p.seqlen_q = a->seqlen_q;
+    p.nheads = a->nheads;
+    p.nheads_k = a->nheads_k;
+    p.group = group;
+    p.rows = rows;
+    p.seqlen_new = a->seqlen_new;
+    p.num_blocks = a->num_blocks;
+    p.page_size = a->page_size;
+    p.max_blocks = a->max_blocks_per_seq;
+    p.rotary_dim = a->rotary_dim;
+    p.seqlen_ro = a->seqlen_ro;
+    p.rotary_interleaved = a->rotary_interleaved;
+    p.rotary_per_token = (a->causal || local) ? 1 : 0;
+    p.q_stride_b = a->q_stride_b;
+    p.q_stride_s = a->q_stride_s;
+    p.q_stride_h = a->q_stride_h;
+    p.o_stride_b = a->o_stride_b;
+    p.o_stride_s = a->o_stride_s;
+    p.o_stride_h = a->o_stride_h;
+    p.k_stride_block = a->k_stride_block;
+    p.k_stride_row = a->k_stride_row;
+    p.k_stride_h = a->k_stride_h;
+    p.v_stride_block = a->v_stride_block;
+    p.v_stride_row = a->v_stride_row;
+    p.v_stride_h = a->v_stride_h;
+    p.ks_stride_block = a->ks_stride_block;
+    p.ks_stride_row = a->ks_stride_row;
+    p.bt_stride_b = a->bt_stride_b;
+    p.scale_log2 = a->softmax_scale * kLog2e;
+    if (a->softcap > 0.f) {
+        p.softcap_pre = a->softmax_scale / a->softcap;
+        p.softcap_post = a->softcap * kLog2e;
+    }
+    p.causal = a->causal;
+    p.window_left = a->window_left;
+    p.window_right = a->window_right;
+    p.nsplits = nsplits;
+    p.split_keys = split_keys;
+    if (nsplits > 1) {
+        const size_t slots = (size_t)a->batch * a->nheads_k * nsplits * rows;
+        p.o_partial = static_cast<float *>(a->workspace);
+        p.lse_partial = p.o_partial + slots * a->headdim_v;
+    }
+
+    hipError_t e;
+    if (is_mla_i8(a))
+        e = fa::launch_decode_mla_i8(p, a->io_dtype, stream);
+    else
+        e = fa::launch_decode_paged(p, a->io_dtype, a->headdim_qk, stream);
+    if (e != hipSuccess) return fail(FA_ERR_LAUNCH, "decode launch failed: %s", hipGetErrorString(e));
+    if (nsplits > 1) {
+        e = fa::launch_splitkv_combine(p, a->io_dtype, a->headdim_v, stream);
+        if (e != hipSuccess) return fail(FA_ERR_LAUNCH, "combine launch failed: %s", hipGetErrorString(e));
+    }
+    return FA_OK;
+}
+
+int fa_rocm_varlen_validate(const fa_varlen_args *a) {
+    if (!a) return fail(FA_ERR_NULL, "args is NULL");
+    if (a->io_dtype != FA_BF16 && a->io_dtype != FA_FP16)
+        return fail(FA_ERR_DTYPE, "FlashAttention only supports FP16 and BF16 data types");
+    if (!a->q || !a->k || !a->v || !a->out || !a->softmax_lse) return fail(FA_ERR_NULL, "q, k, v, out and softmax_lse must be non-NULL");
+    if (!a->cu_seqlens_q) return fail(FA_ERR_NULL, "cu_seqlens_q must be non-NULL");
+    if (!a->block_table && !a->cu_seqlens_k) return fail(FA_ERR_NULL, "cu_seqlens_k must be non-NULL");
+    if (a->block_table && !a->seqused_k) return fail(FA_ERR_NULL, "paged K/V needs seqused_k");
+    if (a->batch <= 0) return fail(FA_ERR_SHAPE, "batch size must be positive");
+    if (a->nheads <= 0 || a->nheads_k <= 0 || a->nheads % a->nheads_k != 0)
+        return fail(FA_ERR_SHAPE, "Number of heads in key/value must divide number of heads in query");
+    if (a->headdim > 256) return fail(FA_ERR_SHAPE, "FlashAttention only supports head dimension at most 256");
+    if (a->headdim != 64 && a->headdim != 128 && a->headdim != 256) return fail(FA_ERR_SHAPE, "head dimension must be 64, 128 or 256");
+    if (a->softcap < 0.f) return fail(FA_ERR_SHAPE, "softcap must be non-negative (0.0 disables softcap)");
+    if (a->max_seqlen_q <= 0) return fail(FA_ERR_SHAPE, "max_seqlen_q must be positive");
+    if (a->block_table && (a->page_size <= 0 || a->page_size % 32 != 0))
+        return fail(FA_ERR_SHAPE, "page_block_size must be a positive multiple of 32");
+    if (a->q_stride_t % 8 || a->q_stride_h % 8 || a->k_stride_t % 8 || a->k_stride_h % 8 || a->v_stride_t % 8 ||
+        a->v_stride_h % 8 || a->o_stride_t % 8 || a->o_stride_h % 8)
+        return fail(FA_ERR_SHAPE, "tensor strides must be multiples of 8 elements (16 bytes)");
+    return FA_OK;
+}
+
+int fa_rocm_varlen_fwd(const fa_varlen_args *a, void *stream_) {
+    const int rc = fa_rocm_varlen_validate(a);
+    if (rc != FA_OK) return rc;
+    fa::PrefillParams pp;
+    std::memset(&pp, 0, sizeof(pp));
+    pp.q = a->q;
+    pp.k = a->k;
+    pp.v = a->v;
+    pp.out = a->out;
+    pp.lse = a->softmax_lse;
+    pp.cu_seqlens_q = a->cu_seqlens_q;
+    pp.cu_seqlens_k = a->cu_seqlens_k;
+    pp.seqused_k = a->seqused_k;
+    pp.block_table = a->block_table;
+    pp.batch = a->batch;
+    pp.nheads = a->nheads;
+    pp.nheads_k = a->nheads_k;
+    pp.group = a->nheads / a->nheads_k;
+    pp.max_seqlen_q = a->max_seqlen_q;
+    pp.total_q = a->total_q;
+    pp.page_size = a->page_size;
+    pp.max_blocks = a->max_blocks_per_seq;
+    pp.q_stride_t = a->q_stride_t;
+    pp.q_stride_h = a->q_stride_h;
+    pp.o_stride_t = a->o_stride_t;
+    pp.o_stride_h = a->o_stride_h;
+    pp.k_stride_t = a->k_stride_t;
+    pp.k_stride_h = a->k_stride_h;
+    pp.k_stride_block = a->k_stride_block;
+    pp.v_stride_t = a->v_stride_t;
+    pp.v_stride_h = a->v_stride_h;
+    pp.v_stride_block = a->v_stride_block;
+    pp.bt_stride_b = a->bt_stride_b;
+    pp.lse_stride_b = 0;
+    pp.lse_stride_h = a->total_q;
+    pp.scale_log2 = a->softmax_scale * kLog2e;
+    if (a->softcap > 0.f) {
+        pp.softcap_pre = a->softmax_scale / a->softcap;
+        pp.softcap_post = a->softcap * kLog2e;
+    }
+    pp.causal = a->causal;
+    pp.window_left = a->window_left;
+    pp.window_right = a->window_right;
+    const hipError_t e = fa::launch_prefill(pp, a->io_dtype, a->headdim, static_cast<hipStream_t>(stream_));
+    if (e != hipSuccess) return fail(FA_ERR_LAUNCH, "prefill launch failed: %s", hipGetErrorString(e));
+    return FA_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,214 @@
+"""Operator layer: `fwd_kvcache` and `varlen_fwd` with the argument order of the reference's
+extension module (csrc/ascend910/flash_attn_npu/flash_api.cpp:356-377, :848-869, exported at
+:1335-1336), implemented over the C ABI of libfa_rocm.so.
+
+Checks that the reference performs with TORCH_CHECK raise RuntimeError with the same text.
+There is no fallback: tensors must live on a ROCm device and the library must be built."""
+from __future__ import annotations
+
+import ctypes as C
+from typing import List, Optional
+
+import torch
+
+from . import _lib
+
+_DT = {torch.bfloat16: _lib.FA_BF16, torch.float16: _lib.FA_FP16, torch.int8: _lib.FA_INT8}
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else t.data_ptr()
+
+
+def _stream(t: torch.Tensor):
+    return C.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def _require(cond: bool, msg: str) -> None:
+    if not cond:
+        raise RuntimeError(msg)
+
+
+def _require_device(*tensors) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError("flash_attn_npu (MI355X build) needs tensors on a ROCm device; there is no CPU path")
+
+
+def fwd_kvcache(q, kcache, vcache, k_, v_, seqlens_k_, rotary_cos_, rotary_sin_, cache_batch_idx_, leftpad_k_,
+                block_table_, alibi_slopes_, out_, softmax_scale, is_causal, window_size_left, window_size_right,
+                softcap, is_rotary_interleaved, num_splits, k_scale_cache_=None, v_scale_cache_=None
+                ) -> List[torch.Tensor]:
+    """mha_fwd_kvcache (flash_api.cpp:356-637) on a paged cache.  Returns [out, softmax_lse]."""
+    lib = _lib.load()
+    is_i8 = kcache.dtype == torch.int8
+    _require(q.dtype in (torch.bfloat16, torch.float16), "FlashAttention only supports FP16 and BF16 data types")
+    if not is_i8:
+        _require(kcache.dtype == q.dtype, "query and key_cache must have the same dtype")
+        _require(vcache.dtype == q.dtype, "query and value_cache must have the same dtype")
+    else:
+        _require(vcache.dtype == torch.int8, "key_cache and value_cache must have the same dtype")
+        _require(k_scale_cache_ is not None, "int8 KV cache needs k_scale_cache")
+    _require(q.stride(-1) == 1, "Input tensor q must have contiguous last dimension")
+    _require(kcache.stride(-1) == 1, "Input tensor kcache must have contiguous last dimension")
+    _require(vcache.stride(-1) == 1, "Input tensor vcache must have contiguous last dimension")
+    _require(block_table_ is not None, "MI355X FlashAttention supports the paged KV cache only: pass block_table")
+    _require(block_table_.dtype == torch.int32, "block_table must have dtype int32")
+    _require(block_table_.stride(-1) == 1, "block_table must have contiguous last dimension")
+    _require(seqlens_k_ is not None, "cache_seqlens must be given with a paged KV cache")
+    _require(seqlens_k_.dtype == torch.int32, "seqlens_k must have dtype int32")
+    _require(alibi_slopes_ is None, "NPU FlashAttention does not support alibi_slopes")
+    _require(leftpad_k_ is None, "NPU FlashAttention does not support leftpad_k")
+    _require(cache_batch_idx_ is None, "MI355X FlashAttention does not support cache_batch_idx")
+    _require(softcap >= 0.0, "softcap must be non-negative (0.0 disables softcap)")
+    _require(q.dim() == 4 and kcache.dim() == 4 and vcache.dim() == 4, "q, kcache and vcache must be 4-D")
+    _require_device(q, kcache, vcache, k_, v_, seqlens_k_, block_table_, rotary_cos_, rotary_sin_)
+
+    B, sq, hq, d = q.shape
+    num_blocks, page, hk, dk = kcache.shape
+    dv = vcache.shape[-1]
+    _require(B > 0, "batch size must be positive")
+    _require(d == dk, "q and kcache must have the same head dimension")
+    _require(hq % hk == 0, "Number of heads in key/value must divide number of heads in query")
+    _require(block_table_.shape[0] == B and seqlens_k_.shape[0] == B, "block_table / cache_seqlens batch mismatch")
+    seqlens_k = seqlens_k_.contiguous()
+
+    if out_ is not None:
+        out = out_
+        _require(out.dtype == q.dtype and tuple(out.shape) == (B, sq, hq, dv) and out.stride(-1) == 1,
+                 "out must have shape (batch_size, seqlen_q, num_heads, head_size_v) and the dtype of q")
+    else:
+        out = torch.empty((B, sq, hq, dv), dtype=q.dtype, device=q.device)
+    lse = torch.empty((B, hq, sq), dtype=torch.float32, device=q.device)
+
+    a = _lib.KvcacheArgs()
+    a.q, a.out, a.softmax_lse = _ptr(q), _ptr(out), _ptr(lse)
+    a.k_cache, a.v_cache = _ptr(kcache), _ptr(vcache)
+    a.k_scale_cache, a.v_scale_cache = _ptr(k_scale_cache_), _ptr(v_scale_cache_)
+    a.cache_seqlens, a.block_table = _ptr(seqlens_k), _ptr(block_table_)
+    a.batch, a.seqlen_q, a.nheads, a.nheads_k = B, sq, hq, hk
+    a.headdim_qk, a.headdim_v = d, dv
+    a.num_blocks, a.page_size, a.max_blocks_per_seq = num_blocks, page, block_table_.shape[1]
+    a.q_stride_b, a.q_stride_s, a.q_stride_h = q.stride(0), q.stride(1), q.stride(2)
+    a.o_stride_b, a.o_stride_s, a.o_stride_h = out.stride(0), out.stride(1), out.stride(2)
+    a.k_stride_block, a.k_stride_row, a.k_stride_h = kcache.stride(0), kcache.stride(1), kcache.stride(2)
+    a.v_stride_block, a.v_stride_row, a.v_stride_h = vcache.stride(0), vcache.stride(1), vcache.stride(2)
+    a.bt_stride_b = block_table_.stride(0)
+    if k_scale_cache_ is not None:
+        _require(k_scale_cache_.dtype == torch.float32 and k_scale_cache_.dim() == 3 and k_scale_cache_.stride(-1) == 1,
+                 "k_scale_cache must be fp32 (num_blocks, page_block_size, nheads_k)")
+        a.ks_stride_block, a.ks_stride_row = k_scale_cache_.stride(0), k_scale_cache_.stride(1)
+        if v_scale_cache_ is not None:
+            _require(v_scale_cache_.stride() == k_scale_cache_.stride() and v_scale_cache_.dtype == torch.float32,
+                     "v_scale_cache must match k_scale_cache's layout")
+    keep = [seqlens_k]
+    if k_ is not None or v_ is not None:
+        _require(k_ is not None and v_ is not None, "k and v must be passed together")
+        _require(k_.dtype == q.dtype and v_.dtype == q.dtype, "Key and value must have the same dtype as query")
+        _require(k_.dim() == 4 and k_.shape[0] == B and k_.shape[2] == hk and k_.shape[3] == d
+                 and tuple(v_.shape) == (B, k_.shape[1], hk, dv), "k / v must be (batch_size, seqlen_new, nheads_k, headdim)")
+        k_ = k_ if k_.stride(-1) == 1 else k_.contiguous()
+        v_ = v_ if v_.stride(-1) == 1 else v_.contiguous()
+        keep += [k_, v_]
+        a.k_new, a.v_new, a.seqlen_new = _ptr(k_), _ptr(v_), k_.shape[1]
+        a.kn_stride_b, a.kn_stride_s, a.kn_stride_h = k_.stride(0), k_.stride(1), k_.stride(2)
+        a.vn_stride_b, a.vn_stride_s, a.vn_stride_h = v_.stride(0), v_.stride(1), v_.stride(2)
+        if rotary_cos_ is not None or rotary_sin_ is not None:
+            _require(rotary_cos_ is not None and rotary_sin_ is not None, "rotary_cos and rotary_sin must be passed together")
+            _require(rotary_cos_.dtype == q.dtype and rotary_sin_.dtype == q.dtype,
+                     "rotary_cos / rotary_sin must have the same dtype as query")
+            _require(rotary_cos_.dim() == 2 and rotary_cos_.shape == rotary_sin_.shape, "rotary_cos / rotary_sin must be (seqlen_ro, rotary_dim / 2)")
+            rc, rs = rotary_cos_.contiguous(), rotary_sin_.contiguous()
+            keep += [rc, rs]
+            a.rotary_cos, a.rotary_sin = _ptr(rc), _ptr(rs)
+            a.seqlen_ro, a.rotary_dim = rc.shape[0], 2 * rc.shape[1]
+            _require(a.rotary_dim <= d, "rotary_dim must be <= headdim")
+            _require(a.rotary_dim % 16 == 0, "Only rotary dimensions divisible by 16 are currently supported")
+    a.io_dtype = _DT[q.dtype]
+    a.kv_dtype = _DT[kcache.dtype]
+    a.softmax_scale, a.softcap = float(softmax_scale), float(softcap)
+    a.causal = int(bool(is_causal))
+    a.window_left, a.window_right = int(window_size_left), int(window_size_right)
+    a.rotary_interleaved = int(bool(is_rotary_interleaved))
+    a.num_splits = int(num_splits)
+
+    _lib.check(lib.fa_rocm_kvcache_validate(C.byref(a)))
+    with torch.cuda.device(q.device):
+        cus = lib.fa_rocm_num_cus()
+        need = lib.fa_rocm_kvcache_workspace_bytes(C.byref(a), cus)
+        if need:
+            ws = torch.empty((need + 3) // 4, dtype=torch.float32, device=q.device)
+            keep.append(ws)
+            a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel() * 4
+        _lib.check(lib.fa_rocm_fwd_kvcache(C.byref(a), _stream(q)))
+    return [out, lse]
+
+
+def varlen_fwd(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k_, leftpad_k_, block_table_, alibi_slopes_,
+               max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale, zero_tensors, is_causal, window_size_left,
+               window_size_right, softcap, return_softmax, gen_) -> List[torch.Tensor]:
+    """mha_varlen_fwd (flash_api.cpp:848-1089).  Returns [out, softmax_lse (Hq, total_q), p, rng_state]."""
+    lib = _lib.load()
+    _require(q.dtype in (torch.bfloat16, torch.float16), "FlashAttention only supports FP16 and BF16 data types")
+    _require(k.dtype == q.dtype, "query and key must have the same dtype")
+    _require(v.dtype == q.dtype, "query and value must have the same dtype")
+    _require(cu_seqlens_q.dtype == torch.int32, "cu_seqlens_q must have dtype int32")
+    _require(q.stride(-1) == 1 and k.stride(-1) == 1 and v.stride(-1) == 1, "Input tensor must have contiguous last dimension")
+    _require(leftpad_k_ is None, "NPU FlashAttention does not support leftpad_k")
+    _require(alibi_slopes_ is None, "NPU FlashAttention does not support alibi_slopes")
+    _require(p_dropout == 0.0, "NPU FlashAttention does not support dropout")
+    _require(not return_softmax, "NPU FlashAttention does not support return_softmax")
+    _require(softcap >= 0.0, "softcap must be non-negative (0.0 disables softcap)")
+    _require_device(q, k, v, cu_seqlens_q, cu_seqlens_k, seqused_k_, block_table_)
+    paged = block_table_ is not None
+    total_q, hq, d = q.shape
+    B = cu_seqlens_q.numel() - 1
+    _require(B > 0, "batch size must be positive")
+    a = _lib.VarlenArgs()
+    if paged:
+        _require(block_table_.dtype == torch.int32, "block_table must have dtype int32")
+        _require(block_table_.stride(-1) == 1, "block_table must have contiguous last dimension")
+        _require(k.dim() == 4 and v.dim() == 4, "paged k / v must be (num_blocks, page_block_size, nheads_k, headdim)")
+        if seqused_k_ is None:
+            _require(cu_seqlens_k is not None, "paged K/V needs seqused_k or cu_seqlens_k")
+            seqused_k_ = (cu_seqlens_k[1:] - cu_seqlens_k[:-1]).to(torch.int32)
+        _require(seqused_k_.dtype == torch.int32, "seqused_k must have dtype int32")
+        seqused_k_ = seqused_k_.contiguous()
+        hk = k.shape[2]
+        a.page_size, a.max_blocks_per_seq = k.shape[1], block_table_.shape[1]
+        a.k_stride_block, a.k_stride_t, a.k_stride_h = k.stride(0), k.stride(1), k.stride(2)
+        a.v_stride_block, a.v_stride_t, a.v_stride_h = v.stride(0), v.stride(1), v.stride(2)
+        a.block_table, a.seqused_k, a.bt_stride_b = _ptr(block_table_), _ptr(seqused_k_), block_table_.stride(0)
+    else:
+        _require(cu_seqlens_k is not None and cu_seqlens_k.dtype == torch.int32, "cu_seqlens_k must have dtype int32")
+        _require(k.dim() == 3 and v.dim() == 3, "k / v must be (total_k, nheads_k, headdim)")
+        hk = k.shape[1]
+        a.k_stride_t, a.k_stride_h = k.stride(0), k.stride(1)
+        a.v_stride_t, a.v_stride_h = v.stride(0), v.stride(1)
+    _require(k.shape[-1] == d and v.shape[-1] == d, "q, k and v must have the same head dimension")
+    _require(d <= 256, "FlashAttention only supports head dimension at most 256")
+    _require(hq % hk == 0, "Number of heads in key/value must divide number of heads in query")
+    cu_q = cu_seqlens_q.contiguous()
+    cu_k = cu_seqlens_k.contiguous() if cu_seqlens_k is not None else None
+    if out_ is not None:
+        out = out_
+        _require(out.dtype == q.dtype and out.shape == q.shape and out.stride(-1) == 1, "out must match q")
+    else:
+        out = torch.empty_like(q, memory_format=torch.contiguous_format)
+    lse = torch.empty((hq, total_q), dtype=torch.float32, device=q.device)
+    a.q, a.k, a.v, a.out, a.softmax_lse = _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse)
+    a.cu_seqlens_q, a.cu_seqlens_k = _ptr(cu_q), _ptr(cu_k)
+    a.batch, a.total_q, a.nheads, a.nheads_k, a.headdim = B, total_q, hq, hk, d
+    a.max_seqlen_q, a.max_seqlen_k = int(max_seqlen_q), int(max_seqlen_k)
+    a.q_stride_t, a.q_stride_h = q.stride(0), q.stride(1)
+    a.o_stride_t, a.o_stride_h = out.stride(0), out.stride(1)
+    a.io_dtype = _DT[q.dtype]
+    a.softmax_scale, a.softcap = float(softmax_scale), float(softcap)
+    a.causal = int(bool(is_causal))
+    a.window_left, a.window_right = int(window_size_left), int(window_size_right)
+    if total_q > 0:
+        with torch.cuda.device(q.device):
+            _lib.check(lib.fa_rocm_varlen_fwd(C.byref(a), _stream(q)))
+    p = torch.empty((0,), dtype=q.dtype, device=q.device)
+    rng_state = torch.empty((2,), dtype=torch.int64, device=q.device)
+    return [out, lse, p, rng_state]

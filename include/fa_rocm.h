@@ -1,0 +1,177 @@
+/*
+ * fa_rocm.h - C ABI of the MI355X (gfx950) paged KV-cache attention library.
+ *
+ * Plain C: pointers, sizes, PODs.  No torch, no HIP types in the signatures (a
+ * stream is passed as void* and must be a hipStream_t or NULL for the default
+ * stream).  Every entry point enqueues work on the given stream and returns;
+ * nothing here synchronises with the host, allocates device memory or keeps
+ * mutable global state, so calls from several host threads on different
+ * streams are safe.  The caller owns every buffer, including the workspace.
+ *
+ * Return value: 0 on success; a negative FA_ERR_* code otherwise, with a
+ * human-readable message retrievable (per host thread) via fa_rocm_last_error().
+ *
+ * Each entry point names the reference interface it stands in for
+ * (paths relative to the MinghuasLab/flash-attention-npu checkout).
+ */
+#ifndef FA_ROCM_H_
+#define FA_ROCM_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FA_ROCM_ABI_VERSION 1
+
+enum fa_dtype { FA_BF16 = 0, FA_FP16 = 1, FA_INT8 = 2 };
+
+enum fa_error {
+    FA_OK = 0,
+    FA_ERR_NULL = -1,        /* a required pointer is NULL                         */
+    FA_ERR_DTYPE = -2,       /* unsupported dtype combination                      */
+    FA_ERR_SHAPE = -3,       /* dimension out of the supported range               */
+    FA_ERR_UNSUPPORTED = -4, /* feature the reference rejects too (alibi, leftpad) */
+    FA_ERR_WORKSPACE = -5,   /* workspace missing or too small                     */
+    FA_ERR_LAUNCH = -6       /* HIP reported a launch error                        */
+};
+
+/*
+ * Arguments of one flash_attn_with_kvcache call on a paged cache.
+ * Strides are in ELEMENTS of the tensor's dtype; the last dimension of every
+ * tensor is contiguous.  Mirrors the reference's kernel-launch record
+ * FwdLaunchArgs (csrc/ascend910/flash_attn_npu/fwd_dispatch.hpp:29-50) plus the
+ * parts of FAInferTilingData (tilingdata.h:34-62) the host fills from shapes.
+ */
+typedef struct fa_kvcache_args {
+    /* tensors (device pointers) */
+    const void *q;               /* (B, Sq, Hq, Dqk)            io dtype                         */
+    void *out;                   /* (B, Sq, Hq, Dv)             io dtype                         */
+    float *softmax_lse;          /* (B, Hq, Sq) fp32, natural log; +inf for rows with no key     */
+    void *k_cache;               /* (num_blocks, page, Hk, Dqk) kv dtype; written when k_new set */
+    void *v_cache;               /* (num_blocks, page, Hk, Dv)  kv dtype; may alias k_cache      */
+    const float *k_scale_cache;  /* (num_blocks, page, Hk) fp32 per-token scale; int8 cache only */
+    const float *v_scale_cache;  /* same for V; NULL = use k_scale_cache                         */
+    const void *k_new;           /* (B, Snew, Hk, Dqk) io dtype or NULL                          */
+    const void *v_new;           /* (B, Snew, Hk, Dv)  io dtype or NULL                          */
+    const void *rotary_cos;      /* (seqlen_ro, rotary_dim/2) io dtype or NULL                   */
+    const void *rotary_sin;      /* same                                                         */
+    const int32_t *cache_seqlens;/* (B,) keys already in the cache, per row                      */
+    const int32_t *block_table;  /* (B, max_blocks_per_seq) page ids                             */
+    void *workspace;             /* >= fa_rocm_kvcache_workspace_bytes(); may be NULL if that is 0 */
+    size_t workspace_bytes;
+
+    /* dimensions */
+    int32_t batch, seqlen_q, nheads, nheads_k;
+    int32_t headdim_qk, headdim_v;
+    int32_t seqlen_new;          /* 0 when k_new == NULL */
+    int32_t num_blocks, page_size, max_blocks_per_seq;
+    int32_t rotary_dim, seqlen_ro;
+
+    /* strides, elements */
+    int64_t q_stride_b, q_stride_s, q_stride_h;
+    int64_t o_stride_b, o_stride_s, o_stride_h;
+    int64_t k_stride_block, k_stride_row, k_stride_h;   /* k_cache */
+    int64_t v_stride_block, v_stride_row, v_stride_h;   /* v_cache */
+    int64_t ks_stride_block, ks_stride_row;              /* scale caches (head stride 1) */
+    int64_t kn_stride_b, kn_stride_s, kn_stride_h;      /* k_new */
+    int64_t vn_stride_b, vn_stride_s, vn_stride_h;      /* v_new */
+    int64_t bt_stride_b;                                 /* block_table row stride */
+
+    /* scalars */
+    int32_t io_dtype;            /* FA_BF16 or FA_FP16                                  */
+    int32_t kv_dtype;            /* same as io_dtype, or FA_INT8 (needs *_scale_cache)  */
+    float softmax_scale;
+    float softcap;               /* 0 = off                                             */
+    int32_t causal;              /* bottom-right aligned                                */
+    int32_t window_left, window_right;  /* -1 = unbounded                              */
+    int32_t rotary_interleaved;
+    int32_t num_splits;          /* 0 = heuristic, 1 = no split, >1 = at most that many */
+} fa_kvcache_args;
+
+/*
+ * Arguments of one flash_attn_varlen_func forward (token-major "TND" layout).
+ * K/V are either dense (total_k, Hk, D) addressed through cu_seqlens_k, or paged
+ * (block_table != NULL) with per-sequence lengths in seqused_k.
+ */
+typedef struct fa_varlen_args {
+    const void *q;               /* (total_q, Hq, D) */
+    const void *k;               /* (total_k, Hk, D) or paged (num_blocks, page, Hk, D) */
+    const void *v;
+    void *out;                   /* (total_q, Hq, D) */
+    float *softmax_lse;          /* (Hq, total_q) fp32 */
+    const int32_t *cu_seqlens_q; /* (B+1,) */
+    const int32_t *cu_seqlens_k; /* (B+1,) ; ignored when paged */
+    const int32_t *seqused_k;    /* (B,) ; paged only */
+    const int32_t *block_table;  /* (B, max_blocks_per_seq) or NULL */
+    int32_t batch, total_q, nheads, nheads_k, headdim;
+    int32_t max_seqlen_q, max_seqlen_k;
+    int32_t page_size, max_blocks_per_seq;
+    int64_t q_stride_t, q_stride_h;
+    int64_t k_stride_t, k_stride_h;   /* dense: token stride ; paged: row stride */
+    int64_t v_stride_t, v_stride_h;
+    int64_t k_stride_block, v_stride_block;
+    int64_t o_stride_t, o_stride_h;
+    int64_t bt_stride_b;
+    int32_t io_dtype;
+    float softmax_scale;
+    float softcap;
+    int32_t causal;
+    int32_t window_left, window_right;
+} fa_varlen_args;
+
+/* Library / device facts. */
+int fa_rocm_abi_version(void);
+const char *fa_rocm_last_error(void);
+/* sizeof the two argument records as this library was compiled (binding self-check). */
+size_t fa_rocm_sizeof_kvcache_args(void);
+size_t fa_rocm_sizeof_varlen_args(void);
+/* Compute units of the current HIP device (256 on MI355X); < 0 on error. */
+int fa_rocm_num_cus(void);
+
+/*
+ * Split-KV decision.  Stands in for the reference's flash-decode heuristic and
+ * partition (csrc/ascend910/flash_attn_npu/flash_api.cpp:525-550, splitBN2S1GS2 :343-354;
+ * forced mode csrc/ascend910/flash_attn_npu_3/fa_split.h:345-350).  Pure host integer code:
+ * needs no GPU.  Writes the keys-per-split granule (a multiple of 256) to *split_keys and
+ * returns the number of split slots per (batch row, kv head), >= 1.  `num_cus` <= 0 means 256.
+ */
+int fa_rocm_choose_splits(const fa_kvcache_args *args, int num_cus, int32_t *split_keys);
+
+/* Bytes of workspace the kvcache call needs for the split partials (0 when unsplit). */
+size_t fa_rocm_kvcache_workspace_bytes(const fa_kvcache_args *args, int num_cus);
+
+/*
+ * Argument validation only (no GPU work): same checks and messages as the reference host
+ * function mha_fwd_kvcache (csrc/ascend910/flash_attn_npu/flash_api.cpp:386-420,455-457).
+ */
+int fa_rocm_kvcache_validate(const fa_kvcache_args *args);
+int fa_rocm_varlen_validate(const fa_varlen_args *args);
+
+/*
+ * flash_attn_with_kvcache on a paged cache: optional in-place append of k_new/v_new
+ * (with rotary), attention of q over cache_seqlens+seqlen_new keys, split-KV combine.
+ * Replaces mha_fwd_kvcache (csrc/ascend910/flash_attn_npu/flash_api.cpp:356-637) and the
+ * launch behind it (fwd_dispatch.hpp:60-67, mha_fwd_kvcache.cpp:1025-1106).
+ */
+int fa_rocm_fwd_kvcache(const fa_kvcache_args *args, void *stream);
+
+/*
+ * flash_attn_varlen_func forward.  Replaces mha_varlen_fwd
+ * (csrc/ascend910/flash_attn_npu/flash_api.cpp:848-1089).
+ */
+int fa_rocm_varlen_fwd(const fa_varlen_args *args, void *stream);
+
+/*
+ * The in-place append on its own (k_new/v_new -> pages, rotary on k_new).  The reference
+ * documents it (flash_attn_npu/flash_attn_npu_interface.py:1460-1467) but its host drops the
+ * tensors (flash_api.cpp:422-427); exposed separately so cache writers can be tested bit-exactly.
+ */
+int fa_rocm_append_kv(const fa_kvcache_args *args, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FA_ROCM_H_ */

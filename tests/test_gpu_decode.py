@@ -1,0 +1,131 @@
+"""GPU parity of the paged decode path (through the C ABI) against the CPU oracle."""
+import pytest
+import torch
+
+import fa_oracle as O
+from helpers import check_out, check_vs_golden, make_paged_case, rotary_tables, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+def run_both(case, **kw):
+    from flash_attn_npu import flash_attn_with_kvcache
+    dev = to_dev(case)
+    print("case", {k: (tuple(v.shape) if isinstance(v, torch.Tensor) else v) for k, v in case.items()}, kw, flush=True)
+    out, lse = flash_attn_with_kvcache(dev["q"], dev["k_cache"], dev["v_cache"], dev["k"], dev["v"],
+                                       cache_seqlens=dev["cache_seqlens"], block_table=dev["block_table"],
+                                       return_softmax_lse=True, **kw)
+    torch.cuda.synchronize()
+    kc, vc = case["k_cache"].clone(), case["v_cache"].clone()
+    okw = {k: v for k, v in kw.items() if k != "num_splits"}
+    ref, ref_lse = O.flash_attn_with_kvcache(case["q"], kc, vc, case["k"], case["v"], cache_seqlens=case["cache_seqlens"],
+                                             block_table=case["block_table"], mode="fp32", **okw)
+    kc2, vc2 = case["k_cache"].clone(), case["v_cache"].clone()
+    gold, gold_lse = O.flash_attn_with_kvcache(case["q"], kc2, vc2, case["k"], case["v"],
+                                               cache_seqlens=case["cache_seqlens"], block_table=case["block_table"],
+                                               mode="golden", **okw)
+    return (out, lse), (ref, ref_lse), (gold, gold_lse), (dev, kc, vc)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("hq,hk", [(8, 2), (32, 8), (8, 8), (16, 1)])
+def test_decode_basic(dtype, hq, hk):
+    case = make_paged_case(3, hq, hk, 128, 256, [300, 511, 1025], dtype=dtype, seed=1)
+    got, ref, gold, _ = run_both(case, causal=True)
+    check_out(got[0], ref[0], got[1], ref[1], "decode_basic")
+    check_vs_golden(got[0], gold[0], got[1], gold[1], "decode_basic")
+
+
+@pytest.mark.parametrize("num_splits", [1, 2, 3, 7])
+def test_decode_split_invariance(num_splits):
+    case = make_paged_case(2, 16, 2, 128, 256, [4096, 2500], seed=2)
+    got, ref, gold, _ = run_both(case, causal=True, num_splits=num_splits)
+    check_out(got[0], ref[0], got[1], ref[1], f"splits={num_splits}")
+
+
+@pytest.mark.parametrize("lens", [[1, 31, 32, 33], [255, 256, 257, 512], [0, 5, 0, 700]])
+def test_decode_ragged_edges(lens):
+    case = make_paged_case(4, 8, 2, 128, 256, lens, seed=3)
+    got, ref, gold, _ = run_both(case, causal=True)
+    check_out(got[0], ref[0], got[1], ref[1], f"lens={lens}")
+
+
+def test_decode_uniform5_distribution():
+    # the reference tests draw U(-5, 5): one dominant key per row
+    case = make_paged_case(2, 8, 2, 128, 128, [2048, 777], seed=4, dist="uniform5")
+    got, ref, gold, _ = run_both(case, causal=False)
+    check_vs_golden(got[0], gold[0], got[1], gold[1], "uniform5")
+
+
+@pytest.mark.parametrize("window", [(64, 0), (542, 647), (4095, 0), (0, 0), (-1, 3)])
+def test_decode_window(window):
+    case = make_paged_case(2, 8, 1, 128, 256, [5000, 1300], seed=5)
+    got, ref, gold, _ = run_both(case, causal=False, window_size=window)
+    check_out(got[0], ref[0], got[1], ref[1], f"window={window}")
+
+
+@pytest.mark.parametrize("sq,hq,hk", [(2, 8, 2), (4, 4, 1), (3, 16, 8), (5, 8, 8), (2, 32, 1)])
+def test_decode_multi_token_causal(sq, hq, hk):
+    case = make_paged_case(2, hq, hk, 128, 256, [700, 259], seqlen_q=sq, seed=6)
+    got, ref, gold, _ = run_both(case, causal=True)
+    check_out(got[0], ref[0], got[1], ref[1], f"sq={sq}")
+
+
+def test_decode_sq_longer_than_keys():
+    # bottom-right causal with Sq > Sk: the first Sq-Sk rows see nothing -> 0 / +inf
+    case = make_paged_case(1, 4, 2, 128, 256, [2], seqlen_q=5, seed=7)
+    got, ref, gold, _ = run_both(case, causal=True)
+    check_out(got[0], ref[0], got[1], ref[1], "sq>sk")
+    assert torch.isinf(got[1][0, :, :3]).all() and (got[0][0, :3] == 0).all()
+
+
+@pytest.mark.parametrize("d", [64, 256])
+def test_decode_headdims(d):
+    case = make_paged_case(2, 8, 2, d, 128, [900, 130], seed=8)
+    got, ref, gold, _ = run_both(case, causal=True, num_splits=1)
+    check_out(got[0], ref[0], got[1], ref[1], f"d={d}")
+    got, ref, gold, _ = run_both(case, causal=True, num_splits=3)
+    check_out(got[0], ref[0], got[1], ref[1], f"d={d} split")
+
+
+def test_decode_softcap():
+    case = make_paged_case(2, 8, 2, 128, 256, [600, 300], seed=9)
+    got, ref, gold, _ = run_both(case, causal=True, softcap=3.0)
+    check_out(got[0], ref[0], got[1], ref[1], "softcap")
+
+
+@pytest.mark.parametrize("interleaved", [False, True])
+@pytest.mark.parametrize("rot", [128, 64])
+def test_append_rotary_bit_exact(interleaved, rot):
+    B, hq, hk, d, page = 4, 8, 2, 128, 256
+    lens = [300, 511, 256, 0]
+    case = make_paged_case(B, hq, hk, d, page, lens, seqlen_new=1, seed=10)
+    cos, sin = rotary_tables(1024, rot)
+    got, ref, gold, (dev, kc, vc) = run_both(case, causal=True, rotary_cos=None, rotary_sin=None)
+    # un-rotated append first: caches must match the oracle's bytes
+    assert torch.equal(dev["k_cache"].cpu().view(torch.int16), kc.view(torch.int16))
+    assert torch.equal(dev["v_cache"].cpu().view(torch.int16), vc.view(torch.int16))
+    check_out(got[0], ref[0], got[1], ref[1], "append")
+    # rotary
+    case = make_paged_case(B, hq, hk, d, page, lens, seqlen_new=1, seed=11)
+    from flash_attn_npu import flash_attn_with_kvcache
+    dev = to_dev(case)
+    out, lse = flash_attn_with_kvcache(dev["q"], dev["k_cache"], dev["v_cache"], dev["k"], dev["v"],
+                                       rotary_cos=cos.cuda(), rotary_sin=sin.cuda(), cache_seqlens=dev["cache_seqlens"],
+                                       block_table=dev["block_table"], causal=True, rotary_interleaved=interleaved,
+                                       return_softmax_lse=True)
+    kc, vc = case["k_cache"].clone(), case["v_cache"].clone()
+    ref, ref_lse = O.flash_attn_with_kvcache(case["q"], kc, vc, case["k"], case["v"], rotary_cos=cos, rotary_sin=sin,
+                                             cache_seqlens=case["cache_seqlens"], block_table=case["block_table"],
+                                             causal=True, rotary_interleaved=interleaved, mode="fp32")
+    assert torch.equal(dev["k_cache"].cpu().view(torch.int16), kc.view(torch.int16)), "rotated K bytes differ"
+    assert torch.equal(dev["v_cache"].cpu().view(torch.int16), vc.view(torch.int16))
+    check_out(out, ref, lse, ref_lse, "append+rotary")
+
+
+def test_append_multi_token_crosses_page():
+    case = make_paged_case(2, 8, 2, 128, 256, [254, 510], seqlen_q=3, seqlen_new=3, seed=12)
+    got, ref, gold, (dev, kc, vc) = run_both(case, causal=True)
+    assert torch.equal(dev["k_cache"].cpu().view(torch.int16), kc.view(torch.int16))
+    assert torch.equal(dev["v_cache"].cpu().view(torch.int16), vc.view(torch.int16))
+    check_out(got[0], ref[0], got[1], ref[1], "append3")
