@@ -1,0 +1,265 @@
+#!/usr/bin/env python3
+"""Benchmark of the paged KV-cache attention path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2|c2_8k|c3a|c3b|c4|c5] [--no-cpu]
+
+A step is one call of the hot path (append + rotary + attention + split combine for the decode
+configs, one varlen forward for c5) on synthetic inputs that are resident in HBM before the
+timed region.  Two input sets are alternated so that no step finds its K/V in the 256 MB
+last-level cache.  Prints ONE JSON line: whole-call throughput (`value`), the roofline record of
+the dominant kernel (its duration measured with HIP events the library records around it on the
+launch stream) and the CPU golden path timed on the host cores of this box.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (os.path.join(ROOT, "flash-attention-npu_amd"), os.path.join(ROOT, "oracle"), os.path.join(ROOT, "tests")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
+
+
+# ----------------------------------------------------------------------------- HIP events
+class HipEvents:
+    """hipEvent_t handles created through the HIP runtime the process already has loaded."""
+
+    def __init__(self, n: int):
+        self.hip = C.CDLL("libamdhip64.so")
+        self.hip.hipEventCreate.argtypes = [C.POINTER(C.c_void_p)]
+        self.hip.hipEventElapsedTime.argtypes = [C.POINTER(C.c_float), C.c_void_p, C.c_void_p]
+        self.hip.hipEventDestroy.argtypes = [C.c_void_p]
+        self.hip.hipEventRecord.argtypes = [C.c_void_p, C.c_void_p]
+        self.ev = (C.c_void_p * n)()
+        for i in range(n):
+            e = C.c_void_p()
+            rc = self.hip.hipEventCreate(C.byref(e))
+            if rc != 0:
+                raise RuntimeError(f"hipEventCreate failed: {rc}")
+            self.ev[i] = e
+
+    def group(self, i: int, width: int = 4):
+        return C.cast(C.byref(self.ev, i * width * C.sizeof(C.c_void_p)), C.POINTER(C.c_void_p))
+
+    def elapsed_ms(self, a: int, b: int) -> float:
+        ms = C.c_float()
+        rc = self.hip.hipEventElapsedTime(C.byref(ms), self.ev[a], self.ev[b])
+        if rc != 0:
+            raise RuntimeError(f"hipEventElapsedTime failed: {rc}")
+        return ms.value
+
+    def record(self, i: int, stream) -> None:
+        self.hip.hipEventRecord(self.ev[i], stream)
+
+    def close(self):
+        for e in self.ev:
+            self.hip.hipEventDestroy(e)
+
+
+# ----------------------------------------------------------------------------- workloads
+def decode_workload(name: str, device, seed: int = 0):
+    """Synthetic inputs of the decode configs (BASELINE.json configs[1..3]); returns a dict."""
+    import torch
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    page = 256
+    if name in ("c2", "c2_8k"):
+        B, hq, hk, d = 64, 32, 8, 128
+        if name == "c2":
+            # uniform in [1024, 8191]: the appended key sits at position len <= 8191 < seqlen_ro
+            lens = torch.randint(1024, 8192, (B,), generator=g)
+        else:
+            lens = torch.full((B,), 8191)
+        snew, rotary, window, spare = 1, True, (-1, -1), 64
+        desc = ("Llama-3-8B bf16 paged decode B=64 32q/8kv d=128 page=256 "
+                + ("lens U[1024,8191]" if name == "c2" else "all rows 8191 keys") + " append+RoPE causal")
+    elif name in ("c3a", "c3b"):
+        B, hq, hk, d = 4, 64, 8, 128
+        lens = torch.full((B,), 131072)
+        snew, rotary, spare = 0, False, 0
+        window = (-1, -1) if name == "c3a" else (4095, 0)
+        desc = f"long-context split-KV decode bf16 B=4 64q/8kv d=128 Lk=131072 window={window} causal"
+    else:
+        raise ValueError(name)
+    pages = [math.ceil((int(l) + snew) / page) for l in lens]
+    pool = sum(pages) + spare
+    perm = torch.randperm(pool, generator=g)
+    bt = torch.zeros(B, max(pages), dtype=torch.int32)
+    o = 0
+    for b in range(B):
+        bt[b, :pages[b]] = perm[o:o + pages[b]].to(torch.int32)
+        o += pages[b]
+    gd = torch.Generator(device=device).manual_seed(seed + 1)
+    dt = torch.bfloat16
+
+    def rn(*shape):
+        return torch.randn(*shape, generator=gd, device=device, dtype=torch.float32).to(dt)
+
+    w = dict(name=name, desc=desc, B=B, hq=hq, hk=hk, d=d, dv=d, page=page, lens=lens, snew=snew, window=window,
+             causal=True, scale=d ** -0.5,
+             q=rn(B, 1, hq, d), k_cache=rn(pool, page, hk, d), v_cache=rn(pool, page, hk, d),
+             cache_seqlens=lens.to(torch.int32).to(device), block_table=bt.to(device), k=None, v=None,
+             rotary_cos=None, rotary_sin=None)
+    if snew:
+        w["k"], w["v"] = rn(B, snew, hk, d), rn(B, snew, hk, d)
+    if rotary:
+        inv = 500000.0 ** (-torch.arange(0, d, 2, dtype=torch.float64) / d)
+        ang = torch.arange(8192, dtype=torch.float64)[:, None] * inv[None, :]
+        w["rotary_cos"], w["rotary_sin"] = torch.cos(ang).to(dt).to(device), torch.sin(ang).to(dt).to(device)
+    return w
+
+
+def decode_algorithmic_bytes(w):
+    """Algorithmic HBM bytes of one decode call: every visible K and V element once, q, out, LSE,
+    the block-table entries touched, plus (separately) the append's read+write."""
+    B, hq, hk, d, dv, page, snew = w["B"], w["hq"], w["hk"], w["d"], w["dv"], w["page"], w["snew"]
+    wl = w["window"][0]
+    kv = 0
+    tbl = 0
+    for l in w["lens"].tolist():
+        lk = l + snew
+        vis = lk if wl < 0 else min(lk, wl + 1)
+        kv += vis * hk * (d * 2 + dv * 2)
+        tbl += 4 * math.ceil(vis / page)
+    attn = kv + tbl + B * hq * (d * 2 + dv * 2) + B * hq * 4
+    append = B * snew * hk * (d + dv) * (2 + 2)
+    return attn, append
+
+
+def bind_decode(w):
+    from flash_attn_npu import flash_attn_npu as ops
+    return ops.bind_kvcache(w["q"], w["k_cache"], w["v_cache"], w["k"], w["v"], w["cache_seqlens"], w["rotary_cos"],
+                            w["rotary_sin"], None, None, w["block_table"], None, None, w["scale"], w["causal"],
+                            w["window"][0], w["window"][1], 0.0, False, 0)
+
+
+def cpu_decode_baseline(w, budget_s: float = 20.0):
+    """The oracle's blocked golden (restated reference test golden) on host cores."""
+    import torch
+    import fa_oracle as O
+    keys = ("q", "k_cache", "v_cache", "k", "v", "cache_seqlens", "block_table", "rotary_cos", "rotary_sin")
+    h = {k: (w[k].cpu() if isinstance(w[k], torch.Tensor) else w[k]) for k in keys}
+    # bounded sample: leading batch rows until the budget is used up
+    B = w["B"]
+    rows = B
+    t0 = time.perf_counter()
+    done = 0
+    times = []
+    for start in range(0, B):
+        sl = slice(start, start + 1)
+        t1 = time.perf_counter()
+        O.flash_attn_with_kvcache(h["q"][sl], h["k_cache"], h["v_cache"],
+                                  None if h["k"] is None else h["k"][sl], None if h["v"] is None else h["v"][sl],
+                                  rotary_cos=h["rotary_cos"], rotary_sin=h["rotary_sin"],
+                                  cache_seqlens=h["cache_seqlens"][sl], block_table=h["block_table"][sl],
+                                  softmax_scale=w["scale"], causal=w["causal"], window_size=w["window"],
+                                  rotary_interleaved=False, mode="golden")
+        times.append(time.perf_counter() - t1)
+        done += 1
+        if time.perf_counter() - t0 > budget_s:
+            break
+    sub = dict(w)
+    sub["lens"] = w["lens"][:done]
+    sub["B"] = done
+    attn, app = decode_algorithmic_bytes(sub)
+    secs = sum(times)
+    return dict(value=(attn + app) / secs / 1e9, unit="GB/s", cores=torch.get_num_threads(), kind="port",
+                sample=f"oracle blocked golden (fp32 math, 512-key chunks) on the first {done} of {rows} batch rows "
+                       f"of the same workload, {secs:.2f} s on {os.cpu_count()} host cpus, "
+                       f"torch threads {torch.get_num_threads()}",
+                ms_per_call_extrapolated=secs / done * rows * 1e3)
+
+
+# ----------------------------------------------------------------------------- main
+def run_decode(args, name):
+    import torch
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    sets = [decode_workload(name, dev, seed=s) for s in (0, 0)]
+    # same seed -> same lengths and table, but two distinct physical pools, so that alternating
+    # them evicts the last-level cache between steps
+    calls = [bind_decode(w) for w in sets]
+    w = sets[0]
+    attn_bytes, append_bytes = decode_algorithmic_bytes(w)
+    total_bytes = attn_bytes + append_bytes
+
+    for i in range(args.warmup):
+        calls[i % 2].run()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        calls[i % 2].run()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall / args.steps * 1e3
+
+    # second timed pass with the library's phase events: duration of the attention kernel alone
+    ev = HipEvents(4 * args.steps)
+    for i in range(args.steps):
+        calls[i % 2].run(events=ev.group(i))
+    torch.cuda.synchronize()
+    k_ms = [ev.elapsed_ms(4 * i + 1, 4 * i + 2) for i in range(args.steps)]
+    a_ms = [ev.elapsed_ms(4 * i + 0, 4 * i + 1) for i in range(args.steps)]
+    c_ms = [ev.elapsed_ms(4 * i + 2, 4 * i + 3) for i in range(args.steps)]
+    ev.close()
+    kern_ms = sum(k_ms) / len(k_ms)
+    achieved = attn_bytes / (kern_ms * 1e-3) / 1e9
+
+    from flash_attn_npu import _lib
+    lib = _lib.load()
+    sk = C.c_int32()
+    nsplits = lib.fa_rocm_choose_splits(C.byref(calls[0].args), lib.fa_rocm_num_cus(), C.byref(sk))
+
+    out = {
+        "metric": "paged_decode_hbm_bandwidth", "value": total_bytes / (ms_per_step * 1e-3) / 1e9, "unit": "GB/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"{name}: {w['desc']}", "batch": w["B"], "q_heads": w["hq"], "kv_heads": w["hk"],
+                   "headdim": w["d"], "page_block_size": w["page"], "sum_keys": int(w["lens"].sum()) + w["B"] * w["snew"],
+                   "kv_splits": nsplits, "split_keys": sk.value, "cold_cache": "two pools alternated"},
+        "us_per_call": ms_per_step * 1e3,
+        "pct_of_hbm_peak": 100.0 * total_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+        "algorithmic_bytes": total_bytes,
+        "roofline": {"bound": "hbm", "kernel": "decode_paged_kernel", "achieved": achieved, "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS, "traffic": None,
+                     "kernel_us": kern_ms * 1e3, "append_us": sum(a_ms) / len(a_ms) * 1e3,
+                     "combine_us": sum(c_ms) / len(c_ms) * 1e3, "algorithmic_bytes_per_launch": attn_bytes},
+    }
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_decode_baseline(w)
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--config", default="c2")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU golden timing")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: the hot path has no cross-GPU exchange and this build uses a single "
+              "MI355X; run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py needs a ROCm GPU", file=sys.stderr)
+        sys.exit(2)
+    if args.config in ("c2", "c2_8k", "c3a", "c3b"):
+        out = run_decode(args, args.config)
+    else:
+        raise SystemExit(f"unknown config {args.config}")
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -212,10 +212,23 @@ int fa_rocm_append_kv(const fa_kvcache_args *a, void *stream) {
     return FA_OK;
 }
 
-int fa_rocm_fwd_kvcache(const fa_kvcache_args *a, void *stream_) {
+static int fwd_kvcache_impl(const fa_kvcache_args *a, void *stream_, void *const *events);
+
+int fa_rocm_fwd_kvcache(const fa_kvcache_args *a, void *stream_) { return fwd_kvcache_impl(a, stream_, nullptr); }
+
+int fa_rocm_fwd_kvcache_profiled(const fa_kvcache_args *a, void *stream_, void *const events[4]) {
+    if (!events) return fail(FA_ERR_NULL, "events is NULL");
+    return fwd_kvcache_impl(a, stream_, events);
+}
+
+static int fwd_kvcache_impl(const fa_kvcache_args *a, void *stream_, void *const *events) {
     int rc = fa_rocm_kvcache_validate(a);
     if (rc != FA_OK) return rc;
     hipStream_t stream = static_cast<hipStream_t>(stream_);
+    auto mark = [&](int i) {
+        if (events) (void)hipEventRecord(static_cast<hipEvent_t>(events[i]), stream);
+    };
+    mark(0);
     const int group = a->nheads / a->nheads_k;
     const int rows = a->seqlen_q * group;
 
@@ -224,6 +237,7 @@ int fa_rocm_fwd_kvcache(const fa_kvcache_args *a, void *stream_) {
         if (rc != FA_OK) return rc;
     }
 
+    mark(1);
     const bool local = a->window_left >= 0 || a->window_right >= 0;
 
     if (!is_mla_i8(a) && rows > fa::kDecodeMaxRows) {
@@ -275,6 +289,8 @@ int fa_rocm_fwd_kvcache(const fa_kvcache_args *a, void *stream_) {
             return fail(FA_ERR_UNSUPPORTED, "rotary embedding needs seqlen_q * (nheads / nheads_k) <= %d", fa::kDecodeMaxRows);
         const hipError_t e = fa::launch_prefill(pp, a->io_dtype, a->headdim_qk, stream);
         if (e != hipSuccess) return fail(FA_ERR_LAUNCH, "prefill launch failed: %s", hipGetErrorString(e));
+        mark(2);
+        mark(3);
         return FA_OK;
     }
 
@@ -350,10 +366,12 @@ int fa_rocm_fwd_kvcache(const fa_kvcache_args *a, void *stream_) {
     else
         e = fa::launch_decode_paged(p, a->io_dtype, a->headdim_qk, stream);
     if (e != hipSuccess) return fail(FA_ERR_LAUNCH, "decode launch failed: %s", hipGetErrorString(e));
+    mark(2);
     if (nsplits > 1) {
         e = fa::launch_splitkv_combine(p, a->io_dtype, a->headdim_v, stream);
         if (e != hipSuccess) return fail(FA_ERR_LAUNCH, "combine launch failed: %s", hipGetErrorString(e));
     }
+    mark(3);
     return FA_OK;
 }
 

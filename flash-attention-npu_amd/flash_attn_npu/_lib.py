@@ -59,6 +59,7 @@ EXPORTS = {
     "fa_rocm_kvcache_validate": (C.c_int, [C.POINTER(KvcacheArgs)]),
     "fa_rocm_varlen_validate": (C.c_int, [C.POINTER(VarlenArgs)]),
     "fa_rocm_fwd_kvcache": (C.c_int, [C.POINTER(KvcacheArgs), _vp]),
+    "fa_rocm_fwd_kvcache_profiled": (C.c_int, [C.POINTER(KvcacheArgs), _vp, C.POINTER(_vp)]),
     "fa_rocm_varlen_fwd": (C.c_int, [C.POINTER(VarlenArgs), _vp]),
     "fa_rocm_append_kv": (C.c_int, [C.POINTER(KvcacheArgs), _vp]),
 }

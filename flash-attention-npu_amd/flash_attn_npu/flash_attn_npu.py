@@ -35,11 +35,40 @@ def _require_device(*tensors) -> None:
             raise RuntimeError("flash_attn_npu (MI355X build) needs tensors on a ROCm device; there is no CPU path")
 
 
+class KvcacheCall:
+    """One validated, fully bound kvcache call: the argument record, the output tensors and the
+    tensors that must stay alive.  `run()` enqueues it on the current stream; a serving loop or a
+    benchmark can bind once and run many times (the record holds raw pointers)."""
+
+    def __init__(self, args, out, lse, keep, device):
+        self.args, self.out, self.lse, self.keep, self.device = args, out, lse, keep, device
+
+    def run(self, events=None) -> None:
+        lib = _lib.load()
+        with torch.cuda.device(self.device):
+            stream = C.c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
+            if events is None:
+                _lib.check(lib.fa_rocm_fwd_kvcache(C.byref(self.args), stream))
+            else:
+                _lib.check(lib.fa_rocm_fwd_kvcache_profiled(C.byref(self.args), stream, events))
+
+
 def fwd_kvcache(q, kcache, vcache, k_, v_, seqlens_k_, rotary_cos_, rotary_sin_, cache_batch_idx_, leftpad_k_,
                 block_table_, alibi_slopes_, out_, softmax_scale, is_causal, window_size_left, window_size_right,
                 softcap, is_rotary_interleaved, num_splits, k_scale_cache_=None, v_scale_cache_=None
                 ) -> List[torch.Tensor]:
     """mha_fwd_kvcache (flash_api.cpp:356-637) on a paged cache.  Returns [out, softmax_lse]."""
+    call = bind_kvcache(q, kcache, vcache, k_, v_, seqlens_k_, rotary_cos_, rotary_sin_, cache_batch_idx_, leftpad_k_,
+                        block_table_, alibi_slopes_, out_, softmax_scale, is_causal, window_size_left,
+                        window_size_right, softcap, is_rotary_interleaved, num_splits, k_scale_cache_, v_scale_cache_)
+    call.run()
+    return [call.out, call.lse]
+
+
+def bind_kvcache(q, kcache, vcache, k_, v_, seqlens_k_, rotary_cos_, rotary_sin_, cache_batch_idx_, leftpad_k_,
+                 block_table_, alibi_slopes_, out_, softmax_scale, is_causal, window_size_left, window_size_right,
+                 softcap, is_rotary_interleaved, num_splits, k_scale_cache_=None, v_scale_cache_=None) -> KvcacheCall:
+    """Checks of mha_fwd_kvcache (flash_api.cpp:386-420,455-457) and binding of the C argument record."""
     lib = _lib.load()
     is_i8 = kcache.dtype == torch.int8
     _require(q.dtype in (torch.bfloat16, torch.float16), "FlashAttention only supports FP16 and BF16 data types")
@@ -101,7 +130,7 @@ def fwd_kvcache(q, kcache, vcache, k_, v_, seqlens_k_, rotary_cos_, rotary_sin_,
         if v_scale_cache_ is not None:
             _require(v_scale_cache_.stride() == k_scale_cache_.stride() and v_scale_cache_.dtype == torch.float32,
                      "v_scale_cache must match k_scale_cache's layout")
-    keep = [seqlens_k]
+    keep = [q, kcache, vcache, seqlens_k, block_table_, k_scale_cache_, v_scale_cache_]
     if k_ is not None or v_ is not None:
         _require(k_ is not None and v_ is not None, "k and v must be passed together")
         _require(k_.dtype == q.dtype and v_.dtype == q.dtype, "Key and value must have the same dtype as query")
@@ -140,8 +169,7 @@ def fwd_kvcache(q, kcache, vcache, k_, v_, seqlens_k_, rotary_cos_, rotary_sin_,
             ws = torch.empty((need + 3) // 4, dtype=torch.float32, device=q.device)
             keep.append(ws)
             a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel() * 4
-        _lib.check(lib.fa_rocm_fwd_kvcache(C.byref(a), _stream(q)))
-    return [out, lse]
+    return KvcacheCall(a, out, lse, keep, q.device)
 
 
 def varlen_fwd(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k_, leftpad_k_, block_table_, alibi_slopes_,

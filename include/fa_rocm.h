@@ -159,6 +159,15 @@ int fa_rocm_varlen_validate(const fa_varlen_args *args);
 int fa_rocm_fwd_kvcache(const fa_kvcache_args *args, void *stream);
 
 /*
+ * Same call with phase timing for benchmarks: `events` holds four hipEvent_t handles that the
+ * library records on `stream` before the append, after it (before the attention kernel), after
+ * the attention kernel and after the combine.  hipEventElapsedTime(events[1], events[2]) is the
+ * attention kernel alone.  No counterpart in the reference (its unused host timers are at
+ * csrc/ascend910/flash_attn_npu_3/flash_api.cpp:99).
+ */
+int fa_rocm_fwd_kvcache_profiled(const fa_kvcache_args *args, void *stream, void *const events[4]);
+
+/*
  * flash_attn_varlen_func forward.  Replaces mha_varlen_fwd
  * (csrc/ascend910/flash_attn_npu/flash_api.cpp:848-1089).
  */
