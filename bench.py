@@ -66,7 +66,7 @@ class HipEvents:
 
 
 # ----------------------------------------------------------------------------- workloads
-def decode_workload(name: str, device, seed: int = 0):
+def decode_workload(name: str, device, seed: int = 0, kv_layout: str = "nhd"):
     """Synthetic inputs of the decode configs (BASELINE.json configs[1..3]); returns a dict."""
     import torch
     g = torch.Generator(device="cpu").manual_seed(seed)
@@ -103,9 +103,17 @@ def decode_workload(name: str, device, seed: int = 0):
     def rn(*shape):
         return torch.randn(*shape, generator=gd, device=device, dtype=torch.float32).to(dt)
 
+    def cache(*shape):
+        # "nhd": (num_blocks, page, Hk, d) contiguous, the layout the API documents;
+        # "hnd": same logical shape, memory laid out (num_blocks, Hk, page, d)
+        if kv_layout == "hnd":
+            nb, pg, h, dd = shape
+            return rn(nb, h, pg, dd).permute(0, 2, 1, 3)
+        return rn(*shape)
+
     w = dict(name=name, desc=desc, B=B, hq=hq, hk=hk, d=d, dv=d, page=page, lens=lens, snew=snew, window=window,
              causal=True, scale=d ** -0.5,
-             q=rn(B, 1, hq, d), k_cache=rn(pool, page, hk, d), v_cache=rn(pool, page, hk, d),
+             q=rn(B, 1, hq, d), k_cache=cache(pool, page, hk, d), v_cache=cache(pool, page, hk, d),
              cache_seqlens=lens.to(torch.int32).to(device), block_table=bt.to(device), k=None, v=None,
              rotary_cos=None, rotary_sin=None)
     if snew:
@@ -134,11 +142,11 @@ def decode_algorithmic_bytes(w):
     return attn, append
 
 
-def bind_decode(w):
+def bind_decode(w, num_splits=0):
     from flash_attn_npu import flash_attn_npu as ops
     return ops.bind_kvcache(w["q"], w["k_cache"], w["v_cache"], w["k"], w["v"], w["cache_seqlens"], w["rotary_cos"],
                             w["rotary_sin"], None, None, w["block_table"], None, None, w["scale"], w["causal"],
-                            w["window"][0], w["window"][1], 0.0, False, 0)
+                            w["window"][0], w["window"][1], 0.0, False, num_splits)
 
 
 def cpu_decode_baseline(w, budget_s: float = 20.0):
@@ -183,10 +191,10 @@ def run_decode(args, name):
     import torch
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    sets = [decode_workload(name, dev, seed=s) for s in (0, 0)]
+    sets = [decode_workload(name, dev, seed=s, kv_layout=args.kv_layout) for s in (0, 0)]
     # same seed -> same lengths and table, but two distinct physical pools, so that alternating
     # them evicts the last-level cache between steps
-    calls = [bind_decode(w) for w in sets]
+    calls = [bind_decode(w, args.num_splits) for w in sets]
     w = sets[0]
     attn_bytes, append_bytes = decode_algorithmic_bytes(w)
     total_bytes = attn_bytes + append_bytes
@@ -215,8 +223,8 @@ def run_decode(args, name):
 
     from flash_attn_npu import _lib
     lib = _lib.load()
-    sk = C.c_int32()
-    nsplits = lib.fa_rocm_choose_splits(C.byref(calls[0].args), lib.fa_rocm_num_cus(), C.byref(sk))
+    plan = _lib.SplitPlan()
+    lib.fa_rocm_plan_kvcache(C.byref(calls[0].args), lib.fa_rocm_num_cus(), C.byref(plan))
 
     out = {
         "metric": "paged_decode_hbm_bandwidth", "value": total_bytes / (ms_per_step * 1e-3) / 1e9, "unit": "GB/s",
@@ -224,7 +232,8 @@ def run_decode(args, name):
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"{name}: {w['desc']}", "batch": w["B"], "q_heads": w["hq"], "kv_heads": w["hk"],
                    "headdim": w["d"], "page_block_size": w["page"], "sum_keys": int(w["lens"].sum()) + w["B"] * w["snew"],
-                   "kv_splits": nsplits, "split_keys": sk.value, "cold_cache": "two pools alternated"},
+                   "split_mode": "balanced" if plan.mode == 1 else "grid", "workgroups": plan.num_wgs,
+                   "kv_splits": plan.nsplits, "split_keys": plan.split_keys, "cold_cache": "two pools alternated", "kv_layout": args.kv_layout},
         "us_per_call": ms_per_step * 1e3,
         "pct_of_hbm_peak": 100.0 * total_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,
         "algorithmic_bytes": total_bytes,
@@ -238,12 +247,34 @@ def run_decode(args, name):
     return out
 
 
+def run_copy(args):
+    """Plain device copy of known size (1 GiB read + 1 GiB written per step): the calibration
+    workload for the FETCH_SIZE / WRITE_SIZE counters and a practical bandwidth yardstick."""
+    import torch
+    n = 1 << 30
+    src = torch.empty(n, dtype=torch.uint8, device="cuda:0").random_(0, 255)
+    dst = torch.empty_like(src)
+    for _ in range(args.warmup):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / args.steps * 1e3
+    return {"metric": "device_copy_bandwidth", "value": 2 * n / (ms * 1e-3) / 1e9, "unit": "GB/s", "n_gpus": 1,
+            "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True,
+            "config": {"workload": "copy: 1 GiB torch copy_ (read 1 GiB + write 1 GiB per step)"}}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--config", default="c2")
+    ap.add_argument("--num-splits", type=int, default=0, help="0 = balanced partition (default), n >= 1 = fixed splits")
+    ap.add_argument("--kv-layout", default="nhd", choices=["nhd", "hnd"], help="memory layout of the paged caches")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU golden timing")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -256,6 +287,8 @@ def main():
         sys.exit(2)
     if args.config in ("c2", "c2_8k", "c3a", "c3b"):
         out = run_decode(args, args.config)
+    elif args.config == "copy":
+        out = run_copy(args)
     else:
         raise SystemExit(f"unknown config {args.config}")
     print(json.dumps(out))

@@ -36,9 +36,40 @@ template <int D> __device__ __forceinline__ int k_tile_offset(int row, int ch) {
     return row * (D * 2) + ((ch ^ (row & DecodeCfg<D>::kSwzMask)) << 4);
 }
 
+// Live key range [lo, hi) of the query block of batch row b, and its 32-key chunk span.
+struct UnitRange {
+    int len_cache, Lk, lo, hi;
+    int c0, nchunks;  // first chunk index (absolute) and number of chunks; nchunks == 0: nothing visible
+};
+
+__device__ __forceinline__ UnitRange unit_range(const DecodeParams &p, int b) {
+    UnitRange u;
+    u.len_cache = p.cache_seqlens[b];
+    u.Lk = u.len_cache + p.seqlen_new;
+    const int off = u.Lk - p.seqlen_q;
+    const int wr_eff = p.causal ? 0 : p.window_right;
+    u.lo = 0;
+    u.hi = u.Lk;
+    if (wr_eff >= 0) u.hi = min(u.Lk, p.seqlen_q - 1 + off + wr_eff + 1);
+    if (p.window_left >= 0) u.lo = max(0, off - p.window_left);
+    // keys the block table cannot address are not read
+    u.hi = min(u.hi, p.max_blocks * p.page_size);
+    if (u.Lk <= 0 || u.hi <= u.lo) {
+        u.lo = u.hi = 0;
+        u.c0 = u.nchunks = 0;
+    } else {
+        u.c0 = u.lo / kChunk;
+        u.nchunks = (u.hi + kChunk - 1) / kChunk - u.c0;
+    }
+    return u;
+}
+
+// One piece of work: query block (b, kvh) against keys [range_lo, range_hi).  Writes the final
+// output when `write_final`, else the normalised fp32 partial and its base-2 LSE into `slot`.
 template <typename T, int D, int RT, int NW, bool SOFTCAP>
-__global__ void __launch_bounds__(NW * 64, (D <= 128 && RT <= 2) ? 2 : 1)
-decode_paged_kernel(const DecodeParams p) {
+__device__ __forceinline__ void process_piece(const DecodeParams &p, const int b, const int kvh, const UnitRange &ur,
+                                              const int range_lo, const int range_hi, const bool write_final,
+                                              const int64_t slot) {
     using Cfg = DecodeCfg<D>;
     constexpr int ROWS = 16 * RT;
     constexpr int K_TILE_BYTES = kChunk * D * 2;
@@ -56,38 +87,120 @@ decode_paged_kernel(const DecodeParams p) {
     const int lq = lane >> 4;   // lane group: MFMA k-slot / key sub-block
     const int ln = lane & 15;   // MFMA row or column index
 
-    const int split = blockIdx.x;
-    const int kvh = blockIdx.y;
-    const int b = blockIdx.z;
-
-    const int len_cache = p.cache_seqlens[b];
-    const int Lk = len_cache + p.seqlen_new;
+    const int len_cache = ur.len_cache;
+    const int Lk = ur.Lk;
     const int Sq = p.seqlen_q;
     const int off = Lk - Sq;
     const int wr_eff = p.causal ? 0 : p.window_right;
     const int wl = p.window_left;
 
-    // live key range of the whole query block
-    int lo = 0, hi = Lk;
-    if (wr_eff >= 0) hi = min(Lk, Sq - 1 + off + wr_eff + 1);
-    if (wl >= 0) lo = max(0, off - wl);
-    const bool empty = (Lk <= 0) || (hi <= lo);
-    const int lo_al = lo & ~(kChunk - 1);
-    // splits this row really has; the grid was sized from shapes, so clamp and let the last split
-    // run to the end of the range if the caller's lengths exceed what the shapes promised
-    const int nsplits_row = empty ? 1 : min(p.nsplits, (hi - lo_al + p.split_keys - 1) / p.split_keys);
-    if (split >= nsplits_row) return;
-    const bool write_final = (nsplits_row == 1);
-
-    int range_lo = lo, range_hi = hi;
-    if (!empty) {
-        range_lo = max(lo, lo_al + split * p.split_keys);
-        range_hi = (split == nsplits_row - 1) ? hi : min(hi, lo_al + (split + 1) * p.split_keys);
-    } else {
-        range_lo = 0;
-        range_hi = 0;
+    // per-lane visible key interval of query row (r*16 + ln), clipped to this split
+    int row_lo[RT], row_hi[RT];
+#pragma unroll
+    for (int r = 0; r < RT; ++r) {
+        const int row = r * 16 + ln;
+        const int qi = row / p.group;
+        int klo = range_lo, khi = range_hi - 1;
+        if (wl >= 0) klo = max(klo, qi + off - wl);
+        if (wr_eff >= 0) khi = min(khi, qi + off + wr_eff);
+        if (row >= p.rows) khi = -1;
+        row_lo[r] = klo;
+        row_hi[r] = khi;
     }
 
+    float m_run[RT], l_run[RT];
+    float4_t o_acc[RT][Cfg::kColTiles];
+#pragma unroll
+    for (int r = 0; r < RT; ++r) {
+        m_run[r] = -INFINITY;
+        l_run[r] = 0.f;
+#pragma unroll
+        for (int t = 0; t < Cfg::kColTiles; ++t) o_acc[r][t] = float4_t{0.f, 0.f, 0.f, 0.f};
+    }
+
+    uint8_t *ktile = s_main + wave * K_TILE_BYTES;
+    const uint8_t *kc_base = reinterpret_cast<const uint8_t *>(p.k_cache) + (int64_t)kvh * p.k_stride_h * 2;
+    const uint8_t *vc_base = reinterpret_cast<const uint8_t *>(p.v_cache) + (int64_t)kvh * p.v_stride_h * 2;
+    const int32_t *bt_row = p.block_table + (int64_t)b * p.bt_stride_b;
+
+    const int c_begin = range_lo / kChunk;
+    const int c_end = (range_hi + kChunk - 1) / kChunk;
+
+    u32x4_t kreg[Cfg::kKLoads];
+    uint32_t vreg[8][Cfg::kVH][Cfg::kVW / 2];
+
+    // per-lane byte offsets inside a page that do not change from chunk to chunk; the per-load
+    // part is wave-uniform and folds into the scalar base address
+    const uint32_t k_row_bytes = (uint32_t)p.k_stride_row * 2u;
+    const uint32_t v_row_bytes = (uint32_t)p.v_stride_row * 2u;
+    const int k_lane_row = lane / Cfg::kLanesPerRow;
+    const uint32_t k_lane_col = (uint32_t)(lane % Cfg::kLanesPerRow) * 16u;
+    const uint32_t v_lane_col = (uint32_t)(ln * Cfg::kVW) * 2u;
+    const uint32_t k_lane_off = (uint32_t)k_lane_row * k_row_bytes + k_lane_col;
+    const uint32_t v_lane_off = (uint32_t)(lq * 4) * v_row_bytes + v_lane_col;
+
+    // page id of chunk c (clamped into the pool so a corrupt table cannot fault)
+    auto fetch_blk = [&](int c) -> int {
+        if (c >= c_end) return 0;
+        int page = (c * kChunk) / p.page_size;
+        page = min(page, p.max_blocks - 1);
+        const int blk = __builtin_amdgcn_readfirstlane(bt_row[page]);
+        return min(max(blk, 0), p.num_blocks - 1);
+    };
+
+    auto load_v = [&](const uint8_t *s2, int e, int hh) {
+        if constexpr (Cfg::kVW == 8) {
+            const u32x4_t t4 = load16(s2);
+            vreg[e][hh][0] = t4[0];
+            vreg[e][hh][1] = t4[1];
+            vreg[e][hh][2] = t4[2];
+            vreg[e][hh][3] = t4[3];
+        } else if constexpr (Cfg::kVW == 4) {
+            const uint2 t2 = *reinterpret_cast<const uint2 *>(s2);
+            vreg[e][hh][0] = t2.x;
+            vreg[e][hh][1] = t2.y;
+        } else {
+            vreg[e][hh][0] = *reinterpret_cast<const uint32_t *>(s2);
+        }
+    };
+
+    auto issue_loads = [&](int c, int blk) {
+        const int key0 = c * kChunk;
+        const int inpage0 = key0 % p.page_size;
+        const int last = Lk - 1 - key0;  // last initialised key, relative to the chunk (>= 0)
+        const uint8_t *kb = kc_base + (int64_t)blk * p.k_stride_block * 2 + (int64_t)inpage0 * k_row_bytes;
+        const uint8_t *vb = vc_base + (int64_t)blk * p.v_stride_block * 2 + (int64_t)inpage0 * v_row_bytes;
+        if (last >= kChunk - 1) {
+#pragma unroll
+            for (int j = 0; j < Cfg::kKLoads; ++j)
+                kreg[j] = load16(kb + (size_t)(j * Cfg::kRowsPerLoad) * k_row_bytes + k_lane_off);
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+#pragma unroll
+                for (int hh = 0; hh < Cfg::kVH; ++hh)
+                    load_v(vb + (size_t)((e >> 2) * 16 + (e & 3)) * v_row_bytes + hh * 256 + v_lane_off, e, hh);
+        } else {
+            // tail chunk: rows past the last written key re-read that key (their scores are masked)
+#pragma unroll
+            for (int j = 0; j < Cfg::kKLoads; ++j) {
+                const int row = min(j * Cfg::kRowsPerLoad + k_lane_row, last);
+                kreg[j] = load16(kb + (uint32_t)row * k_row_bytes + k_lane_col);
+            }
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const int row = min((e >> 2) * 16 + lq * 4 + (e & 3), last);
+#pragma unroll
+                for (int hh = 0; hh < Cfg::kVH; ++hh) load_v(vb + (uint32_t)row * v_row_bytes + v_lane_col + hh * 256, e, hh);
+            }
+        }
+    };
+
+    int c = c_begin + wave;
+    int blk_next = fetch_blk(c);
+    if (c < c_end) issue_loads(c, blk_next);
+    blk_next = fetch_blk(c + NW);
+
+    // (the first chunk is already in flight while Q is staged)
     // ---- stage Q (with rotary) into LDS as 16-bit rows -------------------------------------
     {
         const uint16_t *qbase = reinterpret_cast<const uint16_t *>(p.q) + (int64_t)b * p.q_stride_b;
@@ -138,112 +251,6 @@ decode_paged_kernel(const DecodeParams p) {
 #pragma unroll
         for (int t = 0; t < Cfg::kKSteps; ++t)
             qreg[r][t] = *reinterpret_cast<const u32x4_t *>(&s_q[(r * 16 + ln) * D + t * 32 + lq * 8]);
-
-    // per-lane visible key interval of query row (r*16 + ln), clipped to this split
-    int row_lo[RT], row_hi[RT];
-#pragma unroll
-    for (int r = 0; r < RT; ++r) {
-        const int row = r * 16 + ln;
-        const int qi = row / p.group;
-        int klo = range_lo, khi = range_hi - 1;
-        if (wl >= 0) klo = max(klo, qi + off - wl);
-        if (wr_eff >= 0) khi = min(khi, qi + off + wr_eff);
-        if (row >= p.rows) khi = -1;
-        row_lo[r] = klo;
-        row_hi[r] = khi;
-    }
-
-    float m_run[RT], l_run[RT];
-    float4_t o_acc[RT][Cfg::kColTiles];
-#pragma unroll
-    for (int r = 0; r < RT; ++r) {
-        m_run[r] = -INFINITY;
-        l_run[r] = 0.f;
-#pragma unroll
-        for (int t = 0; t < Cfg::kColTiles; ++t) o_acc[r][t] = float4_t{0.f, 0.f, 0.f, 0.f};
-    }
-
-    uint8_t *ktile = s_main + wave * K_TILE_BYTES;
-    const uint8_t *kc_base = reinterpret_cast<const uint8_t *>(p.k_cache) + (int64_t)kvh * p.k_stride_h * 2;
-    const uint8_t *vc_base = reinterpret_cast<const uint8_t *>(p.v_cache) + (int64_t)kvh * p.v_stride_h * 2;
-    const int32_t *bt_row = p.block_table + (int64_t)b * p.bt_stride_b;
-
-    const int c_begin = range_lo / kChunk;
-    const int c_end = (range_hi + kChunk - 1) / kChunk;
-
-    u32x4_t kreg[Cfg::kKLoads];
-    uint32_t vreg[8][Cfg::kVH][Cfg::kVW / 2];
-
-    // per-lane byte offsets inside a page that do not change from chunk to chunk
-    const uint32_t k_row_bytes = (uint32_t)p.k_stride_row * 2u;
-    const uint32_t v_row_bytes = (uint32_t)p.v_stride_row * 2u;
-    const int k_lane_row = lane / Cfg::kLanesPerRow;
-    const uint32_t k_lane_col = (uint32_t)(lane % Cfg::kLanesPerRow) * 16u;
-    const uint32_t v_lane_col = (uint32_t)(ln * Cfg::kVW) * 2u;
-    uint32_t koff[Cfg::kKLoads], voff[8];
-#pragma unroll
-    for (int j = 0; j < Cfg::kKLoads; ++j) koff[j] = (uint32_t)(j * Cfg::kRowsPerLoad + k_lane_row) * k_row_bytes + k_lane_col;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) voff[e] = (uint32_t)((e >> 2) * 16 + lq * 4 + (e & 3)) * v_row_bytes + v_lane_col;
-
-    // page id of chunk c (clamped into the pool so a corrupt table cannot fault)
-    auto fetch_blk = [&](int c) -> int {
-        if (c >= c_end) return 0;
-        int page = (c * kChunk) / p.page_size;
-        page = min(page, p.max_blocks - 1);
-        const int blk = __builtin_amdgcn_readfirstlane(bt_row[page]);
-        return min(max(blk, 0), p.num_blocks - 1);
-    };
-
-    auto load_v = [&](const uint8_t *s2, int e, int hh) {
-        if constexpr (Cfg::kVW == 8) {
-            const u32x4_t t4 = load16(s2);
-            vreg[e][hh][0] = t4[0];
-            vreg[e][hh][1] = t4[1];
-            vreg[e][hh][2] = t4[2];
-            vreg[e][hh][3] = t4[3];
-        } else if constexpr (Cfg::kVW == 4) {
-            const uint2 t2 = *reinterpret_cast<const uint2 *>(s2);
-            vreg[e][hh][0] = t2.x;
-            vreg[e][hh][1] = t2.y;
-        } else {
-            vreg[e][hh][0] = *reinterpret_cast<const uint32_t *>(s2);
-        }
-    };
-
-    auto issue_loads = [&](int c, int blk) {
-        const int key0 = c * kChunk;
-        const int inpage0 = key0 % p.page_size;
-        const int last = Lk - 1 - key0;  // last initialised key, relative to the chunk (>= 0)
-        const uint8_t *kb = kc_base + (int64_t)blk * p.k_stride_block * 2 + (int64_t)inpage0 * k_row_bytes;
-        const uint8_t *vb = vc_base + (int64_t)blk * p.v_stride_block * 2 + (int64_t)inpage0 * v_row_bytes;
-        if (last >= kChunk - 1) {
-#pragma unroll
-            for (int j = 0; j < Cfg::kKLoads; ++j) kreg[j] = load16(kb + koff[j]);
-#pragma unroll
-            for (int e = 0; e < 8; ++e)
-#pragma unroll
-                for (int hh = 0; hh < Cfg::kVH; ++hh) load_v(vb + voff[e] + hh * 256, e, hh);
-        } else {
-            // tail chunk: rows past the last written key re-read that key (their scores are masked)
-#pragma unroll
-            for (int j = 0; j < Cfg::kKLoads; ++j) {
-                const int row = min(j * Cfg::kRowsPerLoad + k_lane_row, last);
-                kreg[j] = load16(kb + (uint32_t)row * k_row_bytes + k_lane_col);
-            }
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const int row = min((e >> 2) * 16 + lq * 4 + (e & 3), last);
-#pragma unroll
-                for (int hh = 0; hh < Cfg::kVH; ++hh) load_v(vb + (uint32_t)row * v_row_bytes + v_lane_col + hh * 256, e, hh);
-            }
-        }
-    };
-
-    int c = c_begin + wave;
-    int blk_next = fetch_blk(c);
-    if (c < c_end) issue_loads(c, blk_next);
-    blk_next = fetch_blk(c + NW);
 
     while (c < c_end) {
         // ---- move the staged chunk: K -> swizzled LDS tile, V -> transposed operand registers
@@ -368,24 +375,40 @@ decode_paged_kernel(const DecodeParams p) {
         fac[r] = fast_exp2(m_run[r] - mg_use);
     }
 
-    float *o_stage = reinterpret_cast<float *>(s_main);  // [ROWS][D]
-    for (int w = 0; w < NW; ++w) {
-        if (wave == w) {
+    float *o_stage = reinterpret_cast<float *>(s_main);  // [ROWS][D], or [NW][ROWS][D] when RT == 1
+    constexpr bool kParallelMerge = (RT == 1);
+    if constexpr (kParallelMerge) {
+        // every wave drops its rescaled accumulator into its own buffer; the writers add them up
+        float *mine = o_stage + wave * (ROWS * D);
 #pragma unroll
-            for (int r = 0; r < RT; ++r)
+        for (int t = 0; t < Cfg::kColTiles; ++t) {
+            const int hh = t / Cfg::kVW, w2 = t % Cfg::kVW;
 #pragma unroll
-                for (int t = 0; t < Cfg::kColTiles; ++t) {
-                    const int hh = t / Cfg::kVW, w2 = t % Cfg::kVW;
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const int col = hh * 128 + (lq * 4 + i) * Cfg::kVW + w2;
-                        float *dst = &o_stage[(r * 16 + ln) * D + col];
-                        const float v = o_acc[r][t][i] * fac[r];
-                        if (w == 0) *dst = v; else *dst += v;
-                    }
-                }
+            for (int i = 0; i < 4; ++i) {
+                const int col = hh * 128 + (lq * 4 + i) * Cfg::kVW + w2;
+                mine[ln * D + col] = o_acc[0][t][i] * fac[0];
+            }
         }
         __syncthreads();
+    } else {
+        for (int w = 0; w < NW; ++w) {
+            if (wave == w) {
+#pragma unroll
+                for (int r = 0; r < RT; ++r)
+#pragma unroll
+                    for (int t = 0; t < Cfg::kColTiles; ++t) {
+                        const int hh = t / Cfg::kVW, w2 = t % Cfg::kVW;
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            const int col = hh * 128 + (lq * 4 + i) * Cfg::kVW + w2;
+                            float *dst = &o_stage[(r * 16 + ln) * D + col];
+                            const float v = o_acc[r][t][i] * fac[r];
+                            if (w == 0) *dst = v; else *dst += v;
+                        }
+                    }
+            }
+            __syncthreads();
+        }
     }
 
     // ---- write: final output or split partial ------------------------------------------------
@@ -404,7 +427,14 @@ decode_paged_kernel(const DecodeParams p) {
         const float *src = &o_stage[row * D + piece * 8];
         float v[8];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] = src[e] * inv;
+        for (int e = 0; e < 8; ++e) {
+            float a = src[e];
+            if constexpr (kParallelMerge) {
+#pragma unroll
+                for (int w = 1; w < NW; ++w) a += src[w * (ROWS * D) + e];
+            }
+            v[e] = a * inv;
+        }
         const int qi = row / p.group;
         const int g = row - qi * p.group;
         const int head = kvh * p.group + g;
@@ -420,76 +450,264 @@ decode_paged_kernel(const DecodeParams p) {
             if (piece == 0)
                 p.lse[((int64_t)b * p.nheads + head) * Sq + qi] = (lg > 0.f) ? (mg + fast_log2(lg)) * kLn2 : INFINITY;
         } else {
-            const int64_t slot = (((int64_t)b * p.nheads_k + kvh) * p.nsplits + split) * p.rows + row;
-            float *dst = p.o_partial + slot * D + piece * 8;
+            const int64_t srow = slot * p.rows + row;
+            float *dst = p.o_partial + srow * D + piece * 8;
             *reinterpret_cast<float4 *>(dst) = make_float4(v[0], v[1], v[2], v[3]);
             *reinterpret_cast<float4 *>(dst + 4) = make_float4(v[4], v[5], v[6], v[7]);
-            if (piece == 0) p.lse_partial[slot] = (lg > 0.f) ? mg + fast_log2(lg) : -INFINITY;
+            if (piece == 0) p.lse_partial[srow] = (lg > 0.f) ? mg + fast_log2(lg) : -INFINITY;
+        }
+    }
+    __syncthreads();  // the LDS buffers may be reused by the next piece
+}
+
+// ---- grid mode: blockIdx = (split, kv head, batch row), fixed keys per split -------------------
+template <typename T, int D, int RT, int NW, bool SOFTCAP>
+__global__ void __launch_bounds__(NW * 64, (D <= 128 && RT <= 2) ? 2 : 1)
+decode_paged_kernel(const DecodeParams p) {
+    const int split = blockIdx.x;
+    const int kvh = blockIdx.y;
+    const int b = blockIdx.z;
+    const UnitRange ur = unit_range(p, b);
+    const bool empty = ur.nchunks == 0;
+    const int lo_al = ur.c0 * kChunk;
+    // splits this row really has; the grid was sized from shapes, so clamp and let the last split
+    // run to the end of the range if the caller's lengths exceed what the shapes promised
+    const int nsplits_row = empty ? 1 : min(p.nsplits, (ur.hi - lo_al + p.split_keys - 1) / p.split_keys);
+    if (split >= nsplits_row) return;
+    int range_lo = 0, range_hi = 0;
+    if (!empty) {
+        range_lo = max(ur.lo, lo_al + split * p.split_keys);
+        range_hi = (split == nsplits_row - 1) ? ur.hi : min(ur.hi, lo_al + (split + 1) * p.split_keys);
+    }
+    const int64_t slot = ((int64_t)b * p.nheads_k + kvh) * p.nsplits + split;
+    process_piece<T, D, RT, NW, SOFTCAP>(p, b, kvh, ur, range_lo, range_hi, nsplits_row == 1, slot);
+}
+
+// ---- balanced mode ---------------------------------------------------------------------------
+// The chunks of all (batch row, kv head) units, in (b, kvh) order, form one list of W chunks that
+// is cut into gridDim.x equal contiguous shares, one per workgroup, cutting inside a unit where a
+// share ends - the reference's flash-decode partition (flash_api.cpp:97-354, splitBN2S1GS2) done by
+// every workgroup for itself from the device-resident lengths.  A workgroup writes the final
+// output of every unit that lies wholly inside its share and at most two partials.
+
+// exclusive prefix of per-row chunk counts over 256 equal segments of the batch: s_pref[t] =
+// chunks of rows [0, t*seg); s_pref[256] = total.  All threads of a 256-thread block must call.
+__device__ __forceinline__ void batch_chunk_prefix(const DecodeParams &p, int *s_pref, int seg) {
+    __shared__ int s_wave[4];
+    const int tid = threadIdx.x;
+    int sum = 0;
+    for (int b = tid * seg; b < min(p.batch, (tid + 1) * seg); ++b) sum += unit_range(p, b).nchunks;
+    int inc = sum;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const int v = __shfl_up(inc, d, 64);
+        if ((tid & 63) >= d) inc += v;
+    }
+    if ((tid & 63) == 63) s_wave[tid >> 6] = inc;
+    __syncthreads();
+    int base = 0;
+    for (int w = 0; w < (tid >> 6); ++w) base += s_wave[w];
+    s_pref[tid + 1] = base + inc;
+    if (tid == 0) s_pref[0] = 0;
+    __syncthreads();
+}
+
+struct UnitPos {
+    int b;          // batch row
+    int pref;       // chunks of rows before b (one kv head's worth)
+};
+
+// batch row whose units contain list position `pos` (0 <= pos < Hk * total)
+__device__ __forceinline__ UnitPos locate_row(const DecodeParams &p, const int *s_pref, int seg, int64_t pos) {
+    const int target = (int)(pos / p.nheads_k);  // rows with pref <= target < pref + n
+    int lo = 0, hi = 256;                        // segment t with s_pref[t] <= target < s_pref[t+1]
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (s_pref[mid] <= target) lo = mid; else hi = mid;
+    }
+    UnitPos u;
+    u.b = lo * seg;
+    u.pref = s_pref[lo];
+    for (;;) {
+        const int n = unit_range(p, u.b).nchunks;
+        if (target < u.pref + n || u.b + 1 >= p.batch) break;
+        u.pref += n;
+        ++u.b;
+    }
+    return u;
+}
+
+template <typename T, int D, int RT, int NW, bool SOFTCAP>
+__global__ void __launch_bounds__(NW * 64, (D <= 128 && RT <= 2) ? 2 : 1)
+decode_balanced_kernel(const DecodeParams p) {
+    static_assert(NW == 4, "the batch scan assumes 256 threads");
+    __shared__ int s_pref[257];
+    const int seg = (p.batch + 255) / 256;
+    batch_chunk_prefix(p, s_pref, seg);
+    const int64_t W = (int64_t)s_pref[256] * p.nheads_k;
+    const int G = gridDim.x;
+    const int g = blockIdx.x;
+    const int64_t S = max((W + G - 1) / G, (int64_t)1);
+    int64_t pos = (int64_t)g * S;
+    const int64_t end = min(W, pos + S);
+    if (pos >= end) return;
+
+    UnitPos up = locate_row(p, s_pref, seg, pos);
+    UnitRange ur = unit_range(p, up.b);
+    int64_t row_start = (int64_t)up.pref * p.nheads_k;          // list position of unit (b, 0)
+    int kvh = (int)((pos - row_start) / ur.nchunks);
+    int offset = (int)((pos - row_start) - (int64_t)kvh * ur.nchunks);  // chunks into the unit
+    bool first = true;
+    while (pos < end) {
+        const int take = (int)min((int64_t)(ur.nchunks - offset), end - pos);
+        const bool whole = (offset == 0) && (take == ur.nchunks);
+        const int c_lo = ur.c0 + offset;
+        const int range_lo = max(ur.lo, c_lo * kChunk);
+        const int range_hi = min(ur.hi, (c_lo + take) * kChunk);
+        process_piece<T, D, RT, NW, SOFTCAP>(p, up.b, kvh, ur, range_lo, range_hi, whole,
+                                             (int64_t)g * 2 + (first ? 0 : 1));
+        first = false;
+        pos += take;
+        offset = 0;
+        if (++kvh == p.nheads_k) {
+            kvh = 0;
+            do {
+                ++up.b;
+                if (up.b >= p.batch) return;
+                ur = unit_range(p, up.b);
+            } while (ur.nchunks == 0);
         }
     }
 }
 
 // Split-KV combine (CombineScale.hpp:166-194,249-316): LSE = M + log sum exp(lse_s - M),
-// out = sum exp(lse_s - LSE) * O_s.  One workgroup per (batch row, kv head, query row).
-template <typename T, int D>
-__global__ void __launch_bounds__(D / 4) splitkv_combine_kernel(const DecodeParams p) {
+// out = sum exp(lse_s - LSE) * O_s.  One 256-thread workgroup per (query row, kv head, batch row):
+// D/4 column groups x (1024/D) piece lanes, reduced through LDS.
+template <typename T, int D, bool BALANCED>
+__global__ void __launch_bounds__(256) splitkv_combine_kernel(const DecodeParams p) {
+    constexpr int CG = D / 4;        // threads across the columns (4 columns each)
+    constexpr int NPL = 256 / CG;    // piece lanes
+    __shared__ int s_pref[257];
+    __shared__ float s_red[4];
+    __shared__ float s_tot[NPL];
+    __shared__ __attribute__((aligned(16))) float s_acc[NPL][D];
+
     const int row = blockIdx.x;
     const int kvh = blockIdx.y;
     const int b = blockIdx.z;
-    const int tid = threadIdx.x;  // owns 4 columns
-
-    const int Lk = p.cache_seqlens[b] + p.seqlen_new;
+    const int tid = threadIdx.x;
     const int Sq = p.seqlen_q;
-    const int off = Lk - Sq;
-    const int wr_eff = p.causal ? 0 : p.window_right;
-    int lo = 0, hi = Lk;
-    if (wr_eff >= 0) hi = min(Lk, Sq - 1 + off + wr_eff + 1);
-    if (p.window_left >= 0) lo = max(0, off - p.window_left);
-    const bool empty = (Lk <= 0) || (hi <= lo);
-    const int lo_al = lo & ~(kChunk - 1);
-    const int ns = empty ? 1 : min(p.nsplits, (hi - lo_al + p.split_keys - 1) / p.split_keys);
-    if (ns == 1) return;  // the decode kernel already wrote this row
+    const int qi = row / p.group;
+    const int head = kvh * p.group + (row - qi * p.group);
+    uint16_t *out_row = reinterpret_cast<uint16_t *>(p.out) + (int64_t)b * p.o_stride_b + (int64_t)qi * p.o_stride_s +
+                        (int64_t)head * p.o_stride_h;
+    float *lse_out = p.lse + ((int64_t)b * p.nheads + head) * Sq + qi;
 
-    const int64_t slot0 = (((int64_t)b * p.nheads_k + kvh) * p.nsplits) * p.rows + row;
+    const UnitRange ur = unit_range(p, b);
+    int ns;            // pieces of this unit
+    int64_t g_first = 0;
+    bool first_is_late = false;
+    if constexpr (BALANCED) {
+        const int seg = (p.batch + 255) / 256;
+        batch_chunk_prefix(p, s_pref, seg);
+        if (ur.nchunks == 0) {
+            // no visible key: no workgroup owned this unit
+            for (int c = tid; c < D; c += 256) out_row[c] = 0;
+            if (tid == 0) *lse_out = INFINITY;
+            return;
+        }
+        const int64_t W = (int64_t)s_pref[256] * p.nheads_k;
+        const int64_t S = max((W + p.num_wgs - 1) / p.num_wgs, (int64_t)1);
+        // chunks of rows before b
+        const int t = b / seg;
+        int pref = s_pref[t];
+        for (int bb = t * seg; bb < b; ++bb) pref += unit_range(p, bb).nchunks;
+        const int64_t start = (int64_t)pref * p.nheads_k + (int64_t)kvh * ur.nchunks;
+        const int64_t end = start + ur.nchunks;
+        g_first = start / S;
+        const int64_t g_last = (end - 1) / S;
+        ns = (int)(g_last - g_first + 1);
+        first_is_late = (start != g_first * S);
+    } else {
+        const int lo_al = ur.c0 * kChunk;
+        ns = (ur.nchunks == 0) ? 1 : min(p.nsplits, (ur.hi - lo_al + p.split_keys - 1) / p.split_keys);
+    }
+    if (ns == 1) return;  // the decode kernel already wrote this unit
+
+    auto slot_of = [&](int s) -> int64_t {
+        if constexpr (BALANCED)
+            return (g_first + s) * 2 + ((s == 0 && first_is_late) ? 1 : 0);
+        else
+            return ((int64_t)b * p.nheads_k + kvh) * p.nsplits + s;
+    };
+
+    // pass 1: maximum of the partial LSEs
     float mx = -INFINITY;
-    for (int s = 0; s < ns; ++s) mx = fmaxf(mx, p.lse_partial[slot0 + (int64_t)s * p.rows]);
+    for (int s2 = tid; s2 < ns; s2 += 256) mx = fmaxf(mx, p.lse_partial[slot_of(s2) * p.rows + row]);
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) mx = fmaxf(mx, __shfl_xor(mx, d, 64));
+    if ((tid & 63) == 0) s_red[tid >> 6] = mx;
+    __syncthreads();
+    mx = fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
     const float mx_use = (mx == -INFINITY) ? 0.f : mx;
+
+    // pass 2: weighted sum, piece lanes in parallel
+    const int cg = tid % CG;
+    const int pl = tid / CG;
     float tot = 0.f;
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
-    for (int s = 0; s < ns; ++s) {
-        const int64_t slot = slot0 + (int64_t)s * p.rows;
-        const float w = fast_exp2(p.lse_partial[slot] - mx_use);
+    for (int s2 = pl; s2 < ns; s2 += NPL) {
+        const int64_t srow = slot_of(s2) * p.rows + row;
+        const float w = fast_exp2(p.lse_partial[srow] - mx_use);
         tot += w;
-        const float4 o = *reinterpret_cast<const float4 *>(p.o_partial + slot * D + tid * 4);
+        const float4 o = *reinterpret_cast<const float4 *>(p.o_partial + srow * D + cg * 4);
         acc[0] += w * o.x;
         acc[1] += w * o.y;
         acc[2] += w * o.z;
         acc[3] += w * o.w;
     }
-    const float inv = (tot > 0.f) ? 1.f / tot : 0.f;
-    const int qi = row / p.group;
-    const int g = row - qi * p.group;
-    const int head = kvh * p.group + g;
-    uint2 o2;
-    o2.x = pack2<T>(acc[0] * inv, acc[1] * inv);
-    o2.y = pack2<T>(acc[2] * inv, acc[3] * inv);
-    uint16_t *dst = reinterpret_cast<uint16_t *>(p.out) + (int64_t)b * p.o_stride_b + (int64_t)qi * p.o_stride_s +
-                    (int64_t)head * p.o_stride_h + tid * 4;
-    *reinterpret_cast<uint2 *>(dst) = o2;
-    if (tid == 0)
-        p.lse[((int64_t)b * p.nheads + head) * Sq + qi] = (tot > 0.f) ? (mx + fast_log2(tot)) * kLn2 : INFINITY;
+    *reinterpret_cast<float4 *>(&s_acc[pl][cg * 4]) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+    if (cg == 0) s_tot[pl] = tot;
+    __syncthreads();
+    if (pl == 0) {
+        tot = 0.f;
+        acc[0] = acc[1] = acc[2] = acc[3] = 0.f;
+#pragma unroll
+        for (int l = 0; l < NPL; ++l) {
+            tot += s_tot[l];
+            const float4 o = *reinterpret_cast<const float4 *>(&s_acc[l][cg * 4]);
+            acc[0] += o.x;
+            acc[1] += o.y;
+            acc[2] += o.z;
+            acc[3] += o.w;
+        }
+        const float inv = (tot > 0.f) ? 1.f / tot : 0.f;
+        uint2 o2;
+        o2.x = pack2<T>(acc[0] * inv, acc[1] * inv);
+        o2.y = pack2<T>(acc[2] * inv, acc[3] * inv);
+        *reinterpret_cast<uint2 *>(out_row + cg * 4) = o2;
+        if (cg == 0) *lse_out = (tot > 0.f) ? (mx + fast_log2(tot)) * kLn2 : INFINITY;
+    }
 }
 
 template <typename T, int D, int RT>
 static hipError_t launch_decode_rt(const DecodeParams &p, hipStream_t stream) {
     constexpr int NW = 4;
-    dim3 grid(p.nsplits, p.nheads_k, p.batch);
     dim3 block(NW * 64);
     const bool softcap = p.softcap_post != 0.f;
-    if (softcap)
-        hipLaunchKernelGGL((decode_paged_kernel<T, D, RT, NW, true>), grid, block, 0, stream, p);
-    else
-        hipLaunchKernelGGL((decode_paged_kernel<T, D, RT, NW, false>), grid, block, 0, stream, p);
+    if (p.balanced) {
+        dim3 grid(p.num_wgs);
+        if (softcap)
+            hipLaunchKernelGGL((decode_balanced_kernel<T, D, RT, NW, true>), grid, block, 0, stream, p);
+        else
+            hipLaunchKernelGGL((decode_balanced_kernel<T, D, RT, NW, false>), grid, block, 0, stream, p);
+    } else {
+        dim3 grid(p.nsplits, p.nheads_k, p.batch);
+        if (softcap)
+            hipLaunchKernelGGL((decode_paged_kernel<T, D, RT, NW, true>), grid, block, 0, stream, p);
+        else
+            hipLaunchKernelGGL((decode_paged_kernel<T, D, RT, NW, false>), grid, block, 0, stream, p);
+    }
     return hipGetLastError();
 }
 
@@ -513,13 +731,22 @@ hipError_t launch_decode_paged(const DecodeParams &p, int dtype, int headdim, hi
     return dtype == 0 ? launch_decode_t<BF16>(p, headdim, stream) : launch_decode_t<FP16>(p, headdim, stream);
 }
 
-template <typename T> static hipError_t launch_combine_t(const DecodeParams &p, int headdim_v, hipStream_t stream) {
+int decode_wgs_per_cu(int headdim, int rows) { return (headdim <= 128 && rows <= 32) ? 2 : 1; }
+
+template <typename T, int D> static void launch_combine_d(const DecodeParams &p, hipStream_t stream) {
     dim3 grid(p.rows, p.nheads_k, p.batch);
+    if (p.balanced)
+        hipLaunchKernelGGL((splitkv_combine_kernel<T, D, true>), grid, dim3(256), 0, stream, p);
+    else
+        hipLaunchKernelGGL((splitkv_combine_kernel<T, D, false>), grid, dim3(256), 0, stream, p);
+}
+
+template <typename T> static hipError_t launch_combine_t(const DecodeParams &p, int headdim_v, hipStream_t stream) {
     switch (headdim_v) {
-        case 64: hipLaunchKernelGGL((splitkv_combine_kernel<T, 64>), grid, dim3(16), 0, stream, p); break;
-        case 128: hipLaunchKernelGGL((splitkv_combine_kernel<T, 128>), grid, dim3(32), 0, stream, p); break;
-        case 256: hipLaunchKernelGGL((splitkv_combine_kernel<T, 256>), grid, dim3(64), 0, stream, p); break;
-        case 512: hipLaunchKernelGGL((splitkv_combine_kernel<T, 512>), grid, dim3(128), 0, stream, p); break;
+        case 64: launch_combine_d<T, 64>(p, stream); break;
+        case 128: launch_combine_d<T, 128>(p, stream); break;
+        case 256: launch_combine_d<T, 256>(p, stream); break;
+        case 512: launch_combine_d<T, 512>(p, stream); break;
         default: return hipErrorInvalidValue;
     }
     return hipGetLastError();

@@ -36,7 +36,8 @@ struct DecodeParams {
     float softcap_pre;     // softmax_scale / softcap            (softcap on)
     float softcap_post;    // softcap * log2(e)
     int32_t causal, window_left, window_right;
-    int32_t nsplits, split_keys;
+    int32_t nsplits, split_keys;   // grid mode: split slots per unit, keys per split
+    int32_t balanced, num_wgs;     // balanced mode: workgroups sharing the chunk list equally
 };
 
 struct AppendParams {
@@ -91,6 +92,9 @@ hipError_t launch_decode_paged(const DecodeParams &p, int dtype, int headdim, hi
 hipError_t launch_splitkv_combine(const DecodeParams &p, int dtype, int headdim_v, hipStream_t stream);
 hipError_t launch_decode_mla_i8(const DecodeParams &p, int dtype, hipStream_t stream);
 hipError_t launch_prefill(const PrefillParams &p, int dtype, int headdim, hipStream_t stream);
+
+// Resident decode workgroups per compute unit for a head dimension / query-block height.
+int decode_wgs_per_cu(int headdim, int rows);
 
 // Largest query block (seqlen_q * group) the decode kernel packs into one workgroup.
 constexpr int kDecodeMaxRows = 64;

@@ -10,6 +10,7 @@
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 
 #include "../../include/fa_rocm.h"
@@ -123,46 +124,52 @@ int fa_rocm_kvcache_validate(const fa_kvcache_args *a) {
     return FA_OK;
 }
 
-int fa_rocm_choose_splits(const fa_kvcache_args *a, int num_cus, int32_t *split_keys) {
-    if (!a) return fail(FA_ERR_NULL, "args is NULL");
+int fa_rocm_plan_kvcache(const fa_kvcache_args *a, int num_cus, fa_split_plan *plan) {
+    if (!a || !plan) return fail(FA_ERR_NULL, "args or plan is NULL");
     if (num_cus <= 0) num_cus = 256;
+    std::memset(plan, 0, sizeof(*plan));
+    const int group = a->nheads / (a->nheads_k > 0 ? a->nheads_k : 1);
+    const size_t rows = (size_t)a->seqlen_q * group;
+    const size_t slot_bytes = rows * ((size_t)a->headdim_v + 1) * sizeof(float);
+    if (a->num_splits == 0) {
+        plan->mode = FA_SPLIT_BALANCED;
+        plan->nsplits = 1;
+        const int per_cu = is_mla_i8(a) ? 1 : fa::decode_wgs_per_cu(a->headdim_qk, (int)rows);
+        plan->num_wgs = num_cus * per_cu;
+        // tuning aid: FA_ROCM_DECODE_WGS overrides the workgroup count of the balanced partition
+        if (const char *env = std::getenv("FA_ROCM_DECODE_WGS")) {
+            const int v = std::atoi(env);
+            if (v > 0) plan->num_wgs = v;
+        }
+        // every workgroup writes at most two partials (the units cut at the two ends of its share)
+        plan->workspace_bytes = (size_t)plan->num_wgs * 2 * slot_bytes;
+        return FA_OK;
+    }
     const int64_t bound = live_keys_bound(a);
     const int64_t granule = 256;
     int64_t sk;
     if (a->num_splits == 1) {
         sk = (bound + granule - 1) / granule * granule;
-    } else if (a->num_splits > 1) {
+    } else {
         // forced mode (flash_attn_npu_3/fa_split.h:345-350): blocks per split = ceil(nblk / num_splits)
         const int64_t nblk = (bound + granule - 1) / granule;
         const int64_t per = (nblk + a->num_splits - 1) / a->num_splits;
         sk = per * granule;
-    } else {
-        // heuristic: enough workgroups to give every CU several, but at least 1024 keys per split
-        // so that the per-split prologue/merge stays small next to the stream
-        const int64_t units = (int64_t)a->batch * a->nheads_k;
-        const int64_t target_wgs = (int64_t)num_cus * 8;
-        int64_t want = (target_wgs + units - 1) / units;  // splits per unit
-        if (want < 1) want = 1;
-        sk = (bound + want - 1) / want;
-        sk = (sk + granule - 1) / granule * granule;
-        if (sk < 1024) sk = 1024;
     }
     if (sk > (1 << 30)) sk = 1 << 30;
     int64_t n = (bound + sk - 1) / sk;
     if (n < 1) n = 1;
-    if (split_keys) *split_keys = (int32_t)sk;
-    return (int)n;
+    plan->mode = FA_SPLIT_GRID;
+    plan->nsplits = (int32_t)n;
+    plan->split_keys = (int32_t)sk;
+    plan->workspace_bytes = n > 1 ? (size_t)a->batch * a->nheads_k * n * slot_bytes : 0;
+    return FA_OK;
 }
 
 size_t fa_rocm_kvcache_workspace_bytes(const fa_kvcache_args *a, int num_cus) {
-    if (!a) return 0;
-    int32_t sk = 0;
-    const int n = fa_rocm_choose_splits(a, num_cus, &sk);
-    if (n <= 1) return 0;
-    const int group = a->nheads / (a->nheads_k > 0 ? a->nheads_k : 1);
-    const size_t rows = (size_t)a->seqlen_q * group;
-    const size_t slots = (size_t)a->batch * a->nheads_k * n * rows;
-    return slots * ((size_t)a->headdim_v + 1) * sizeof(float);
+    fa_split_plan plan;
+    if (fa_rocm_plan_kvcache(a, num_cus, &plan) != FA_OK) return 0;
+    return plan.workspace_bytes;
 }
 
 static void fill_append(const fa_kvcache_args *a, fa::AppendParams &p) {
@@ -296,9 +303,10 @@ static int fwd_kvcache_impl(const fa_kvcache_args *a, void *stream_, void *const
 
     int cus = device_cus();
     if (cus <= 0) cus = 256;
-    int32_t split_keys = 0;
-    const int nsplits = fa_rocm_choose_splits(a, cus, &split_keys);
-    const size_t need = fa_rocm_kvcache_workspace_bytes(a, cus);
+    fa_split_plan plan;
+    rc = fa_rocm_plan_kvcache(a, cus, &plan);
+    if (rc != FA_OK) return rc;
+    const size_t need = plan.workspace_bytes;
     if (need > 0 && (!a->workspace || a->workspace_bytes < need))
         return fail(FA_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", need, a->workspace ? a->workspace_bytes : (size_t)0);
 
@@ -352,10 +360,13 @@ static int fwd_kvcache_impl(const fa_kvcache_args *a, void *stream_, void *const
     p.causal = a->causal;
     p.window_left = a->window_left;
     p.window_right = a->window_right;
-    p.nsplits = nsplits;
-    p.split_keys = split_keys;
-    if (nsplits > 1) {
-        const size_t slots = (size_t)a->batch * a->nheads_k * nsplits * rows;
+    p.nsplits = plan.nsplits;
+    p.split_keys = plan.split_keys > 0 ? plan.split_keys : 256;
+    p.balanced = plan.mode == FA_SPLIT_BALANCED;
+    p.num_wgs = plan.num_wgs;
+    const bool needs_combine = need > 0;
+    if (needs_combine) {
+        const size_t slots = need / (((size_t)a->headdim_v + 1) * sizeof(float));   // slot rows
         p.o_partial = static_cast<float *>(a->workspace);
         p.lse_partial = p.o_partial + slots * a->headdim_v;
     }
@@ -367,7 +378,7 @@ static int fwd_kvcache_impl(const fa_kvcache_args *a, void *stream_, void *const
         e = fa::launch_decode_paged(p, a->io_dtype, a->headdim_qk, stream);
     if (e != hipSuccess) return fail(FA_ERR_LAUNCH, "decode launch failed: %s", hipGetErrorString(e));
     mark(2);
-    if (nsplits > 1) {
+    if (needs_combine) {
         e = fa::launch_splitkv_combine(p, a->io_dtype, a->headdim_v, stream);
         if (e != hipSuccess) return fail(FA_ERR_LAUNCH, "combine launch failed: %s", hipGetErrorString(e));
     }

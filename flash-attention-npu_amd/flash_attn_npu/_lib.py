@@ -48,13 +48,18 @@ class VarlenArgs(C.Structure):
     )
 
 
+class SplitPlan(C.Structure):
+    """Mirror of struct fa_split_plan (include/fa_rocm.h)."""
+    _fields_ = [("mode", _i32), ("nsplits", _i32), ("split_keys", _i32), ("num_wgs", _i32), ("workspace_bytes", _sz)]
+
+
 EXPORTS = {
     "fa_rocm_abi_version": (C.c_int, []),
     "fa_rocm_last_error": (C.c_char_p, []),
     "fa_rocm_sizeof_kvcache_args": (_sz, []),
     "fa_rocm_sizeof_varlen_args": (_sz, []),
     "fa_rocm_num_cus": (C.c_int, []),
-    "fa_rocm_choose_splits": (C.c_int, [C.POINTER(KvcacheArgs), C.c_int, C.POINTER(_i32)]),
+    "fa_rocm_plan_kvcache": (C.c_int, [C.POINTER(KvcacheArgs), C.c_int, C.POINTER(SplitPlan)]),
     "fa_rocm_kvcache_workspace_bytes": (_sz, [C.POINTER(KvcacheArgs), C.c_int]),
     "fa_rocm_kvcache_validate": (C.c_int, [C.POINTER(KvcacheArgs)]),
     "fa_rocm_varlen_validate": (C.c_int, [C.POINTER(VarlenArgs)]),

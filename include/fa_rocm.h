@@ -132,15 +132,28 @@ size_t fa_rocm_sizeof_varlen_args(void);
 int fa_rocm_num_cus(void);
 
 /*
- * Split-KV decision.  Stands in for the reference's flash-decode heuristic and
- * partition (csrc/ascend910/flash_attn_npu/flash_api.cpp:525-550, splitBN2S1GS2 :343-354;
- * forced mode csrc/ascend910/flash_attn_npu_3/fa_split.h:345-350).  Pure host integer code:
- * needs no GPU.  Writes the keys-per-split granule (a multiple of 256) to *split_keys and
- * returns the number of split slots per (batch row, kv head), >= 1.  `num_cus` <= 0 means 256.
+ * Split-KV plan of a kvcache call, decided from shapes alone (per-row lengths stay on the device).
+ * Stands in for the reference's flash-decode heuristic and partition
+ * (csrc/ascend910/flash_attn_npu/flash_api.cpp:525-550, splitBN2S1GS2 :343-354; forced mode
+ * csrc/ascend910/flash_attn_npu_3/fa_split.h:345-350).
+ *   mode FA_SPLIT_BALANCED (num_splits == 0): `num_wgs` workgroups share the list of all 32-key
+ *     chunks of all (batch row, kv head) units equally, cutting inside a unit where a share ends;
+ *     the shares are computed on the device from cache_seqlens.
+ *   mode FA_SPLIT_GRID (num_splits >= 1): every unit is cut into at most `nsplits` ranges of
+ *     `split_keys` keys (a multiple of 256); num_splits == 1 gives nsplits == 1 (no split).
+ * Pure host integer code: needs no GPU.  `num_cus` <= 0 means 256.
  */
-int fa_rocm_choose_splits(const fa_kvcache_args *args, int num_cus, int32_t *split_keys);
+enum fa_split_mode { FA_SPLIT_GRID = 0, FA_SPLIT_BALANCED = 1 };
+typedef struct fa_split_plan {
+    int32_t mode;
+    int32_t nsplits;          /* grid mode: split slots per unit (>= 1)          */
+    int32_t split_keys;       /* grid mode: keys per split                       */
+    int32_t num_wgs;          /* balanced mode: workgroups launched              */
+    size_t workspace_bytes;   /* fp32 partial outputs + LSEs the call needs      */
+} fa_split_plan;
+int fa_rocm_plan_kvcache(const fa_kvcache_args *args, int num_cus, fa_split_plan *plan);
 
-/* Bytes of workspace the kvcache call needs for the split partials (0 when unsplit). */
+/* Bytes of workspace the kvcache call needs (plan.workspace_bytes; 0 when nothing is split). */
 size_t fa_rocm_kvcache_workspace_bytes(const fa_kvcache_args *args, int num_cus);
 
 /*
