@@ -247,6 +247,94 @@ def run_decode(args, name):
     return out
 
 
+def prefill_workload(device, seed: int = 0):
+    """BASELINE.json configs[4]: 16 sequences, lengths uniform in [512, 4096] rescaled to a total of
+    32768 tokens (largest remainder), 32 q heads / 8 kv heads, d = 128, bf16, causal."""
+    import torch
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    raw = torch.randint(512, 4097, (16,), generator=g).double()
+    scaled = raw * (32768.0 / raw.sum())
+    lens = scaled.floor().long()
+    rem = 32768 - int(lens.sum())
+    order = torch.argsort(scaled - lens.double(), descending=True)
+    lens[order[:rem]] += 1
+    cu = torch.zeros(17, dtype=torch.int32)
+    cu[1:] = lens.cumsum(0).to(torch.int32)
+    gd = torch.Generator(device=device).manual_seed(seed + 1)
+
+    def rn(*shape):
+        return torch.randn(*shape, generator=gd, device=device, dtype=torch.float32).to(torch.bfloat16)
+
+    return dict(lens=lens, cu=cu.to(device), q=rn(32768, 32, 128), k=rn(32768, 8, 128), v=rn(32768, 8, 128),
+                max_len=int(lens.max()), hq=32, hk=8, d=128)
+
+
+def run_prefill(args):
+    import torch
+    from flash_attn_npu import flash_attn_npu as ops
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    w = prefill_workload(dev)
+    scale = w["d"] ** -0.5
+    flops = sum(4.0 * int(l) * int(l) * w["d"] * w["hq"] / 2.0 for l in w["lens"])
+    out = torch.empty_like(w["q"])
+
+    def step():
+        return ops.varlen_fwd(w["q"], w["k"], w["v"], out, w["cu"], w["cu"], None, None, None, None, w["max_len"],
+                              w["max_len"], 0.0, scale, False, True, -1, -1, 0.0, False, None)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) / args.steps * 1e3
+    # kernel duration: one kernel per call, bracketed by events on the launch stream
+    ev = HipEvents(2 * args.steps)
+    stream = C.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+    for i in range(args.steps):
+        ev.record(2 * i, stream)
+        step()
+        ev.record(2 * i + 1, stream)
+    torch.cuda.synchronize()
+    kern_ms = sum(ev.elapsed_ms(2 * i, 2 * i + 1) for i in range(args.steps)) / args.steps
+    ev.close()
+    achieved = flops / (kern_ms * 1e-3) / 1e12
+    res = {
+        "metric": "varlen_prefill_fwd_tflops", "value": flops / (ms_per_step * 1e-3) / 1e12, "unit": "TFLOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "c5: varlen prefill forward bf16, 16 sequences (lengths U[512,4096] rescaled to 32768 "
+                               "tokens), 32q/8kv heads, d=128, causal", "seq_lens": [int(x) for x in w["lens"]],
+                   "flop_count": "sum 4*S^2*d*Hq / 2"},
+        "us_per_call": ms_per_step * 1e3, "algorithmic_flops": flops,
+        "pct_of_mfma_peak": 100.0 * flops / (ms_per_step * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
+        "roofline": {"bound": "mfma", "kernel": "prefill_kernel", "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS,
+                     "unit": "TFLOP/s", "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
+                     "kernel_us": kern_ms * 1e3},
+    }
+    if not args.no_cpu:
+        import fa_oracle as O
+        q, k, v, cu = w["q"].cpu(), w["k"].cpu(), w["v"].cpu(), w["cu"].cpu()
+        done_flops, secs, n = 0.0, 0.0, 0
+        for b in range(16):
+            a, e = int(cu[b]), int(cu[b + 1])
+            c1 = torch.tensor([0, e - a], dtype=torch.int32)
+            t1 = time.perf_counter()
+            O.flash_attn_varlen(q[a:e], k[a:e], v[a:e], c1, c1, e - a, e - a, softmax_scale=scale, causal=True, mode="golden")
+            secs += time.perf_counter() - t1
+            done_flops += 4.0 * (e - a) * (e - a) * w["d"] * w["hq"] / 2.0
+            n += 1
+            if secs > 20.0:
+                break
+        res["cpu_baseline"] = dict(value=done_flops / secs / 1e12, unit="TFLOP/s", cores=torch.get_num_threads(), kind="port",
+                                   sample=f"oracle blocked golden on the first {n} of 16 sequences, {secs:.2f} s on "
+                                          f"{os.cpu_count()} host cpus, torch threads {torch.get_num_threads()}")
+    return res
+
+
 def run_copy(args):
     """Plain device copy of known size (1 GiB read + 1 GiB written per step): the calibration
     workload for the FETCH_SIZE / WRITE_SIZE counters and a practical bandwidth yardstick."""
@@ -287,6 +375,8 @@ def main():
         sys.exit(2)
     if args.config in ("c2", "c2_8k", "c3a", "c3b"):
         out = run_decode(args, args.config)
+    elif args.config == "c5":
+        out = run_prefill(args)
     elif args.config == "copy":
         out = run_copy(args)
     else:

@@ -403,6 +403,8 @@ int fa_rocm_varlen_validate(const fa_varlen_args *a) {
     if (a->max_seqlen_q <= 0) return fail(FA_ERR_SHAPE, "max_seqlen_q must be positive");
     if (a->block_table && (a->page_size <= 0 || a->page_size % 32 != 0))
         return fail(FA_ERR_SHAPE, "page_block_size must be a positive multiple of 32");
+    if (a->block_table && (a->num_blocks <= 0 || a->max_blocks_per_seq <= 0))
+        return fail(FA_ERR_SHAPE, "empty block_table or cache");
     if (a->q_stride_t % 8 || a->q_stride_h % 8 || a->k_stride_t % 8 || a->k_stride_h % 8 || a->v_stride_t % 8 ||
         a->v_stride_h % 8 || a->o_stride_t % 8 || a->o_stride_h % 8)
         return fail(FA_ERR_SHAPE, "tensor strides must be multiples of 8 elements (16 bytes)");
@@ -431,6 +433,7 @@ int fa_rocm_varlen_fwd(const fa_varlen_args *a, void *stream_) {
     pp.total_q = a->total_q;
     pp.page_size = a->page_size;
     pp.max_blocks = a->max_blocks_per_seq;
+    pp.num_blocks = a->num_blocks;
     pp.q_stride_t = a->q_stride_t;
     pp.q_stride_h = a->q_stride_h;
     pp.o_stride_t = a->o_stride_t;

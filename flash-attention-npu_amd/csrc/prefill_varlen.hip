@@ -1,5 +1,342 @@
+// Tiled attention forward on the bf16/fp16 MFMA for gfx950: variable-length (token-major) prefill
+// over dense or paged K/V, and kvcache calls whose query block is too tall for the decode kernel.
+//
+// Stands in for the reference's FAInfer kernel in TND layout (csrc/ascend910/flash_attn_npu/
+// mha_fwd_kvcache.cpp:436-970 with per-sequence offsets :469-475,505-507; host mha_varlen_fwd,
+// flash_api.cpp:848-1089).  Where the reference ping-pongs S, P and O_tmp between its matrix and
+// vector cores through global memory, everything between the K/V tile loads and the final store
+// stays in registers here:
+//   * one workgroup = 128 query rows of one (sequence, q head); 4 waves x 32 rows;
+//   * K/V tiles of 64 keys are fetched once per workgroup with 16-byte coalesced loads and
+//     double-buffered in LDS (K rows XOR-swizzled so MFMA operand reads are conflict free);
+//   * S^T = K Q^T and O^T = V^T P^T on the 32x32x16 MFMA: a query row is one lane column in both
+//     products, so the running max / sum / rescale never leave the lane (one xor-32 exchange);
+//   * V operands are read as whole rows and transposed in registers with v_perm;
+//   * key tiles outside the causal / window range of the 128-row block are never loaded.
 #include "fa_device.h"
 #include "fa_kernels.h"
+
 namespace fa {
-hipError_t launch_prefill(const PrefillParams &, int, int, hipStream_t) { return hipErrorNotSupported; }
+
+constexpr int kBM = 128;  // query rows per workgroup
+constexpr int kBN = 64;   // keys per tile
+
+template <int D> struct PrefillCfg {
+    static constexpr int kKSteps = D / 16;        // MFMA k-steps of QK^T
+    static constexpr int kMT = D / 32;            // 32-column tiles of O^T
+    static constexpr int kCPL = D / 32;           // V columns a lane owns per key row
+    static constexpr int kChunks = D / 8;         // 16-byte pieces per row
+    static constexpr int kSwz = (kChunks >= 16) ? 15 : kChunks - 1;
+    static constexpr int kTileBytes = kBN * D * 2;
+    static constexpr int kPieces = kBN * kChunks / 256;  // 16-byte pieces per thread per tile
+};
+
+template <typename T, int D, bool PAGED, bool SOFTCAP>
+__global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) prefill_kernel(const PrefillParams p) {
+    using Cfg = PrefillCfg<D>;
+    __shared__ __attribute__((aligned(16))) uint8_t s_k[2][Cfg::kTileBytes];
+    __shared__ __attribute__((aligned(16))) uint8_t s_v[2][Cfg::kTileBytes];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lh = lane >> 5;   // half: MFMA k-slot
+    const int ln = lane & 31;   // MFMA row / column
+
+    const int mb = gridDim.x - 1 - blockIdx.x;  // tall causal blocks first
+    const int h = blockIdx.y;
+    const int b = blockIdx.z;
+    const int hk = h / p.group;
+
+    int q0, Sq, k0 = 0, Sk;
+    if (p.cu_seqlens_q) {
+        q0 = p.cu_seqlens_q[b];
+        Sq = p.cu_seqlens_q[b + 1] - q0;
+    } else {
+        q0 = 0;
+        Sq = p.seqlen_q_fixed;
+    }
+    if constexpr (PAGED) {
+        Sk = p.seqused_k[b] + p.seqlen_k_add;
+        Sk = min(Sk, p.max_blocks * p.page_size);
+    } else {
+        k0 = p.cu_seqlens_k[b];
+        Sk = p.cu_seqlens_k[b + 1] - k0;
+    }
+    if (mb * kBM >= Sq) return;
+    const int off = Sk - Sq;
+    const int wr_eff = p.causal ? 0 : p.window_right;
+    const int wl = p.window_left;
+
+    const uint16_t *qb = reinterpret_cast<const uint16_t *>(p.q) + (int64_t)b * p.q_stride_b + (int64_t)h * p.q_stride_h;
+    uint16_t *ob = reinterpret_cast<uint16_t *>(p.out) + (int64_t)b * p.o_stride_b + (int64_t)h * p.o_stride_h;
+    float *lse_b = p.lse + (int64_t)b * p.lse_stride_b + (int64_t)h * p.lse_stride_h;
+
+    // key range the whole 128-row block can see
+    const int r_lo = mb * kBM;
+    const int r_hi = min(Sq, r_lo + kBM) - 1;
+    int k_lo = 0, k_hi = Sk;
+    if (wl >= 0) k_lo = max(0, r_lo + off - wl);
+    if (wr_eff >= 0) k_hi = min(Sk, r_hi + off + wr_eff + 1);
+    k_hi = max(k_hi, 0);
+
+    const int my_row = r_lo + wave * 32 + ln;   // query row of this lane column
+    const bool row_ok = my_row < Sq;
+
+    if (k_hi <= k_lo) {
+        // nothing visible for the whole block: out = 0, lse = +inf
+        if (row_ok) {
+            uint16_t *dst = ob + (int64_t)(q0 + my_row) * p.o_stride_t;
+            for (int c = lh * (D / 2); c < (lh + 1) * (D / 2); c += 8) store16(dst + c, u32x4_t{0, 0, 0, 0});
+            if (lh == 0) lse_b[q0 + my_row] = INFINITY;
+        }
+        return;
+    }
+
+    // per-lane visible interval of its row (inclusive bounds)
+    int klo_r = 0, khi_r = Sk - 1;
+    if (wl >= 0) klo_r = max(0, my_row + off - wl);
+    if (wr_eff >= 0) khi_r = min(Sk - 1, my_row + off + wr_eff);
+    // bounds that decide, per wave, whether a tile needs element masks
+    const int rw0 = r_lo + wave * 32;
+    const int rw1 = min(Sq - 1, rw0 + 31);
+    const int wave_klo_max = (wl >= 0) ? max(0, rw1 + off - wl) : 0;
+    const int wave_khi_min = (wr_eff >= 0) ? min(Sk - 1, rw0 + off + wr_eff) : Sk - 1;
+
+    // Q^T operand: lane (lh, ln) holds row ln, elements t*16 + lh*8 .. +7
+    u32x4_t qreg[Cfg::kKSteps];
+    {
+        const uint16_t *src = qb + (int64_t)(q0 + min(my_row, Sq - 1)) * p.q_stride_t + lh * 8;
+#pragma unroll
+        for (int t = 0; t < Cfg::kKSteps; ++t) {
+            qreg[t] = load16(src + t * 16);
+            if (!row_ok) qreg[t] = u32x4_t{0, 0, 0, 0};
+        }
+    }
+
+    // ---- K/V tile fetch: 256 threads x kPieces 16-byte pieces each --------------------------
+    const uint16_t *kbase = reinterpret_cast<const uint16_t *>(p.k) + (int64_t)hk * p.k_stride_h;
+    const uint16_t *vbase = reinterpret_cast<const uint16_t *>(p.v) + (int64_t)hk * p.v_stride_h;
+    const int32_t *bt_row = PAGED ? p.block_table + (int64_t)b * p.bt_stride_b : nullptr;
+
+    u32x4_t kst[Cfg::kPieces], vst[Cfg::kPieces];
+    auto fetch_tile = [&](int kt) {
+#pragma unroll
+        for (int i = 0; i < Cfg::kPieces; ++i) {
+            const int piece = tid + 256 * i;
+            const int row = piece / Cfg::kChunks;
+            const int ch = piece % Cfg::kChunks;
+            const int key = min(kt * kBN + row, Sk - 1);
+            int64_t koff, voff;
+            if constexpr (PAGED) {
+                const int page = key / p.page_size;
+                int blk = bt_row[page];
+                blk = min(max(blk, 0), p.num_blocks - 1);
+                const int inpage = key - page * p.page_size;
+                koff = (int64_t)blk * p.k_stride_block + (int64_t)inpage * p.k_stride_t;
+                voff = (int64_t)blk * p.v_stride_block + (int64_t)inpage * p.v_stride_t;
+            } else {
+                koff = (int64_t)(k0 + key) * p.k_stride_t;
+                voff = (int64_t)(k0 + key) * p.v_stride_t;
+            }
+            kst[i] = load16(kbase + koff + ch * 8);
+            vst[i] = load16(vbase + voff + ch * 8);
+        }
+    };
+    auto stash_tile = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < Cfg::kPieces; ++i) {
+            const int piece = tid + 256 * i;
+            const int row = piece / Cfg::kChunks;
+            const int ch = piece % Cfg::kChunks;
+            *reinterpret_cast<u32x4_t *>(&s_k[buf][row * (D * 2) + ((ch ^ (row & Cfg::kSwz)) << 4)]) = kst[i];
+            *reinterpret_cast<u32x4_t *>(&s_v[buf][row * (D * 2) + (ch << 4)]) = vst[i];
+        }
+    };
+
+    float m_run = -INFINITY, l_run = 0.f;
+    float16_t o_acc[Cfg::kMT];
+#pragma unroll
+    for (int t = 0; t < Cfg::kMT; ++t)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o_acc[t][r] = 0.f;
+
+    const int kt_begin = k_lo / kBN;
+    const int kt_end = (k_hi + kBN - 1) / kBN;
+    fetch_tile(kt_begin);
+    stash_tile(0);
+    __syncthreads();
+
+    int cur = 0;
+    for (int kt = kt_begin; kt < kt_end; ++kt) {
+        const bool more = kt + 1 < kt_end;
+        if (more) fetch_tile(kt + 1);
+        __builtin_amdgcn_sched_barrier(0);
+
+        // ---- S^T = K Q^T for the two 32-key halves of the tile
+        float16_t s[2];
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s[tt][r] = 0.f;
+#pragma unroll
+        for (int t = 0; t < Cfg::kKSteps; ++t)
+#pragma unroll
+            for (int tt = 0; tt < 2; ++tt) {
+                const int row = tt * 32 + ln;
+                const u32x4_t a = *reinterpret_cast<const u32x4_t *>(
+                    &s_k[cur][row * (D * 2) + (((t * 2 + lh) ^ (row & Cfg::kSwz)) << 4)]);
+                s[tt] = mfma32<T>(a, qreg[t], s[tt]);
+            }
+
+        // ---- online softmax; lane column = query row, register r of half tt = key
+        //      kt*64 + tt*32 + 8*(r/4) + 4*lh + r%4
+        const int tile0 = kt * kBN;
+        const bool need_mask = (tile0 < wave_klo_max) || (tile0 + kBN - 1 > wave_khi_min);
+        float mloc = -INFINITY;
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                float v = s[tt][r];
+                if constexpr (SOFTCAP) {
+                    const float y = v * p.softcap_pre;
+                    const float e2 = __expf(2.f * y);
+                    v = p.softcap_post * (1.f - 2.f / (e2 + 1.f));
+                } else {
+                    v *= p.scale_log2;
+                }
+                if (need_mask) {
+                    const int key = tile0 + tt * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
+                    v = (key >= klo_r && key <= khi_r) ? v : -INFINITY;
+                }
+                s[tt][r] = v;
+                mloc = fmaxf(mloc, v);
+            }
+        mloc = fmaxf(mloc, xor_shuffle(mloc, 32));
+        const float m_new = fmaxf(m_run, mloc);
+        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+        const float alpha = fast_exp2(m_run - m_use);
+        m_run = m_new;
+        float psum = 0.f;
+        u32x4_t pk[2][2];
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                s[tt][r] = fast_exp2(s[tt][r] - m_use);
+                psum += s[tt][r];
+            }
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+                for (int u = 0; u < 4; ++u) pk[tt][ks][u] = pack2<T>(s[tt][8 * ks + 2 * u], s[tt][8 * ks + 2 * u + 1]);
+        }
+        l_run = l_run * alpha + psum;
+#pragma unroll
+        for (int t = 0; t < Cfg::kMT; ++t)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) o_acc[t][r] *= alpha;
+
+        // ---- O^T += V^T P^T, 16 keys per step; V rows read whole and transposed in registers
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) {
+                uint32_t vr[8][Cfg::kCPL / 2 > 0 ? Cfg::kCPL / 2 : 1];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const int row = tt * 32 + 16 * ks + 8 * (e >> 2) + 4 * lh + (e & 3);
+                    const uint8_t *src = &s_v[cur][row * (D * 2) + ln * (Cfg::kCPL * 2)];
+                    if constexpr (Cfg::kCPL == 8) {
+                        const u32x4_t t4 = *reinterpret_cast<const u32x4_t *>(src);
+                        vr[e][0] = t4[0]; vr[e][1] = t4[1]; vr[e][2] = t4[2]; vr[e][3] = t4[3];
+                    } else if constexpr (Cfg::kCPL == 4) {
+                        const uint2 t2 = *reinterpret_cast<const uint2 *>(src);
+                        vr[e][0] = t2.x; vr[e][1] = t2.y;
+                    } else {
+                        vr[e][0] = *reinterpret_cast<const uint32_t *>(src);
+                    }
+                }
+#pragma unroll
+                for (int w2 = 0; w2 < Cfg::kCPL / 2; ++w2) {
+                    u32x4_t a_lo, a_hi;
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        a_lo[u] = __builtin_amdgcn_perm(vr[2 * u + 1][w2], vr[2 * u][w2], 0x05040100u);
+                        a_hi[u] = __builtin_amdgcn_perm(vr[2 * u + 1][w2], vr[2 * u][w2], 0x07060302u);
+                    }
+                    o_acc[2 * w2] = mfma32<T>(a_lo, pk[tt][ks], o_acc[2 * w2]);
+                    o_acc[2 * w2 + 1] = mfma32<T>(a_hi, pk[tt][ks], o_acc[2 * w2 + 1]);
+                }
+            }
+
+        if (more) stash_tile(cur ^ 1);
+        __syncthreads();
+        cur ^= 1;
+    }
+
+    // ---- epilogue: O^T / l, store.  Register r of column tile t is V column
+    //      (8*(r/4) + 4*lh + r%4) * kCPL + t of query row ln.
+    l_run += xor_shuffle(l_run, 32);
+    const float inv = (l_run > 0.f) ? 1.f / l_run : 0.f;
+    if (row_ok) {
+        uint16_t *dst = ob + (int64_t)(q0 + my_row) * p.o_stride_t;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int col = (8 * (r >> 2) + 4 * lh + (r & 3)) * Cfg::kCPL;
+            if constexpr (Cfg::kCPL == 4) {
+                uint2 o2;
+                o2.x = pack2<T>(o_acc[0][r] * inv, o_acc[1][r] * inv);
+                o2.y = pack2<T>(o_acc[2][r] * inv, o_acc[3][r] * inv);
+                *reinterpret_cast<uint2 *>(dst + col) = o2;
+            } else if constexpr (Cfg::kCPL == 8) {
+                u32x4_t o4;
+                o4[0] = pack2<T>(o_acc[0][r] * inv, o_acc[1][r] * inv);
+                o4[1] = pack2<T>(o_acc[2][r] * inv, o_acc[3][r] * inv);
+                o4[2] = pack2<T>(o_acc[4][r] * inv, o_acc[5][r] * inv);
+                o4[3] = pack2<T>(o_acc[6][r] * inv, o_acc[7][r] * inv);
+                store16(dst + col, o4);
+            } else {
+                *reinterpret_cast<uint32_t *>(dst + col) = pack2<T>(o_acc[0][r] * inv, o_acc[1][r] * inv);
+            }
+        }
+        if (lh == 0) lse_b[q0 + my_row] = (l_run > 0.f) ? (m_run + fast_log2(l_run)) * kLn2 : INFINITY;
+    }
+}
+
+template <typename T, int D> static hipError_t launch_prefill_d(const PrefillParams &p, hipStream_t stream) {
+    const int num_mb = (p.max_seqlen_q + kBM - 1) / kBM;
+    dim3 grid(num_mb, p.nheads, p.batch);
+    dim3 block(256);
+    const bool softcap = p.softcap_post != 0.f;
+    const bool paged = p.block_table != nullptr;
+    if (paged) {
+        if (softcap)
+            hipLaunchKernelGGL((prefill_kernel<T, D, true, true>), grid, block, 0, stream, p);
+        else
+            hipLaunchKernelGGL((prefill_kernel<T, D, true, false>), grid, block, 0, stream, p);
+    } else {
+        if (softcap)
+            hipLaunchKernelGGL((prefill_kernel<T, D, false, true>), grid, block, 0, stream, p);
+        else
+            hipLaunchKernelGGL((prefill_kernel<T, D, false, false>), grid, block, 0, stream, p);
+    }
+    return hipGetLastError();
+}
+
+template <typename T> static hipError_t launch_prefill_t(const PrefillParams &p, int headdim, hipStream_t stream) {
+    switch (headdim) {
+        case 64: return launch_prefill_d<T, 64>(p, stream);
+        case 128: return launch_prefill_d<T, 128>(p, stream);
+        case 256: return launch_prefill_d<T, 256>(p, stream);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+hipError_t launch_prefill(const PrefillParams &p, int dtype, int headdim, hipStream_t stream) {
+    if (p.max_seqlen_q <= 0 || p.batch <= 0) return hipSuccess;
+    return dtype == 0 ? launch_prefill_t<BF16>(p, headdim, stream) : launch_prefill_t<FP16>(p, headdim, stream);
+}
+
 }  // namespace fa

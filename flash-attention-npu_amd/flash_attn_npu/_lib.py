@@ -40,7 +40,7 @@ class VarlenArgs(C.Structure):
         [(n, _vp) for n in ("q", "k", "v", "out", "softmax_lse", "cu_seqlens_q", "cu_seqlens_k", "seqused_k",
                             "block_table")]
         + [(n, _i32) for n in ("batch", "total_q", "nheads", "nheads_k", "headdim", "max_seqlen_q", "max_seqlen_k",
-                               "page_size", "max_blocks_per_seq")]
+                               "page_size", "max_blocks_per_seq", "num_blocks")]
         + [(n, _i64) for n in ("q_stride_t", "q_stride_h", "k_stride_t", "k_stride_h", "v_stride_t", "v_stride_h",
                                "k_stride_block", "v_stride_block", "o_stride_t", "o_stride_h", "bt_stride_b")]
         + [("io_dtype", _i32), ("softmax_scale", _f32), ("softcap", _f32), ("causal", _i32), ("window_left", _i32),

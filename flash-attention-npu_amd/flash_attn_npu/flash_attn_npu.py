@@ -203,7 +203,7 @@ def varlen_fwd(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k_, leftpad_k_
         _require(seqused_k_.dtype == torch.int32, "seqused_k must have dtype int32")
         seqused_k_ = seqused_k_.contiguous()
         hk = k.shape[2]
-        a.page_size, a.max_blocks_per_seq = k.shape[1], block_table_.shape[1]
+        a.page_size, a.max_blocks_per_seq, a.num_blocks = k.shape[1], block_table_.shape[1], k.shape[0]
         a.k_stride_block, a.k_stride_t, a.k_stride_h = k.stride(0), k.stride(1), k.stride(2)
         a.v_stride_block, a.v_stride_t, a.v_stride_h = v.stride(0), v.stride(1), v.stride(2)
         a.block_table, a.seqused_k, a.bt_stride_b = _ptr(block_table_), _ptr(seqused_k_), block_table_.stride(0)

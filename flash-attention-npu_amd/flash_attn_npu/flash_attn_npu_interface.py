@@ -175,10 +175,14 @@ class FlashAttnVarlenFunc(torch.autograd.Function):
         if softmax_scale is None:
             softmax_scale = q.shape[-1] ** (-0.5)
         head_size_og = q.size(2)
-        if head_size_og % 8 != 0:
-            q = torch.nn.functional.pad(q, [0, 8 - head_size_og % 8])
-            k = torch.nn.functional.pad(k, [0, 8 - head_size_og % 8])
-            v = torch.nn.functional.pad(v, [0, 8 - head_size_og % 8])
+        # The reference pads the head dimension to a multiple of 8 (flash_attn_npu_interface.py:897-901);
+        # the gfx950 kernels are built for 64, 128 and 256, so pad with zeros to the next of those
+        # (zero columns change neither QK^T nor the kept columns of PV).
+        head_size_pad = next((x for x in (64, 128, 256) if x >= head_size_og), head_size_og)
+        if head_size_pad != head_size_og and block_table is None:
+            q = torch.nn.functional.pad(q, [0, head_size_pad - head_size_og])
+            k = torch.nn.functional.pad(k, [0, head_size_pad - head_size_og])
+            v = torch.nn.functional.pad(v, [0, head_size_pad - head_size_og])
         fwd = _wrapped_flash_attn_varlen_forward if torch.compiler.is_compiling() else _varlen_forward_eager
         out_padded, softmax_lse, S_dmask, rng_state = fwd(
             q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dropout_p, softmax_scale,

@@ -108,7 +108,7 @@ typedef struct fa_varlen_args {
     const int32_t *block_table;  /* (B, max_blocks_per_seq) or NULL */
     int32_t batch, total_q, nheads, nheads_k, headdim;
     int32_t max_seqlen_q, max_seqlen_k;
-    int32_t page_size, max_blocks_per_seq;
+    int32_t page_size, max_blocks_per_seq, num_blocks;   /* paged only */
     int64_t q_stride_t, q_stride_h;
     int64_t k_stride_t, k_stride_h;   /* dense: token stride ; paged: row stride */
     int64_t v_stride_t, v_stride_h;

@@ -1,0 +1,134 @@
+"""GPU parity of the tiled forward (varlen prefill, paged varlen, tall kvcache blocks) against the
+CPU oracle.  Shapes follow the reference's varlen cases (tests/test_flash_attn_npu_v2.py:522-560)."""
+import pytest
+import torch
+
+import fa_oracle as O
+from helpers import check_out, check_vs_golden, make_paged_case, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+def varlen_case(seqs_q, seqs_k, hq, hk, d, dtype=torch.bfloat16, seed=0, dist="normal"):
+    g = torch.Generator().manual_seed(seed)
+
+    def rnd(*shape):
+        if dist == "normal":
+            return torch.randn(*shape, generator=g)
+        return -5.0 + 10.0 * torch.rand(*shape, generator=g)
+
+    tq, tk = sum(seqs_q), sum(seqs_k)
+    cu_q = torch.tensor([0] + list(torch.tensor(seqs_q).cumsum(0)), dtype=torch.int32)
+    cu_k = torch.tensor([0] + list(torch.tensor(seqs_k).cumsum(0)), dtype=torch.int32)
+    return dict(q=rnd(tq, hq, d).to(dtype), k=rnd(tk, hk, d).to(dtype), v=rnd(tk, hk, d).to(dtype),
+                cu_q=cu_q, cu_k=cu_k, max_q=max(seqs_q), max_k=max(seqs_k))
+
+
+def run_varlen(c, **kw):
+    from flash_attn_npu import flash_attn_varlen_func
+    print("varlen", tuple(c["q"].shape), tuple(c["k"].shape), c["cu_q"].tolist(), c["cu_k"].tolist(), kw, flush=True)
+    out, lse, _ = flash_attn_varlen_func(c["q"].cuda(), c["k"].cuda(), c["v"].cuda(), c["cu_q"].cuda(), c["cu_k"].cuda(),
+                                         c["max_q"], c["max_k"], return_attn_probs=True, **kw)
+    torch.cuda.synchronize()
+    ref, ref_lse = O.flash_attn_varlen(c["q"], c["k"], c["v"], c["cu_q"], c["cu_k"], c["max_q"], c["max_k"], mode="fp32", **kw)
+    gold, gold_lse = O.flash_attn_varlen(c["q"], c["k"], c["v"], c["cu_q"], c["cu_k"], c["max_q"], c["max_k"], mode="golden", **kw)
+    return (out, lse), (ref, ref_lse), (gold, gold_lse)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("causal", [False, True])
+def test_varlen_basic(dtype, causal):
+    c = varlen_case([128, 300, 77, 512], [128, 300, 77, 512], 8, 2, 128, dtype=dtype, seed=1)
+    got, ref, gold = run_varlen(c, causal=causal)
+    check_out(got[0], ref[0], got[1], ref[1], "varlen_basic")
+    check_vs_golden(got[0], gold[0], got[1], gold[1], "varlen_basic")
+
+
+@pytest.mark.parametrize("seqs_q,seqs_k", [([100, 257], [300, 257]), ([300, 64], [100, 700]), ([1, 129, 5], [64, 130, 1000])])
+@pytest.mark.parametrize("causal", [False, True])
+def test_varlen_sq_ne_sk(seqs_q, seqs_k, causal):
+    c = varlen_case(seqs_q, seqs_k, 4, 4, 128, seed=2)
+    got, ref, gold = run_varlen(c, causal=causal)
+    check_out(got[0], ref[0], got[1], ref[1], "sq_ne_sk")
+
+
+@pytest.mark.parametrize("d", [64, 256, 111, 192])
+def test_varlen_headdims(d):
+    c = varlen_case([200, 130], [200, 130], 5 if d == 111 else 4, 1, d, seed=3)
+    got, ref, gold = run_varlen(c, causal=True)
+    check_out(got[0], ref[0], got[1], ref[1], f"d={d}")
+
+
+@pytest.mark.parametrize("window", [(64, 0), (100, 30), (-1, 17), (5, -1), (0, 0)])
+def test_varlen_window(window):
+    c = varlen_case([300, 150], [300, 400], 4, 2, 128, seed=4)
+    got, ref, gold = run_varlen(c, causal=False, window_size=window)
+    check_out(got[0], ref[0], got[1], ref[1], f"window={window}")
+
+
+def test_varlen_softcap_and_uniform5():
+    c = varlen_case([256, 100], [256, 100], 4, 2, 128, seed=5)
+    got, ref, gold = run_varlen(c, causal=True, softcap=5.0)
+    check_out(got[0], ref[0], got[1], ref[1], "softcap")
+    c = varlen_case([512, 64], [512, 64], 4, 1, 128, seed=6, dist="uniform5")
+    got, ref, gold = run_varlen(c, causal=True)
+    check_vs_golden(got[0], gold[0], got[1], gold[1], "uniform5")
+
+
+def test_varlen_per_sequence_independence():
+    from flash_attn_npu import flash_attn_varlen_func
+    c = varlen_case([150, 260, 33], [150, 260, 33], 4, 2, 128, seed=7)
+    q, k, v = c["q"].cuda(), c["k"].cuda(), c["v"].cuda()
+    full = flash_attn_varlen_func(q, k, v, c["cu_q"].cuda(), c["cu_k"].cuda(), c["max_q"], c["max_k"], causal=True)
+    for b in range(3):
+        a, e = int(c["cu_q"][b]), int(c["cu_q"][b + 1])
+        cu = torch.tensor([0, e - a], dtype=torch.int32).cuda()
+        one = flash_attn_varlen_func(q[a:e], k[a:e], v[a:e], cu, cu, e - a, e - a, causal=True)
+        assert torch.equal(one, full[a:e])
+
+
+def test_varlen_paged_kv():
+    from flash_attn_npu import flash_attn_varlen_func
+    lens_k = [700, 130, 1025]
+    lens_q = [64, 130, 300]
+    case = make_paged_case(3, 8, 2, 128, 256, lens_k, seed=8)
+    g = torch.Generator().manual_seed(9)
+    q = torch.randn(sum(lens_q), 8, 128, generator=g).to(torch.bfloat16)
+    cu_q = torch.tensor([0, 64, 194, 494], dtype=torch.int32)
+    cu_k = torch.tensor([0, 700, 830, 1855], dtype=torch.int32)
+    out, lse, _ = flash_attn_varlen_func(q.cuda(), case["k_cache"].cuda(), case["v_cache"].cuda(), cu_q.cuda(), cu_k.cuda(),
+                                         max(lens_q), max(lens_k), causal=True, return_attn_probs=True,
+                                         block_table=case["block_table"].cuda())
+    kl = torch.cat([O.gather_paged(case["k_cache"], case["block_table"][b], lens_k[b]) for b in range(3)])
+    vl = torch.cat([O.gather_paged(case["v_cache"], case["block_table"][b], lens_k[b]) for b in range(3)])
+    ref, ref_lse = O.flash_attn_varlen(q, kl, vl, cu_q, cu_k, max(lens_q), max(lens_k), causal=True, mode="fp32")
+    check_out(out, ref, lse, ref_lse, "paged varlen")
+
+
+@pytest.mark.parametrize("sq,hq,hk", [(128, 8, 2), (1024, 4, 4), (33, 8, 1), (17, 16, 2)])
+def test_kvcache_tall_query_blocks(sq, hq, hk):
+    # chunked prefill through the kvcache call: seqlen_q * group > 64 runs on the tiled kernel
+    from flash_attn_npu import flash_attn_with_kvcache
+    case = make_paged_case(2, hq, hk, 128, 128, [2048, 1100], seqlen_q=sq, seqlen_new=0, seed=10)
+    dev = to_dev(case)
+    for causal in (True, False):
+        out, lse = flash_attn_with_kvcache(dev["q"], dev["k_cache"], dev["v_cache"], cache_seqlens=dev["cache_seqlens"],
+                                           block_table=dev["block_table"], causal=causal, return_softmax_lse=True)
+        ref, ref_lse = O.flash_attn_with_kvcache(case["q"], case["k_cache"], case["v_cache"],
+                                                 cache_seqlens=case["cache_seqlens"], block_table=case["block_table"],
+                                                 causal=causal, mode="fp32")
+        check_out(out, ref, lse, ref_lse, f"tall sq={sq} causal={causal}")
+
+
+def test_kvcache_tall_with_append():
+    from flash_attn_npu import flash_attn_with_kvcache
+    case = make_paged_case(2, 8, 2, 128, 256, [500, 100], seqlen_q=200, seqlen_new=200, seed=11)
+    dev = to_dev(case)
+    out, lse = flash_attn_with_kvcache(dev["q"], dev["k_cache"], dev["v_cache"], dev["k"], dev["v"],
+                                       cache_seqlens=dev["cache_seqlens"], block_table=dev["block_table"], causal=True,
+                                       return_softmax_lse=True)
+    kc, vc = case["k_cache"].clone(), case["v_cache"].clone()
+    ref, ref_lse = O.flash_attn_with_kvcache(case["q"], kc, vc, case["k"], case["v"], cache_seqlens=case["cache_seqlens"],
+                                             block_table=case["block_table"], causal=True, mode="fp32")
+    assert torch.equal(dev["k_cache"].cpu().view(torch.int16), kc.view(torch.int16))
+    check_out(out, ref, lse, ref_lse, "tall append")
