@@ -125,17 +125,52 @@ def decode_workload(name: str, device, seed: int = 0, kv_layout: str = "nhd"):
     return w
 
 
+def mla_workload(device, seed: int = 0):
+    """BASELINE.json configs[3]: DeepSeek-V3-shaped latent decode, int8 cache with per-token fp32 scales."""
+    import torch
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    B, hq, page = 32, 128, 256
+    lens = torch.randint(2048, 16385, (B,), generator=g)
+    pages = [math.ceil(int(l) / page) for l in lens]
+    pool = sum(pages) + 8
+    perm = torch.randperm(pool, generator=g)
+    bt = torch.zeros(B, max(pages), dtype=torch.int32)
+    o = 0
+    for b in range(B):
+        bt[b, :pages[b]] = perm[o:o + pages[b]].to(torch.int32)
+        o += pages[b]
+    gd = torch.Generator(device=device).manual_seed(seed + 1)
+    latent = torch.randn(pool, page, 1, 576, generator=gd, device=device, dtype=torch.float32).to(torch.bfloat16)
+    # symmetric per-token quantiser: scale = absmax / 127 (fp32), code = clamp(rne(x / scale), -127, 127)
+    xf = latent.float()
+    scale = xf.abs().amax(dim=-1, keepdim=True) / 127.0
+    safe = torch.where(scale > 0, scale, torch.ones_like(scale))
+    code = torch.clamp(torch.round(xf / safe), -127, 127).to(torch.int8)
+    q = torch.randn(B, 1, hq, 576, generator=gd, device=device, dtype=torch.float32).to(torch.bfloat16)
+    return dict(name="c4", desc="DeepSeek-V3-shaped MLA decode, int8 latent cache (576 B + fp32 scale per token, V aliased "
+                                 "to the first 512 dims), B=32, 128 q heads, lens U[2048,16384], causal",
+                B=B, hq=hq, hk=1, d=576, dv=512, page=page, lens=lens, snew=0, window=(-1, -1), causal=True,
+                scale=192 ** -0.5, q=q, k_cache=code, v_cache=code[..., :512], k_scale=scale.squeeze(-1).contiguous(),
+                cache_seqlens=lens.to(torch.int32).to(device), block_table=bt.to(device), k=None, v=None,
+                rotary_cos=None, rotary_sin=None)
+
+
 def decode_algorithmic_bytes(w):
     """Algorithmic HBM bytes of one decode call: every visible K and V element once, q, out, LSE,
     the block-table entries touched, plus (separately) the append's read+write."""
     B, hq, hk, d, dv, page, snew = w["B"], w["hq"], w["hk"], w["d"], w["dv"], w["page"], w["snew"]
     wl = w["window"][0]
+    if w["k_cache"].dtype.itemsize == 1:
+        # aliased int8 latent: 576 code bytes + one fp32 scale per token, read once
+        per_key = d + 4
+    else:
+        per_key = hk * (d * 2 + dv * 2)
     kv = 0
     tbl = 0
     for l in w["lens"].tolist():
         lk = l + snew
         vis = lk if wl < 0 else min(lk, wl + 1)
-        kv += vis * hk * (d * 2 + dv * 2)
+        kv += vis * per_key
         tbl += 4 * math.ceil(vis / page)
     attn = kv + tbl + B * hq * (d * 2 + dv * 2) + B * hq * 4
     append = B * snew * hk * (d + dv) * (2 + 2)
@@ -146,15 +181,17 @@ def bind_decode(w, num_splits=0):
     from flash_attn_npu import flash_attn_npu as ops
     return ops.bind_kvcache(w["q"], w["k_cache"], w["v_cache"], w["k"], w["v"], w["cache_seqlens"], w["rotary_cos"],
                             w["rotary_sin"], None, None, w["block_table"], None, None, w["scale"], w["causal"],
-                            w["window"][0], w["window"][1], 0.0, False, num_splits)
+                            w["window"][0], w["window"][1], 0.0, False, num_splits, w.get("k_scale"), None)
 
 
 def cpu_decode_baseline(w, budget_s: float = 20.0):
     """The oracle's blocked golden (restated reference test golden) on host cores."""
     import torch
     import fa_oracle as O
-    keys = ("q", "k_cache", "v_cache", "k", "v", "cache_seqlens", "block_table", "rotary_cos", "rotary_sin")
-    h = {k: (w[k].cpu() if isinstance(w[k], torch.Tensor) else w[k]) for k in keys}
+    keys = ("q", "k_cache", "v_cache", "k", "v", "cache_seqlens", "block_table", "rotary_cos", "rotary_sin", "k_scale")
+    h = {k: (w[k].cpu() if isinstance(w.get(k), torch.Tensor) else w.get(k)) for k in keys}
+    if h["k_scale"] is not None:
+        h["v_cache"] = h["k_cache"][..., :w["dv"]]
     # bounded sample: leading batch rows until the budget is used up
     B = w["B"]
     rows = B
@@ -169,7 +206,7 @@ def cpu_decode_baseline(w, budget_s: float = 20.0):
                                   rotary_cos=h["rotary_cos"], rotary_sin=h["rotary_sin"],
                                   cache_seqlens=h["cache_seqlens"][sl], block_table=h["block_table"][sl],
                                   softmax_scale=w["scale"], causal=w["causal"], window_size=w["window"],
-                                  rotary_interleaved=False, mode="golden")
+                                  rotary_interleaved=False, k_scale_cache=h["k_scale"], mode="golden")
         times.append(time.perf_counter() - t1)
         done += 1
         if time.perf_counter() - t0 > budget_s:
@@ -191,7 +228,10 @@ def run_decode(args, name):
     import torch
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    sets = [decode_workload(name, dev, seed=s, kv_layout=args.kv_layout) for s in (0, 0)]
+    if name == "c4":
+        sets = [mla_workload(dev, seed=s) for s in (0, 0)]
+    else:
+        sets = [decode_workload(name, dev, seed=s, kv_layout=args.kv_layout) for s in (0, 0)]
     # same seed -> same lengths and table, but two distinct physical pools, so that alternating
     # them evicts the last-level cache between steps
     calls = [bind_decode(w, args.num_splits) for w in sets]
@@ -226,6 +266,7 @@ def run_decode(args, name):
     plan = _lib.SplitPlan()
     lib.fa_rocm_plan_kvcache(C.byref(calls[0].args), lib.fa_rocm_num_cus(), C.byref(plan))
 
+    kernel_name = "decode_mla_i8_kernel" if name == "c4" else "decode_paged_kernel"
     out = {
         "metric": "paged_decode_hbm_bandwidth", "value": total_bytes / (ms_per_step * 1e-3) / 1e9, "unit": "GB/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
@@ -237,11 +278,18 @@ def run_decode(args, name):
         "us_per_call": ms_per_step * 1e3,
         "pct_of_hbm_peak": 100.0 * total_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,
         "algorithmic_bytes": total_bytes,
-        "roofline": {"bound": "hbm", "kernel": "decode_paged_kernel", "achieved": achieved, "peak": HBM_PEAK_GBPS,
+        "roofline": {"bound": "hbm", "kernel": kernel_name, "achieved": achieved, "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS, "traffic": None,
                      "kernel_us": kern_ms * 1e3, "append_us": sum(a_ms) / len(a_ms) * 1e3,
                      "combine_us": sum(c_ms) / len(c_ms) * 1e3, "algorithmic_bytes_per_launch": attn_bytes},
     }
+    if name == "c4":
+        # arithmetic intensity of this config is above the ridge: report the matrix-core side too
+        flops = 2.0 * w["hq"] * (w["d"] + w["dv"]) * float(w["lens"].sum())
+        out["dtype"] = "int8 cache, bf16 MFMA"
+        out["roofline_mfma"] = {"bound": "mfma", "achieved": flops / (kern_ms * 1e-3) / 1e12, "peak": MFMA_BF16_PEAK_TFLOPS,
+                                "unit": "TFLOP/s", "frac": flops / (kern_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
+                                "algorithmic_flops": flops}
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_decode_baseline(w)
     return out
@@ -373,7 +421,7 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py needs a ROCm GPU", file=sys.stderr)
         sys.exit(2)
-    if args.config in ("c2", "c2_8k", "c3a", "c3b"):
+    if args.config in ("c2", "c2_8k", "c3a", "c3b", "c4"):
         out = run_decode(args, args.config)
     elif args.config == "c5":
         out = run_prefill(args)

@@ -13,12 +13,10 @@
 //   * S^T = K Q^T and O^T = V^T P^T run on the 16x16x32 MFMA so the softmax state of a query row
 //     lives in one lane column for both products (no cross-lane traffic for the rescale);
 //   * lengths are read on the device; no host copy of cache_seqlens, no mask tensor.
-#include "fa_device.h"
-#include "fa_kernels.h"
+#include "decode_common.h"
 
 namespace fa {
 
-constexpr int kChunk = 32;  // keys per wave step
 
 template <int D> struct DecodeCfg {
     static constexpr int kLanesPerRow = D / 8;            // 16-byte pieces in one K row
@@ -34,34 +32,6 @@ template <int D> struct DecodeCfg {
 // byte offset of 16-byte piece `ch` of row `row` in a wave's swizzled K tile
 template <int D> __device__ __forceinline__ int k_tile_offset(int row, int ch) {
     return row * (D * 2) + ((ch ^ (row & DecodeCfg<D>::kSwzMask)) << 4);
-}
-
-// Live key range [lo, hi) of the query block of batch row b, and its 32-key chunk span.
-struct UnitRange {
-    int len_cache, Lk, lo, hi;
-    int c0, nchunks;  // first chunk index (absolute) and number of chunks; nchunks == 0: nothing visible
-};
-
-__device__ __forceinline__ UnitRange unit_range(const DecodeParams &p, int b) {
-    UnitRange u;
-    u.len_cache = p.cache_seqlens[b];
-    u.Lk = u.len_cache + p.seqlen_new;
-    const int off = u.Lk - p.seqlen_q;
-    const int wr_eff = p.causal ? 0 : p.window_right;
-    u.lo = 0;
-    u.hi = u.Lk;
-    if (wr_eff >= 0) u.hi = min(u.Lk, p.seqlen_q - 1 + off + wr_eff + 1);
-    if (p.window_left >= 0) u.lo = max(0, off - p.window_left);
-    // keys the block table cannot address are not read
-    u.hi = min(u.hi, p.max_blocks * p.page_size);
-    if (u.Lk <= 0 || u.hi <= u.lo) {
-        u.lo = u.hi = 0;
-        u.c0 = u.nchunks = 0;
-    } else {
-        u.c0 = u.lo / kChunk;
-        u.nchunks = (u.hi + kChunk - 1) / kChunk - u.c0;
-    }
-    return u;
 }
 
 // One piece of work: query block (b, kvh) against keys [range_lo, range_hi).  Writes the final
@@ -490,94 +460,13 @@ decode_paged_kernel(const DecodeParams p) {
 // every workgroup for itself from the device-resident lengths.  A workgroup writes the final
 // output of every unit that lies wholly inside its share and at most two partials.
 
-// exclusive prefix of per-row chunk counts over 256 equal segments of the batch: s_pref[t] =
-// chunks of rows [0, t*seg); s_pref[256] = total.  All threads of a 256-thread block must call.
-__device__ __forceinline__ void batch_chunk_prefix(const DecodeParams &p, int *s_pref, int seg) {
-    __shared__ int s_wave[4];
-    const int tid = threadIdx.x;
-    int sum = 0;
-    for (int b = tid * seg; b < min(p.batch, (tid + 1) * seg); ++b) sum += unit_range(p, b).nchunks;
-    int inc = sum;
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-        const int v = __shfl_up(inc, d, 64);
-        if ((tid & 63) >= d) inc += v;
-    }
-    if ((tid & 63) == 63) s_wave[tid >> 6] = inc;
-    __syncthreads();
-    int base = 0;
-    for (int w = 0; w < (tid >> 6); ++w) base += s_wave[w];
-    s_pref[tid + 1] = base + inc;
-    if (tid == 0) s_pref[0] = 0;
-    __syncthreads();
-}
-
-struct UnitPos {
-    int b;          // batch row
-    int pref;       // chunks of rows before b (one kv head's worth)
-};
-
-// batch row whose units contain list position `pos` (0 <= pos < Hk * total)
-__device__ __forceinline__ UnitPos locate_row(const DecodeParams &p, const int *s_pref, int seg, int64_t pos) {
-    const int target = (int)(pos / p.nheads_k);  // rows with pref <= target < pref + n
-    int lo = 0, hi = 256;                        // segment t with s_pref[t] <= target < s_pref[t+1]
-    while (hi - lo > 1) {
-        const int mid = (lo + hi) >> 1;
-        if (s_pref[mid] <= target) lo = mid; else hi = mid;
-    }
-    UnitPos u;
-    u.b = lo * seg;
-    u.pref = s_pref[lo];
-    for (;;) {
-        const int n = unit_range(p, u.b).nchunks;
-        if (target < u.pref + n || u.b + 1 >= p.batch) break;
-        u.pref += n;
-        ++u.b;
-    }
-    return u;
-}
-
 template <typename T, int D, int RT, int NW, bool SOFTCAP>
 __global__ void __launch_bounds__(NW * 64, (D <= 128 && RT <= 2) ? 2 : 1)
 decode_balanced_kernel(const DecodeParams p) {
     static_assert(NW == 4, "the batch scan assumes 256 threads");
-    __shared__ int s_pref[257];
-    const int seg = (p.batch + 255) / 256;
-    batch_chunk_prefix(p, s_pref, seg);
-    const int64_t W = (int64_t)s_pref[256] * p.nheads_k;
-    const int G = gridDim.x;
-    const int g = blockIdx.x;
-    const int64_t S = max((W + G - 1) / G, (int64_t)1);
-    int64_t pos = (int64_t)g * S;
-    const int64_t end = min(W, pos + S);
-    if (pos >= end) return;
-
-    UnitPos up = locate_row(p, s_pref, seg, pos);
-    UnitRange ur = unit_range(p, up.b);
-    int64_t row_start = (int64_t)up.pref * p.nheads_k;          // list position of unit (b, 0)
-    int kvh = (int)((pos - row_start) / ur.nchunks);
-    int offset = (int)((pos - row_start) - (int64_t)kvh * ur.nchunks);  // chunks into the unit
-    bool first = true;
-    while (pos < end) {
-        const int take = (int)min((int64_t)(ur.nchunks - offset), end - pos);
-        const bool whole = (offset == 0) && (take == ur.nchunks);
-        const int c_lo = ur.c0 + offset;
-        const int range_lo = max(ur.lo, c_lo * kChunk);
-        const int range_hi = min(ur.hi, (c_lo + take) * kChunk);
-        process_piece<T, D, RT, NW, SOFTCAP>(p, up.b, kvh, ur, range_lo, range_hi, whole,
-                                             (int64_t)g * 2 + (first ? 0 : 1));
-        first = false;
-        pos += take;
-        offset = 0;
-        if (++kvh == p.nheads_k) {
-            kvh = 0;
-            do {
-                ++up.b;
-                if (up.b >= p.batch) return;
-                ur = unit_range(p, up.b);
-            } while (ur.nchunks == 0);
-        }
-    }
+    balanced_driver(p, [&](int b, int kvh, const UnitRange &ur, int range_lo, int range_hi, bool whole, int64_t slot) {
+        process_piece<T, D, RT, NW, SOFTCAP>(p, b, kvh, ur, range_lo, range_hi, whole, slot);
+    });
 }
 
 // Split-KV combine (CombineScale.hpp:166-194,249-316): LSE = M + log sum exp(lse_s - M),

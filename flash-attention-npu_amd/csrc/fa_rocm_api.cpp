@@ -97,6 +97,13 @@ int fa_rocm_kvcache_validate(const fa_kvcache_args *a) {
         if (a->headdim_qk != 576 || a->headdim_v != 512 || a->nheads_k != 1)
             return fail(FA_ERR_SHAPE, "int8 KV cache supports the latent layout only (1 kv head, 576/512 dims)");
         if (a->k_new) return fail(FA_ERR_UNSUPPORTED, "append into an int8 KV cache is not supported");
+        if (a->seqlen_q != 1 || a->nheads % 64 != 0)
+            return fail(FA_ERR_SHAPE, "int8 KV cache needs seqlen_q == 1 and a multiple of 64 query heads");
+        if (a->v_cache != a->k_cache || a->v_stride_block != a->k_stride_block || a->v_stride_row != a->k_stride_row)
+            return fail(FA_ERR_UNSUPPORTED, "int8 KV cache: v_cache must be the view k_cache[..., :512] of the latent cache");
+        if (a->softcap > 0.f) return fail(FA_ERR_UNSUPPORTED, "softcap is not supported with an int8 KV cache");
+        if (a->k_stride_row % 16 || a->k_stride_block % 16)
+            return fail(FA_ERR_SHAPE, "int8 cache strides must be multiples of 16 bytes");
     } else {
         if (a->headdim_qk > 256) return fail(FA_ERR_SHAPE, "FlashAttention only supports head dimension at most 256");
         if (a->headdim_qk != a->headdim_v) return fail(FA_ERR_SHAPE, "k and v head dimensions must match");
@@ -129,9 +136,10 @@ int fa_rocm_plan_kvcache(const fa_kvcache_args *a, int num_cus, fa_split_plan *p
     if (num_cus <= 0) num_cus = 256;
     std::memset(plan, 0, sizeof(*plan));
     const int group = a->nheads / (a->nheads_k > 0 ? a->nheads_k : 1);
-    const size_t rows = (size_t)a->seqlen_q * group;
+    // the int8 latent kernel works on units of 64 query heads and always uses the balanced partition
+    const size_t rows = is_mla_i8(a) ? 64 : (size_t)a->seqlen_q * group;
     const size_t slot_bytes = rows * ((size_t)a->headdim_v + 1) * sizeof(float);
-    if (a->num_splits == 0) {
+    if (a->num_splits == 0 || is_mla_i8(a)) {
         plan->mode = FA_SPLIT_BALANCED;
         plan->nsplits = 1;
         const int per_cu = is_mla_i8(a) ? 1 : fa::decode_wgs_per_cu(a->headdim_qk, (int)rows);
@@ -372,10 +380,15 @@ static int fwd_kvcache_impl(const fa_kvcache_args *a, void *stream_, void *const
     }
 
     hipError_t e;
-    if (is_mla_i8(a))
+    if (is_mla_i8(a)) {
+        p.nheads_k = a->nheads / 64;   // units per batch row: 64-head halves
+        p.group = 64;
+        p.rows = 64;
         e = fa::launch_decode_mla_i8(p, a->io_dtype, stream);
-    else
+    }
+    else {
         e = fa::launch_decode_paged(p, a->io_dtype, a->headdim_qk, stream);
+    }
     if (e != hipSuccess) return fail(FA_ERR_LAUNCH, "decode launch failed: %s", hipGetErrorString(e));
     mark(2);
     if (needs_combine) {

@@ -1,0 +1,67 @@
+"""GPU parity of the int8 latent (MLA) decode against the CPU oracle (dequantise-then-golden)."""
+import math
+
+import pytest
+import torch
+
+import fa_oracle as O
+from helpers import check_out, check_vs_golden
+
+pytestmark = pytest.mark.gpu
+
+
+def mla_case(B, hq, lens, page=256, seed=0, spare=2, zero_token=False):
+    g = torch.Generator().manual_seed(seed)
+    pages = [max(1, math.ceil(l / page)) for l in lens]
+    pool = sum(pages) + spare
+    perm = torch.randperm(pool, generator=g)
+    bt = torch.zeros(B, max(pages), dtype=torch.int32)
+    o = 0
+    for b in range(B):
+        bt[b, :pages[b]] = perm[o:o + pages[b]].to(torch.int32)
+        o += pages[b]
+    latent = torch.randn(pool, page, 1, 576, generator=g).to(torch.bfloat16)
+    if zero_token:
+        latent[bt[0, 0].item(), 3] = 0          # an all-zero token: scale 0, codes 0
+    code, scale = O.quantize_per_token(latent)
+    q = torch.randn(B, 1, hq, 576, generator=g).to(torch.bfloat16)
+    return dict(q=q, k_cache=code, k_scale=scale, block_table=bt, cache_seqlens=torch.tensor(lens, dtype=torch.int32))
+
+
+def run(case):
+    from flash_attn_npu import flash_attn_with_kvcache
+    kc = case["k_cache"].cuda()
+    print("mla", tuple(case["q"].shape), case["cache_seqlens"].tolist(), flush=True)
+    out, lse = flash_attn_with_kvcache(case["q"].cuda(), kc, kc[..., :512], cache_seqlens=case["cache_seqlens"].cuda(),
+                                       block_table=case["block_table"].cuda(), softmax_scale=192 ** -0.5, causal=True,
+                                       return_softmax_lse=True, k_scale_cache=case["k_scale"].cuda())
+    torch.cuda.synchronize()
+    res = {}
+    for mode in ("fp32", "golden"):
+        res[mode] = O.flash_attn_with_kvcache(case["q"], case["k_cache"], case["k_cache"][..., :512],
+                                              cache_seqlens=case["cache_seqlens"], block_table=case["block_table"],
+                                              softmax_scale=192 ** -0.5, causal=True, k_scale_cache=case["k_scale"], mode=mode)
+    return (out, lse), res["fp32"], res["golden"]
+
+
+@pytest.mark.parametrize("hq", [128, 64])
+def test_mla_basic(hq):
+    case = mla_case(3, hq, [700, 2048, 33], seed=1)
+    got, ref, gold = run(case)
+    check_out(got[0], ref[0], got[1], ref[1], "mla")
+    check_vs_golden(got[0], gold[0], got[1], gold[1], "mla")
+
+
+def test_mla_ragged_and_empty():
+    case = mla_case(5, 128, [1, 0, 255, 257, 5000], seed=2, zero_token=True)
+    got, ref, gold = run(case)
+    check_out(got[0], ref[0], got[1], ref[1], "mla ragged")
+
+
+def test_mla_codes_and_scales_untouched():
+    case = mla_case(2, 128, [900, 300], seed=3)
+    from flash_attn_npu import flash_attn_with_kvcache
+    kc, ks = case["k_cache"].cuda(), case["k_scale"].cuda()
+    flash_attn_with_kvcache(case["q"].cuda(), kc, kc[..., :512], cache_seqlens=case["cache_seqlens"].cuda(),
+                            block_table=case["block_table"].cuda(), softmax_scale=192 ** -0.5, causal=True, k_scale_cache=ks)
+    assert torch.equal(kc.cpu(), case["k_cache"]) and torch.equal(ks.cpu(), case["k_scale"])
