@@ -16,21 +16,31 @@ namespace fa {
 constexpr int kChunk = 32;  // keys per wave step
 
 // Live key range [lo, hi) of the query block of batch row b, and its 32-key chunk span.
+// M of the window normalisation for a decode launch: the batch maximum of the key counts when a
+// window was requested, else irrelevant (1).  Every thread of the workgroup must call.
+__device__ __forceinline__ int window_norm_m(const DecodeParams &p) {
+    if (p.window_left < 0 && p.window_right < 0) return 1;
+    return block_max_keys(p.cache_seqlens, p.batch, p.seqlen_new);
+}
+
 struct UnitRange {
     int len_cache, Lk, lo, hi;
+    int wl, wr;       // window after normalisation (-1 = unbounded); causal gives wr = 0
     int c0, nchunks;  // first chunk index (absolute) and number of chunks; nchunks == 0: nothing visible
 };
 
-__device__ __forceinline__ UnitRange unit_range(const DecodeParams &p, int b) {
+__device__ __forceinline__ UnitRange unit_range(const DecodeParams &p, int b, int M) {
     UnitRange u;
     u.len_cache = p.cache_seqlens[b];
     u.Lk = u.len_cache + p.seqlen_new;
     const int off = u.Lk - p.seqlen_q;
-    const int wr_eff = p.causal ? 0 : p.window_right;
+    u.wl = p.window_left;
+    u.wr = p.window_right;
+    normalize_window(u.wl, u.wr, p.causal, M);
     u.lo = 0;
     u.hi = u.Lk;
-    if (wr_eff >= 0) u.hi = min(u.Lk, p.seqlen_q - 1 + off + wr_eff + 1);
-    if (p.window_left >= 0) u.lo = max(0, off - p.window_left);
+    if (u.wr >= 0) u.hi = min(u.Lk, p.seqlen_q - 1 + off + u.wr + 1);
+    if (u.wl >= 0) u.lo = max(0, off - u.wl);
     // keys the block table cannot address are not read
     u.hi = min(u.hi, p.max_blocks * p.page_size);
     if (u.Lk <= 0 || u.hi <= u.lo) {
@@ -45,11 +55,11 @@ __device__ __forceinline__ UnitRange unit_range(const DecodeParams &p, int b) {
 
 // exclusive prefix of per-row chunk counts over 256 equal segments of the batch: s_pref[t] =
 // chunks of rows [0, t*seg); s_pref[256] = total.  All threads of a 256-thread block must call.
-__device__ __forceinline__ void batch_chunk_prefix(const DecodeParams &p, int *s_pref, int seg) {
+__device__ __forceinline__ void batch_chunk_prefix(const DecodeParams &p, int *s_pref, int seg, int M) {
     __shared__ int s_wave[4];
     const int tid = threadIdx.x;
     int sum = 0;
-    for (int b = tid * seg; b < min(p.batch, (tid + 1) * seg); ++b) sum += unit_range(p, b).nchunks;
+    for (int b = tid * seg; b < min(p.batch, (tid + 1) * seg); ++b) sum += unit_range(p, b, M).nchunks;
     int inc = sum;
 #pragma unroll
     for (int d = 1; d < 64; d <<= 1) {
@@ -71,7 +81,7 @@ struct UnitPos {
 };
 
 // batch row whose units contain list position `pos` (0 <= pos < Hk * total)
-__device__ __forceinline__ UnitPos locate_row(const DecodeParams &p, const int *s_pref, int seg, int64_t pos) {
+__device__ __forceinline__ UnitPos locate_row(const DecodeParams &p, const int *s_pref, int seg, int64_t pos, int M) {
     const int target = (int)(pos / p.nheads_k);  // rows with pref <= target < pref + n
     int lo = 0, hi = 256;                        // segment t with s_pref[t] <= target < s_pref[t+1]
     while (hi - lo > 1) {
@@ -82,7 +92,7 @@ __device__ __forceinline__ UnitPos locate_row(const DecodeParams &p, const int *
     u.b = lo * seg;
     u.pref = s_pref[lo];
     for (;;) {
-        const int n = unit_range(p, u.b).nchunks;
+        const int n = unit_range(p, u.b, M).nchunks;
         if (target < u.pref + n || u.b + 1 >= p.batch) break;
         u.pref += n;
         ++u.b;
@@ -98,7 +108,8 @@ template <typename PieceFn>
 __device__ __forceinline__ void balanced_driver(const DecodeParams &p, PieceFn piece) {
     __shared__ int s_pref[257];
     const int seg = (p.batch + 255) / 256;
-    batch_chunk_prefix(p, s_pref, seg);
+    const int M = window_norm_m(p);
+    batch_chunk_prefix(p, s_pref, seg, M);
     const int64_t W = (int64_t)s_pref[256] * p.nheads_k;
     const int G = gridDim.x;
     const int g = blockIdx.x;
@@ -107,8 +118,8 @@ __device__ __forceinline__ void balanced_driver(const DecodeParams &p, PieceFn p
     const int64_t end = min(W, pos + S);
     if (pos >= end) return;
 
-    UnitPos up = locate_row(p, s_pref, seg, pos);
-    UnitRange ur = unit_range(p, up.b);
+    UnitPos up = locate_row(p, s_pref, seg, pos, M);
+    UnitRange ur = unit_range(p, up.b, M);
     const int64_t row_start = (int64_t)up.pref * p.nheads_k;   // list position of unit (b, 0)
     int kvh = (int)((pos - row_start) / ur.nchunks);
     int offset = (int)((pos - row_start) - (int64_t)kvh * ur.nchunks);  // chunks into the unit
@@ -128,7 +139,7 @@ __device__ __forceinline__ void balanced_driver(const DecodeParams &p, PieceFn p
             do {
                 ++up.b;
                 if (up.b >= p.batch) return;
-                ur = unit_range(p, up.b);
+                ur = unit_range(p, up.b, M);
             } while (ur.nchunks == 0);
         }
     }

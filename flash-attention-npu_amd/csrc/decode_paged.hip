@@ -61,8 +61,8 @@ __device__ __forceinline__ void process_piece(const DecodeParams &p, const int b
     const int Lk = ur.Lk;
     const int Sq = p.seqlen_q;
     const int off = Lk - Sq;
-    const int wr_eff = p.causal ? 0 : p.window_right;
-    const int wl = p.window_left;
+    const int wr_eff = ur.wr;
+    const int wl = ur.wl;
 
     // per-lane visible key interval of query row (r*16 + ln), clipped to this split
     int row_lo[RT], row_hi[RT];
@@ -437,7 +437,7 @@ decode_paged_kernel(const DecodeParams p) {
     const int split = blockIdx.x;
     const int kvh = blockIdx.y;
     const int b = blockIdx.z;
-    const UnitRange ur = unit_range(p, b);
+    const UnitRange ur = unit_range(p, b, window_norm_m(p));
     const bool empty = ur.nchunks == 0;
     const int lo_al = ur.c0 * kChunk;
     // splits this row really has; the grid was sized from shapes, so clamp and let the last split
@@ -492,13 +492,14 @@ __global__ void __launch_bounds__(256) splitkv_combine_kernel(const DecodeParams
                         (int64_t)head * p.o_stride_h;
     float *lse_out = p.lse + ((int64_t)b * p.nheads + head) * Sq + qi;
 
-    const UnitRange ur = unit_range(p, b);
+    const int M = window_norm_m(p);
+    const UnitRange ur = unit_range(p, b, M);
     int ns;            // pieces of this unit
     int64_t g_first = 0;
     bool first_is_late = false;
     if constexpr (BALANCED) {
         const int seg = (p.batch + 255) / 256;
-        batch_chunk_prefix(p, s_pref, seg);
+        batch_chunk_prefix(p, s_pref, seg, M);
         if (ur.nchunks == 0) {
             // no visible key: no workgroup owned this unit
             for (int c = tid; c < D; c += 256) out_row[c] = 0;
@@ -510,7 +511,7 @@ __global__ void __launch_bounds__(256) splitkv_combine_kernel(const DecodeParams
         // chunks of rows before b
         const int t = b / seg;
         int pref = s_pref[t];
-        for (int bb = t * seg; bb < b; ++bb) pref += unit_range(p, bb).nchunks;
+        for (int bb = t * seg; bb < b; ++bb) pref += unit_range(p, bb, M).nchunks;
         const int64_t start = (int64_t)pref * p.nheads_k + (int64_t)kvh * ur.nchunks;
         const int64_t end = start + ur.nchunks;
         g_first = start / S;

@@ -97,6 +97,39 @@ __device__ __forceinline__ float quad_rows_sum(float v) {
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 
+// Window normalisation of the reference host (csrc/ascend910/flash_attn_npu/flash_api.cpp:483-505):
+// a side >= M is unbounded, causal forces right = 0; if what remains is a true window (not plain
+// causal), an unbounded side becomes M.  On return -1 still means unbounded.
+__device__ __forceinline__ void normalize_window(int &wl, int &wr, int causal, int M) {
+    if (M > 0 && wl >= M) wl = -1;
+    if (M > 0 && wr >= M) wr = -1;
+    if (causal) wr = 0;
+    const bool is_causal = wl < 0 && wr == 0;
+    const bool is_local = (wl >= 0 || wr >= 0) && !is_causal;
+    if (is_local) {
+        if (wl < 0) wl = M;
+        if (wr < 0) wr = M;
+    }
+}
+
+// Largest key count of the batch, max_b(seqlens[b] + add): the M of the window normalisation, which
+// the reference obtains by copying the lengths to the host (flash_api.cpp:459,477-481).  Every
+// thread of the workgroup must call; the result is the same in all of them.
+__device__ __forceinline__ int block_max_keys(const int32_t *seqlens, int batch, int add) {
+    __shared__ int s_max[16];
+    int m = 0;
+    for (int b = threadIdx.x; b < batch; b += blockDim.x) m = max(m, seqlens[b] + add);
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) m = max(m, __shfl_xor(m, d, 64));
+    const int nw = (blockDim.x + 63) >> 6;
+    if ((threadIdx.x & 63) == 0) s_max[threadIdx.x >> 6] = m;
+    __syncthreads();
+    m = s_max[0];
+    for (int w = 1; w < nw; ++w) m = max(m, s_max[w]);
+    __syncthreads();
+    return m;
+}
+
 // 16-byte global load / store through plain vector types
 __device__ __forceinline__ u32x4_t load16(const void *p) { return *reinterpret_cast<const u32x4_t *>(p); }
 __device__ __forceinline__ void store16(void *p, const u32x4_t &v) { *reinterpret_cast<u32x4_t *>(p) = v; }

@@ -83,7 +83,7 @@ struct PrefillParams {
     int64_t lse_stride_b, lse_stride_h;     // lse index = b*stride_b + h*stride_h + token
     float scale_log2, softcap_pre, softcap_post;
     int32_t causal, window_left, window_right;
-    int32_t num_m_blocks;                   // q tiles per sequence (grid.x)
+    int32_t window_norm_m;                  // key count the window is normalised with; 0 = each row's own
 };
 
 // dtype: 0 = bf16, 1 = fp16 (enum fa_dtype).  All return hipError_t of the launch.

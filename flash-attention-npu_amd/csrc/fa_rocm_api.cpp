@@ -300,6 +300,7 @@ static int fwd_kvcache_impl(const fa_kvcache_args *a, void *stream_, void *const
         pp.causal = a->causal;
         pp.window_left = a->window_left;
         pp.window_right = a->window_right;
+        pp.window_norm_m = 0;
         if (a->rotary_cos)
             return fail(FA_ERR_UNSUPPORTED, "rotary embedding needs seqlen_q * (nheads / nheads_k) <= %d", fa::kDecodeMaxRows);
         const hipError_t e = fa::launch_prefill(pp, a->io_dtype, a->headdim_qk, stream);
@@ -465,9 +466,11 @@ int fa_rocm_varlen_fwd(const fa_varlen_args *a, void *stream_) {
         pp.softcap_pre = a->softmax_scale / a->softcap;
         pp.softcap_post = a->softcap * kLog2e;
     }
+    // window normalisation with max_seqlen_k, as mha_varlen_fwd does (flash_api.cpp:938-943)
     pp.causal = a->causal;
     pp.window_left = a->window_left;
     pp.window_right = a->window_right;
+    pp.window_norm_m = a->max_seqlen_k;
     const hipError_t e = fa::launch_prefill(pp, a->io_dtype, a->headdim, static_cast<hipStream_t>(stream_));
     if (e != hipSuccess) return fail(FA_ERR_LAUNCH, "prefill launch failed: %s", hipGetErrorString(e));
     return FA_OK;

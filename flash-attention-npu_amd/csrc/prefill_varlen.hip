@@ -63,10 +63,18 @@ __global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) prefill_kernel(const 
         k0 = p.cu_seqlens_k[b];
         Sk = p.cu_seqlens_k[b + 1] - k0;
     }
+    // window normalisation: the varlen host passes max_seqlen_k as the reference does
+    // (flash_api.cpp:938-943); the kvcache layout has the lengths on the device only, so the batch
+    // maximum is reduced here when a window was requested
+    int wl = p.window_left, wr_eff = p.window_right;
+    int norm_m = p.window_norm_m;
+    if constexpr (PAGED) {
+        if (norm_m <= 0 && (wl >= 0 || wr_eff >= 0)) norm_m = block_max_keys(p.seqused_k, p.batch, p.seqlen_k_add);
+    }
+    if (norm_m <= 0) norm_m = max(Sk, 1);
+    normalize_window(wl, wr_eff, p.causal, norm_m);
     if (mb * kBM >= Sq) return;
     const int off = Sk - Sq;
-    const int wr_eff = p.causal ? 0 : p.window_right;
-    const int wl = p.window_left;
 
     const uint16_t *qb = reinterpret_cast<const uint16_t *>(p.q) + (int64_t)b * p.q_stride_b + (int64_t)h * p.q_stride_h;
     uint16_t *ob = reinterpret_cast<uint16_t *>(p.out) + (int64_t)b * p.o_stride_b + (int64_t)h * p.o_stride_h;

@@ -1,0 +1,143 @@
+"""CPU checks of the C ABI: the library loads without a GPU, exports every symbol the header
+declares, agrees with the Python binding on the argument records, validates arguments with the
+reference's messages, and plans splits consistently.  No compute call is made here."""
+import ctypes as C
+import os
+import re
+
+import pytest
+import torch
+
+from flash_attn_npu import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def header_functions():
+    text = open(os.path.join(ROOT, "include", "fa_rocm.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(fa_rocm_\w+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = C.CDLL(_lib.LIB_PATH)
+    names = header_functions()
+    assert len(names) >= 12
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in include/fa_rocm.h but not exported"
+    assert set(names) == set(_lib.EXPORTS), "binding and header list different entry points"
+
+
+def test_record_sizes_and_version():
+    lib = _lib.load()
+    assert lib.fa_rocm_abi_version() == 1
+    assert lib.fa_rocm_sizeof_kvcache_args() == C.sizeof(_lib.KvcacheArgs)
+    assert lib.fa_rocm_sizeof_varlen_args() == C.sizeof(_lib.VarlenArgs)
+
+
+def good_args():
+    a = _lib.KvcacheArgs()
+    for f in ("q", "out", "softmax_lse", "k_cache", "v_cache", "cache_seqlens", "block_table"):
+        setattr(a, f, 0x1000)
+    a.batch, a.seqlen_q, a.nheads, a.nheads_k, a.headdim_qk, a.headdim_v = 64, 1, 32, 8, 128, 128
+    a.num_blocks, a.page_size, a.max_blocks_per_seq = 1300, 256, 33
+    a.q_stride_b, a.q_stride_s, a.q_stride_h = 4096, 4096, 128
+    a.o_stride_b, a.o_stride_s, a.o_stride_h = 4096, 4096, 128
+    a.k_stride_block, a.k_stride_row, a.k_stride_h = 256 * 1024, 1024, 128
+    a.v_stride_block, a.v_stride_row, a.v_stride_h = 256 * 1024, 1024, 128
+    a.bt_stride_b = 33
+    a.io_dtype = a.kv_dtype = _lib.FA_BF16
+    a.softmax_scale = 128 ** -0.5
+    a.causal, a.window_left, a.window_right = 1, -1, -1
+    return a
+
+
+def expect_error(a, text):
+    lib = _lib.load()
+    assert lib.fa_rocm_kvcache_validate(C.byref(a)) != 0
+    assert text in _lib.last_error(), _lib.last_error()
+
+
+def test_validate_messages_follow_the_reference():
+    lib = _lib.load()
+    assert lib.fa_rocm_kvcache_validate(C.byref(good_args())) == 0
+    a = good_args(); a.io_dtype = 7
+    expect_error(a, "FlashAttention only supports FP16 and BF16 data types")          # flash_api.cpp:386
+    a = good_args(); a.kv_dtype = _lib.FA_FP16
+    expect_error(a, "query and key_cache must have the same dtype")                   # :387
+    a = good_args(); a.nheads = 30
+    expect_error(a, "Number of heads in key/value must divide number of heads in query")   # :457
+    a = good_args(); a.headdim_qk = a.headdim_v = 512
+    expect_error(a, "FlashAttention only supports head dimension at most 256")        # :456
+    a = good_args(); a.batch = 0
+    expect_error(a, "batch size must be positive")                                    # :455
+    a = good_args(); a.softcap = -1.0
+    expect_error(a, "softcap must be non-negative")                                   # :419
+    a = good_args(); a.block_table = None
+    expect_error(a, "block_table")
+    a = good_args(); a.q = None
+    expect_error(a, "non-NULL")
+    a = good_args(); a.page_size = 100
+    expect_error(a, "multiple of 32")
+    a = good_args(); a.k_new = 0x1000
+    expect_error(a, "k and v must be passed together")
+    a = good_args(); a.rotary_cos = a.rotary_sin = 0x1000
+    expect_error(a, "rotary embedding is only applied when k and v are passed")
+    a = good_args(); a.kv_dtype = _lib.FA_INT8
+    expect_error(a, "int8 KV cache needs k_scale_cache")
+    assert lib.fa_rocm_kvcache_validate(None) != 0
+
+
+def test_split_plan_invariants():
+    lib = _lib.load()
+    plan = _lib.SplitPlan()
+    a = good_args()
+    assert lib.fa_rocm_plan_kvcache(C.byref(a), 256, C.byref(plan)) == 0
+    assert plan.mode == 1 and plan.num_wgs == 512                      # balanced: two workgroups per CU
+    rows = 4
+    assert plan.workspace_bytes == 512 * 2 * rows * (128 + 1) * 4 == lib.fa_rocm_kvcache_workspace_bytes(C.byref(a), 256)
+    a.num_splits = 1
+    lib.fa_rocm_plan_kvcache(C.byref(a), 256, C.byref(plan))
+    assert plan.mode == 0 and plan.nsplits == 1 and plan.workspace_bytes == 0 and plan.split_keys >= 33 * 256
+    for n in (2, 3, 7, 33, 100):
+        a.num_splits = n
+        lib.fa_rocm_plan_kvcache(C.byref(a), 256, C.byref(plan))
+        assert 1 <= plan.nsplits <= n and plan.split_keys % 256 == 0
+        assert plan.nsplits * plan.split_keys >= 33 * 256               # the splits cover every addressable key
+        assert plan.workspace_bytes == (64 * 8 * plan.nsplits * rows * 129 * 4 if plan.nsplits > 1 else 0)
+    # a window bounds the live range: fewer keys per split
+    a.num_splits, a.window_left, a.window_right, a.causal = 4, 4095, 0, 0
+    lib.fa_rocm_plan_kvcache(C.byref(a), 256, C.byref(plan))
+    assert plan.nsplits * plan.split_keys >= 4096 + 32 and plan.split_keys <= 1280
+
+
+def test_operator_layer_fails_loudly_without_gpu_tensors():
+    from flash_attn_npu import flash_attn_varlen_func, flash_attn_with_kvcache
+    q = torch.zeros(1, 1, 8, 128, dtype=torch.bfloat16)
+    kc = torch.zeros(4, 256, 2, 128, dtype=torch.bfloat16)
+    bt = torch.zeros(1, 2, dtype=torch.int32)
+    with pytest.raises(RuntimeError, match="ROCm device"):
+        flash_attn_with_kvcache(q, kc, kc, cache_seqlens=5, block_table=bt)
+    with pytest.raises(RuntimeError, match="FP16 and BF16"):
+        flash_attn_with_kvcache(q.float(), kc.float(), kc.float(), cache_seqlens=5, block_table=bt)
+    with pytest.raises(RuntimeError, match="block_table"):
+        flash_attn_with_kvcache(q, kc, kc, cache_seqlens=5)
+    with pytest.raises(RuntimeError, match="alibi"):
+        flash_attn_with_kvcache(q, kc, kc, cache_seqlens=5, block_table=bt, alibi_slopes=torch.zeros(8))
+    with pytest.raises(RuntimeError, match="leftpad"):
+        flash_attn_with_kvcache(q, kc, kc, cache_seqlens=5, block_table=bt, cache_leftpad=torch.zeros(1, dtype=torch.int32))
+    cu = torch.tensor([0, 4], dtype=torch.int32)
+    x = torch.zeros(4, 8, 128, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="dropout"):
+        flash_attn_varlen_func(x, x, x, cu, cu, 4, 4, dropout_p=0.1)
+    with pytest.raises(RuntimeError, match="ROCm device"):
+        flash_attn_varlen_func(x, x, x, cu, cu, 4, 4)
+    with pytest.raises(RuntimeError, match="inference forward only"):
+        flash_attn_varlen_func(x.requires_grad_(), x, x, cu, cu, 4, 4)
+
+
+def test_missing_library_is_an_error(monkeypatch):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libfa_rocm.so")
+    with pytest.raises(RuntimeError, match="no CPU or PyTorch fallback"):
+        _lib.load()

@@ -129,3 +129,12 @@ def test_append_multi_token_crosses_page():
     assert torch.equal(dev["k_cache"].cpu().view(torch.int16), kc.view(torch.int16))
     assert torch.equal(dev["v_cache"].cpu().view(torch.int16), vc.view(torch.int16))
     check_out(got[0], ref[0], got[1], ref[1], "append3")
+
+
+@pytest.mark.parametrize("window", [(0, -1), (-1, 1), (1, 1), (3, 0), (-1, 7)])
+def test_decode_window_more_queries_than_keys(window):
+    # Sq > Sk: the reference's host normalisation (side >= Sk unbounded, unbounded side := Sk) is not
+    # mask-neutral here; kernel and oracle must agree on it
+    case = make_paged_case(2, 4, 2, 128, 256, [2, 1], seqlen_q=5, seed=13)
+    got, ref, gold, _ = run_both(case, causal=False, window_size=window)
+    check_out(got[0], ref[0], got[1], ref[1], f"sq>sk window={window}")

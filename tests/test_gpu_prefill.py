@@ -132,3 +132,10 @@ def test_kvcache_tall_with_append():
                                              block_table=case["block_table"], causal=True, mode="fp32")
     assert torch.equal(dev["k_cache"].cpu().view(torch.int16), kc.view(torch.int16))
     check_out(out, ref, lse, ref_lse, "tall append")
+
+
+@pytest.mark.parametrize("window", [(0, -1), (-1, 1), (2, 2), (-1, 40)])
+def test_varlen_window_more_queries_than_keys(window):
+    c = varlen_case([200, 40], [30, 90], 4, 2, 128, seed=12)
+    got, ref, gold = run_varlen(c, causal=False, window_size=window)
+    check_out(got[0], ref[0], got[1], ref[1], f"sq>sk window={window}")
