@@ -55,11 +55,17 @@ __device__ __forceinline__ UnitRange unit_range(const DecodeParams &p, int b, in
 
 // exclusive prefix of per-row chunk counts over 256 equal segments of the batch: s_pref[t] =
 // chunks of rows [0, t*seg); s_pref[256] = total.  All threads of a 256-thread block must call.
-__device__ __forceinline__ void batch_chunk_prefix(const DecodeParams &p, int *s_pref, int seg, int M) {
+// Returns whether some batch row has no visible key at all.
+__device__ __forceinline__ bool batch_chunk_prefix(const DecodeParams &p, int *s_pref, int seg, int M) {
     __shared__ int s_wave[4];
     const int tid = threadIdx.x;
     int sum = 0;
-    for (int b = tid * seg; b < min(p.batch, (tid + 1) * seg); ++b) sum += unit_range(p, b, M).nchunks;
+    bool empty_row = false;
+    for (int b = tid * seg; b < min(p.batch, (tid + 1) * seg); ++b) {
+        const int n = unit_range(p, b, M).nchunks;
+        sum += n;
+        empty_row |= (n == 0);
+    }
     int inc = sum;
 #pragma unroll
     for (int d = 1; d < 64; d <<= 1) {
@@ -67,12 +73,13 @@ __device__ __forceinline__ void batch_chunk_prefix(const DecodeParams &p, int *s
         if ((tid & 63) >= d) inc += v;
     }
     if ((tid & 63) == 63) s_wave[tid >> 6] = inc;
-    __syncthreads();
+    const bool any_empty = __syncthreads_or(empty_row ? 1 : 0) != 0;
     int base = 0;
     for (int w = 0; w < (tid >> 6); ++w) base += s_wave[w];
     s_pref[tid + 1] = base + inc;
     if (tid == 0) s_pref[0] = 0;
     __syncthreads();
+    return any_empty;
 }
 
 struct UnitPos {
@@ -101,46 +108,125 @@ __device__ __forceinline__ UnitPos locate_row(const DecodeParams &p, const int *
 }
 
 
+// Where a unit's pieces live: it is cut over workgroups g_first .. g_first + ns - 1; piece s sits
+// in slot 2*(g_first + s), except that piece 0 sits in the odd slot when its workgroup's share
+// started in an earlier unit.
+struct UnitPieces {
+    int ns;
+    int64_t g_first;
+    bool first_is_late;
+    __device__ __forceinline__ int64_t slot(int s) const { return (g_first + s) * 2 + ((s == 0 && first_is_late) ? 1 : 0); }
+};
+
+// Split-KV merge of one query row by one wave (CombineScale.hpp:166-194,249-316):
+// LSE = M + log sum exp(lse_s - M), out = sum exp(lse_s - LSE) * O_s.  Lanes own DV/64 columns.
+template <typename T, int DV, typename SlotFn>
+__device__ __forceinline__ void combine_row_wave(const DecodeParams &p, int b, int kvh, int row, int ns, SlotFn slot_of) {
+    constexpr int CPL = DV / 64;   // columns per lane (2, 4 or 8)
+    static_assert(CPL == 1 || CPL == 2 || CPL == 4 || CPL == 8, "column split");
+    const int lane = threadIdx.x & 63;
+    float mx = -INFINITY;
+    for (int s = lane; s < ns; s += 64) mx = fmaxf(mx, p.lse_partial[slot_of(s) * p.rows + row]);
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) mx = fmaxf(mx, __shfl_xor(mx, d, 64));
+    const float mx_use = (mx == -INFINITY) ? 0.f : mx;
+    float tot = 0.f;
+    float acc[CPL];
+#pragma unroll
+    for (int c = 0; c < CPL; ++c) acc[c] = 0.f;
+    for (int s = 0; s < ns; ++s) {
+        const int64_t srow = slot_of(s) * p.rows + row;
+        const float w = fast_exp2(p.lse_partial[srow] - mx_use);
+        tot += w;
+        const float *src = p.o_partial + srow * DV + lane * CPL;
+#pragma unroll
+        for (int c = 0; c < CPL; ++c) acc[c] += w * src[c];
+    }
+    const float inv = (tot > 0.f) ? 1.f / tot : 0.f;
+    const int qi = row / p.group;
+    const int head = kvh * p.group + (row - qi * p.group);
+    uint16_t *dst = reinterpret_cast<uint16_t *>(p.out) + (int64_t)b * p.o_stride_b + (int64_t)qi * p.o_stride_s +
+                    (int64_t)head * p.o_stride_h + lane * CPL;
+    if constexpr (CPL == 1) {
+        dst[0] = from_float<T>(acc[0] * inv);
+    } else {
+#pragma unroll
+        for (int c = 0; c < CPL; c += 2) *reinterpret_cast<uint32_t *>(dst + c) = pack2<T>(acc[c] * inv, acc[c + 1] * inv);
+    }
+    if (lane == 0)
+        p.lse[((int64_t)b * p.nheads + head) * p.seqlen_q + qi] = (tot > 0.f) ? (mx + fast_log2(tot)) * kLn2 : INFINITY;
+}
+
+// out = 0, lse = +inf for every row of a unit that has no visible key (init_outputs.hpp:58-102)
+template <int DV> __device__ __forceinline__ void init_empty_unit(const DecodeParams &p, int b, int kvh) {
+    for (int idx = threadIdx.x; idx < p.rows * (DV / 8); idx += blockDim.x) {
+        const int row = idx / (DV / 8);
+        const int piece = idx - row * (DV / 8);
+        const int qi = row / p.group;
+        const int head = kvh * p.group + (row - qi * p.group);
+        uint16_t *dst = reinterpret_cast<uint16_t *>(p.out) + (int64_t)b * p.o_stride_b + (int64_t)qi * p.o_stride_s +
+                        (int64_t)head * p.o_stride_h + piece * 8;
+        store16(dst, u32x4_t{0, 0, 0, 0});
+        if (piece == 0) p.lse[((int64_t)b * p.nheads + head) * p.seqlen_q + qi] = INFINITY;
+    }
+}
+
 // Walks the share of workgroup blockIdx.x and calls piece(b, kvh, unit, range_lo, range_hi, whole,
-// slot) for every piece in it.  `whole`: the piece is a complete unit (write the final output);
-// otherwise the partial goes to slot 2*g (piece starts the share) or 2*g + 1.
-template <typename PieceFn>
+// slot, pieces) for every piece in it.  `whole`: the piece is a complete unit (write the final
+// output); otherwise the partial goes to slot 2*g (piece starts the share) or 2*g + 1.  Units
+// without a visible key belong to no share: workgroup g initialises units g, g + G, ...
+template <int DV, typename PieceFn>
 __device__ __forceinline__ void balanced_driver(const DecodeParams &p, PieceFn piece) {
     __shared__ int s_pref[257];
     const int seg = (p.batch + 255) / 256;
     const int M = window_norm_m(p);
-    batch_chunk_prefix(p, s_pref, seg, M);
+    const bool any_empty = batch_chunk_prefix(p, s_pref, seg, M);
     const int64_t W = (int64_t)s_pref[256] * p.nheads_k;
     const int G = gridDim.x;
     const int g = blockIdx.x;
     const int64_t S = max((W + G - 1) / G, (int64_t)1);
     int64_t pos = (int64_t)g * S;
     const int64_t end = min(W, pos + S);
-    if (pos >= end) return;
 
-    UnitPos up = locate_row(p, s_pref, seg, pos, M);
-    UnitRange ur = unit_range(p, up.b, M);
-    const int64_t row_start = (int64_t)up.pref * p.nheads_k;   // list position of unit (b, 0)
-    int kvh = (int)((pos - row_start) / ur.nchunks);
-    int offset = (int)((pos - row_start) - (int64_t)kvh * ur.nchunks);  // chunks into the unit
-    bool first = true;
-    while (pos < end) {
-        const int take = (int)min((int64_t)(ur.nchunks - offset), end - pos);
-        const bool whole = (offset == 0) && (take == ur.nchunks);
-        const int c_lo = ur.c0 + offset;
-        const int range_lo = max(ur.lo, c_lo * kChunk);
-        const int range_hi = min(ur.hi, (c_lo + take) * kChunk);
-        piece(up.b, kvh, ur, range_lo, range_hi, whole, (int64_t)g * 2 + (first ? 0 : 1));
-        first = false;
-        pos += take;
-        offset = 0;
-        if (++kvh == p.nheads_k) {
-            kvh = 0;
-            do {
-                ++up.b;
-                if (up.b >= p.batch) return;
-                ur = unit_range(p, up.b, M);
-            } while (ur.nchunks == 0);
+    if (pos < end) {
+        UnitPos up = locate_row(p, s_pref, seg, pos, M);
+        UnitRange ur = unit_range(p, up.b, M);
+        const int64_t row_start = (int64_t)up.pref * p.nheads_k;   // list position of unit (b, 0)
+        int kvh = (int)((pos - row_start) / ur.nchunks);
+        int offset = (int)((pos - row_start) - (int64_t)kvh * ur.nchunks);  // chunks into the unit
+        bool first = true;
+        while (pos < end) {
+            const int take = (int)min((int64_t)(ur.nchunks - offset), end - pos);
+            const bool whole = (offset == 0) && (take == ur.nchunks);
+            const int c_lo = ur.c0 + offset;
+            const int range_lo = max(ur.lo, c_lo * kChunk);
+            const int range_hi = min(ur.hi, (c_lo + take) * kChunk);
+            UnitPieces pcs;
+            const int64_t u_start = pos - offset;
+            pcs.g_first = u_start / S;
+            pcs.ns = (int)((u_start + ur.nchunks - 1) / S - pcs.g_first + 1);
+            pcs.first_is_late = (u_start != pcs.g_first * S);
+            piece(up.b, kvh, ur, range_lo, range_hi, whole, (int64_t)g * 2 + (first ? 0 : 1), pcs);
+            first = false;
+            pos += take;
+            offset = 0;
+            if (++kvh == p.nheads_k) {
+                kvh = 0;
+                do {
+                    ++up.b;
+                    if (up.b < p.batch) ur = unit_range(p, up.b, M);
+                } while (up.b < p.batch && ur.nchunks == 0);
+                if (up.b >= p.batch) break;
+            }
+        }
+    }
+
+    if (any_empty) {
+        // rare: rows with no visible key
+        const int units = p.batch * p.nheads_k;
+        for (int u = g; u < units; u += G) {
+            const int b = u / p.nheads_k;
+            if (unit_range(p, b, M).nchunks == 0) init_empty_unit<DV>(p, b, u - b * p.nheads_k);
         }
     }
 }

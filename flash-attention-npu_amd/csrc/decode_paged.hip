@@ -464,76 +464,41 @@ template <typename T, int D, int RT, int NW, bool SOFTCAP>
 __global__ void __launch_bounds__(NW * 64, (D <= 128 && RT <= 2) ? 2 : 1)
 decode_balanced_kernel(const DecodeParams p) {
     static_assert(NW == 4, "the batch scan assumes 256 threads");
-    balanced_driver(p, [&](int b, int kvh, const UnitRange &ur, int range_lo, int range_hi, bool whole, int64_t slot) {
+    balanced_driver<D>(p, [&](int b, int kvh, const UnitRange &ur, int range_lo, int range_hi, bool whole, int64_t slot,
+                              const UnitPieces &pcs) {
         process_piece<T, D, RT, NW, SOFTCAP>(p, b, kvh, ur, range_lo, range_hi, whole, slot);
     });
 }
 
-// Split-KV combine (CombineScale.hpp:166-194,249-316): LSE = M + log sum exp(lse_s - M),
-// out = sum exp(lse_s - LSE) * O_s.  One 256-thread workgroup per (query row, kv head, batch row):
-// D/4 column groups x (1024/D) piece lanes, reduced through LDS.
-template <typename T, int D, bool BALANCED>
-__global__ void __launch_bounds__(256) splitkv_combine_kernel(const DecodeParams p) {
-    constexpr int CG = D / 4;        // threads across the columns (4 columns each)
-    constexpr int NPL = 256 / CG;    // piece lanes
-    __shared__ int s_pref[257];
-    __shared__ float s_red[4];
-    __shared__ float s_tot[NPL];
-    __shared__ __attribute__((aligned(16))) float s_acc[NPL][D];
-
+// Split-KV combine (CombineScale.hpp:166-194,249-316), one wave per query row.
+// Grid mode: one 64-thread workgroup per (query row, kv head, batch row).
+template <typename T, int D>
+__global__ void __launch_bounds__(64) splitkv_combine_kernel(const DecodeParams p) {
     const int row = blockIdx.x;
     const int kvh = blockIdx.y;
     const int b = blockIdx.z;
-    const int tid = threadIdx.x;
-    const int Sq = p.seqlen_q;
-    const int qi = row / p.group;
-    const int head = kvh * p.group + (row - qi * p.group);
-    uint16_t *out_row = reinterpret_cast<uint16_t *>(p.out) + (int64_t)b * p.o_stride_b + (int64_t)qi * p.o_stride_s +
-                        (int64_t)head * p.o_stride_h;
-    float *lse_out = p.lse + ((int64_t)b * p.nheads + head) * Sq + qi;
-
-    const int M = window_norm_m(p);
-    const UnitRange ur = unit_range(p, b, M);
-    int ns;            // pieces of this unit
-    int64_t g_first = 0;
-    bool first_is_late = false;
-    if constexpr (BALANCED) {
-        const int seg = (p.batch + 255) / 256;
-        batch_chunk_prefix(p, s_pref, seg, M);
-        if (ur.nchunks == 0) {
-            // no visible key: no workgroup owned this unit
-            for (int c = tid; c < D; c += 256) out_row[c] = 0;
-            if (tid == 0) *lse_out = INFINITY;
-            return;
-        }
-        const int64_t W = (int64_t)s_pref[256] * p.nheads_k;
-        const int64_t S = max((W + p.num_wgs - 1) / p.num_wgs, (int64_t)1);
-        // chunks of rows before b
-        const int t = b / seg;
-        int pref = s_pref[t];
-        for (int bb = t * seg; bb < b; ++bb) pref += unit_range(p, bb, M).nchunks;
-        const int64_t start = (int64_t)pref * p.nheads_k + (int64_t)kvh * ur.nchunks;
-        const int64_t end = start + ur.nchunks;
-        g_first = start / S;
-        const int64_t g_last = (end - 1) / S;
-        ns = (int)(g_last - g_first + 1);
-        first_is_late = (start != g_first * S);
-    } else {
-        const int lo_al = ur.c0 * kChunk;
-        ns = (ur.nchunks == 0) ? 1 : min(p.nsplits, (ur.hi - lo_al + p.split_keys - 1) / p.split_keys);
-    }
+    const UnitRange ur = unit_range(p, b, window_norm_m(p));
+    const int lo_al = ur.c0 * kChunk;
+    const int ns = (ur.nchunks == 0) ? 1 : min(p.nsplits, (ur.hi - lo_al + p.split_keys - 1) / p.split_keys);
     if (ns == 1) return;  // the decode kernel already wrote this unit
+    combine_row_wave<T, D>(p, b, kvh, row, ns,
+                           [&](int s) -> int64_t { return ((int64_t)b * p.nheads_k + kvh) * p.nsplits + s; });
+}
 
-    auto slot_of = [&](int s) -> int64_t {
-        if constexpr (BALANCED)
-            return (g_first + s) * 2 + ((s == 0 && first_is_late) ? 1 : 0);
-        else
-            return ((int64_t)b * p.nheads_k + kvh) * p.nsplits + s;
-    };
+// Merge of one query row by a whole 256-thread workgroup: D/4 column groups x (1024/D) piece
+// lanes, reduced through LDS.  Every thread of the workgroup must call.
+template <typename T, int D>
+__device__ __forceinline__ void combine_row_block(const DecodeParams &p, int b, int kvh, int row, const UnitPieces &pcs) {
+    constexpr int CG = D / 4;        // threads across the columns (4 columns each)
+    constexpr int NPL = 256 / CG;    // piece lanes
+    __shared__ float s_red[4];
+    __shared__ float s_tot[NPL];
+    __shared__ __attribute__((aligned(16))) float s_acc[NPL][D];
+    const int tid = threadIdx.x;
+    const int ns = pcs.ns;
 
-    // pass 1: maximum of the partial LSEs
     float mx = -INFINITY;
-    for (int s2 = tid; s2 < ns; s2 += 256) mx = fmaxf(mx, p.lse_partial[slot_of(s2) * p.rows + row]);
+    for (int s2 = tid; s2 < ns; s2 += 256) mx = fmaxf(mx, p.lse_partial[pcs.slot(s2) * p.rows + row]);
 #pragma unroll
     for (int d = 32; d >= 1; d >>= 1) mx = fmaxf(mx, __shfl_xor(mx, d, 64));
     if ((tid & 63) == 0) s_red[tid >> 6] = mx;
@@ -541,13 +506,12 @@ __global__ void __launch_bounds__(256) splitkv_combine_kernel(const DecodeParams
     mx = fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
     const float mx_use = (mx == -INFINITY) ? 0.f : mx;
 
-    // pass 2: weighted sum, piece lanes in parallel
     const int cg = tid % CG;
     const int pl = tid / CG;
     float tot = 0.f;
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
     for (int s2 = pl; s2 < ns; s2 += NPL) {
-        const int64_t srow = slot_of(s2) * p.rows + row;
+        const int64_t srow = pcs.slot(s2) * p.rows + row;
         const float w = fast_exp2(p.lse_partial[srow] - mx_use);
         tot += w;
         const float4 o = *reinterpret_cast<const float4 *>(p.o_partial + srow * D + cg * 4);
@@ -572,12 +536,44 @@ __global__ void __launch_bounds__(256) splitkv_combine_kernel(const DecodeParams
             acc[3] += o.w;
         }
         const float inv = (tot > 0.f) ? 1.f / tot : 0.f;
+        const int qi = row / p.group;
+        const int head = kvh * p.group + (row - qi * p.group);
+        uint16_t *out_row = reinterpret_cast<uint16_t *>(p.out) + (int64_t)b * p.o_stride_b + (int64_t)qi * p.o_stride_s +
+                            (int64_t)head * p.o_stride_h;
         uint2 o2;
         o2.x = pack2<T>(acc[0] * inv, acc[1] * inv);
         o2.y = pack2<T>(acc[2] * inv, acc[3] * inv);
         *reinterpret_cast<uint2 *>(out_row + cg * 4) = o2;
-        if (cg == 0) *lse_out = (tot > 0.f) ? (mx + fast_log2(tot)) * kLn2 : INFINITY;
+        if (cg == 0)
+            p.lse[((int64_t)b * p.nheads + head) * p.seqlen_q + qi] = (tot > 0.f) ? (mx + fast_log2(tot)) * kLn2 : INFINITY;
     }
+    __syncthreads();   // s_acc / s_red are reused by the next row
+}
+
+// Balanced mode: blockIdx = (row group, kv head, batch row).  The workgroup recomputes the partition,
+// finds the unit's pieces and merges query rows blockIdx.x, blockIdx.x + gridDim.x, ...
+template <typename T, int D>
+__global__ void __launch_bounds__(256) splitkv_combine_balanced_kernel(const DecodeParams p) {
+    __shared__ int s_pref[257];
+    const int kvh = blockIdx.y;
+    const int b = blockIdx.z;
+    const int M = window_norm_m(p);
+    const int seg = (p.batch + 255) / 256;
+    batch_chunk_prefix(p, s_pref, seg, M);
+    const UnitRange ur = unit_range(p, b, M);
+    if (ur.nchunks == 0) return;   // the decode kernel initialised this unit
+    const int64_t W = (int64_t)s_pref[256] * p.nheads_k;
+    const int64_t S = max((W + p.num_wgs - 1) / p.num_wgs, (int64_t)1);
+    const int t = b / seg;
+    int pref = s_pref[t];
+    for (int bb = t * seg; bb < b; ++bb) pref += unit_range(p, bb, M).nchunks;
+    const int64_t start = (int64_t)pref * p.nheads_k + (int64_t)kvh * ur.nchunks;
+    UnitPieces pcs;
+    pcs.g_first = start / S;
+    pcs.ns = (int)((start + ur.nchunks - 1) / S - pcs.g_first + 1);
+    pcs.first_is_late = (start != pcs.g_first * S);
+    if (pcs.ns == 1) return;       // written whole by one workgroup
+    for (int row = blockIdx.x; row < p.rows; row += gridDim.x) combine_row_block<T, D>(p, b, kvh, row, pcs);
 }
 
 template <typename T, int D, int RT>
@@ -624,11 +620,15 @@ hipError_t launch_decode_paged(const DecodeParams &p, int dtype, int headdim, hi
 int decode_wgs_per_cu(int headdim, int rows) { return (headdim <= 128 && rows <= 32) ? 2 : 1; }
 
 template <typename T, int D> static void launch_combine_d(const DecodeParams &p, hipStream_t stream) {
-    dim3 grid(p.rows, p.nheads_k, p.batch);
-    if (p.balanced)
-        hipLaunchKernelGGL((splitkv_combine_kernel<T, D, true>), grid, dim3(256), 0, stream, p);
-    else
-        hipLaunchKernelGGL((splitkv_combine_kernel<T, D, false>), grid, dim3(256), 0, stream, p);
+    if (p.balanced) {
+        // one workgroup per unit when there are many units, one per query row when there are few
+        const int units = p.nheads_k * p.batch;
+        const int row_groups = max(1, min(p.rows, 1024 / max(units, 1)));
+        hipLaunchKernelGGL((splitkv_combine_balanced_kernel<T, D>), dim3(row_groups, p.nheads_k, p.batch), dim3(256), 0,
+                           stream, p);
+    } else {
+        hipLaunchKernelGGL((splitkv_combine_kernel<T, D>), dim3(p.rows, p.nheads_k, p.batch), dim3(64), 0, stream, p);
+    }
 }
 
 template <typename T> static hipError_t launch_combine_t(const DecodeParams &p, int headdim_v, hipStream_t stream) {

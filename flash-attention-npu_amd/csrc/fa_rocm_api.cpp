@@ -247,16 +247,15 @@ static int fwd_kvcache_impl(const fa_kvcache_args *a, void *stream_, void *const
     const int group = a->nheads / a->nheads_k;
     const int rows = a->seqlen_q * group;
 
-    if (a->k_new) {
-        rc = fa_rocm_append_kv(a, stream_);
-        if (rc != FA_OK) return rc;
-    }
-
-    mark(1);
     const bool local = a->window_left >= 0 || a->window_right >= 0;
 
     if (!is_mla_i8(a) && rows > fa::kDecodeMaxRows) {
         // query block too tall for the decode kernel: tiled forward over the paged cache
+        if (a->k_new) {
+            rc = fa_rocm_append_kv(a, stream_);
+            if (rc != FA_OK) return rc;
+        }
+        mark(1);
         fa::PrefillParams pp;
         std::memset(&pp, 0, sizeof(pp));
         pp.q = a->q;
@@ -375,10 +374,16 @@ static int fwd_kvcache_impl(const fa_kvcache_args *a, void *stream_, void *const
     p.num_wgs = plan.num_wgs;
     const bool needs_combine = need > 0;
     if (needs_combine) {
-        const size_t slots = need / (((size_t)a->headdim_v + 1) * sizeof(float));   // slot rows
+        const size_t slot_rows = need / (((size_t)a->headdim_v + 1) * sizeof(float));
         p.o_partial = static_cast<float *>(a->workspace);
-        p.lse_partial = p.o_partial + slots * a->headdim_v;
+        p.lse_partial = p.o_partial + slot_rows * a->headdim_v;
     }
+
+    if (a->k_new) {
+        rc = fa_rocm_append_kv(a, stream_);
+        if (rc != FA_OK) return rc;
+    }
+    mark(1);
 
     hipError_t e;
     if (is_mla_i8(a)) {
