@@ -74,9 +74,11 @@ def decode_workload(name: str, device, seed: int = 0, kv_layout: str = "nhd"):
     import torch
     g = torch.Generator(device="cpu").manual_seed(seed)
     page = 256
-    if name in ("c2", "c2_8k"):
+    if name in ("c2", "c2_8k") or name.startswith("c2_u"):
         B, hq, hk, d = 64, 32, 8, 128
-        if name == "c2":
+        if name.startswith("c2_u"):
+            lens = torch.full((B,), int(name[4:]))      # c2_u<len>: every row the same length (scaling probe)
+        elif name == "c2":
             # uniform in [1024, 8191]: the appended key sits at position len <= 8191 < seqlen_ro
             lens = torch.randint(1024, 8192, (B,), generator=g)
         else:
@@ -276,7 +278,7 @@ def run_decode(args, name):
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"{name}: {w['desc']}", "batch": w["B"], "q_heads": w["hq"], "kv_heads": w["hk"],
                    "headdim": w["d"], "page_block_size": w["page"], "sum_keys": int(w["lens"].sum()) + w["B"] * w["snew"],
-                   "split_mode": "balanced" if plan.mode == 1 else "grid", "workgroups": plan.num_wgs,
+                   "split_mode": "balanced" if plan.mode == 1 else "grid", "workgroups": plan.num_wgs, "workers": plan.num_workers,
                    "kv_splits": plan.nsplits, "split_keys": plan.split_keys, "cold_cache": "two pools alternated", "kv_layout": args.kv_layout},
         "us_per_call": ms_per_step * 1e3,
         "pct_of_hbm_peak": 100.0 * total_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,
@@ -425,7 +427,7 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py needs a ROCm GPU", file=sys.stderr)
         sys.exit(2)
-    if args.config in ("c2", "c2_8k", "c3a", "c3b", "c4"):
+    if args.config in ("c2", "c2_8k", "c3a", "c3b", "c4") or args.config.startswith("c2_u"):
         out = run_decode(args, args.config)
     elif args.config == "c5":
         out = run_prefill(args)

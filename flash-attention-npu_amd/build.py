@@ -18,6 +18,7 @@ SOURCES = [
     "fa_rocm_api.cpp",
     "append_rope.hip",
     "decode_paged.hip",
+    "decode_wave.hip",
     "decode_mla_i8.hip",
     "prefill_varlen.hip",
 ]

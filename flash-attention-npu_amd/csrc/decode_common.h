@@ -171,64 +171,96 @@ template <int DV> __device__ __forceinline__ void init_empty_unit(const DecodePa
     }
 }
 
-// Walks the share of workgroup blockIdx.x and calls piece(b, kvh, unit, range_lo, range_hi, whole,
-// slot, pieces) for every piece in it.  `whole`: the piece is a complete unit (write the final
-// output); otherwise the partial goes to slot 2*g (piece starts the share) or 2*g + 1.  Units
-// without a visible key belong to no share: workgroup g initialises units g, g + G, ...
+// The balanced partition of a launch: W chunks in the list, S chunks per worker share.
+struct Partition {
+    int M;          // window normalisation key count
+    int seg;        // batch rows per prefix segment
+    int64_t W, S;
+    bool any_empty; // some batch row has no visible key
+};
+
+// Block-level (256 threads, contains barriers): prefix sums into s_pref[257], share size for
+// p.num_workers workers (never below p.min_share chunks).
+__device__ __forceinline__ Partition make_partition(const DecodeParams &p, int *s_pref) {
+    Partition pt;
+    pt.seg = (p.batch + 255) / 256;
+    pt.M = window_norm_m(p);
+    pt.any_empty = batch_chunk_prefix(p, s_pref, pt.seg, pt.M);
+    pt.W = (int64_t)s_pref[256] * p.nheads_k;
+    pt.S = max((pt.W + p.num_workers - 1) / p.num_workers, (int64_t)max(p.min_share, 1));
+    return pt;
+}
+
+// chunks of batch rows before b (one kv head's worth)
+__device__ __forceinline__ int chunks_before(const DecodeParams &p, const Partition &pt, const int *s_pref, int b) {
+    const int t = b / pt.seg;
+    int pref = s_pref[t];
+    for (int bb = t * pt.seg; bb < b; ++bb) pref += unit_range(p, bb, pt.M).nchunks;
+    return pref;
+}
+
+__device__ __forceinline__ UnitPieces unit_pieces(const Partition &pt, int64_t unit_start, int nchunks) {
+    UnitPieces pcs;
+    pcs.g_first = unit_start / pt.S;
+    pcs.ns = (int)((unit_start + nchunks - 1) / pt.S - pcs.g_first + 1);
+    pcs.first_is_late = (unit_start != pcs.g_first * pt.S);
+    return pcs;
+}
+
+// Walks the share of `worker` and calls piece(b, kvh, unit, range_lo, range_hi, whole, slot) for
+// every piece in it.  `whole`: the piece is a complete unit (write the final output); otherwise
+// the partial goes to slot 2*worker (piece starts the share) or 2*worker + 1.  No barriers inside:
+// a worker may be a workgroup or a single wave.
+template <typename PieceFn>
+__device__ __forceinline__ void walk_share(const DecodeParams &p, const Partition &pt, const int *s_pref, int64_t worker,
+                                           PieceFn piece) {
+    int64_t pos = worker * pt.S;
+    const int64_t end = min(pt.W, pos + pt.S);
+    if (pos >= end) return;
+    UnitPos up = locate_row(p, s_pref, pt.seg, pos, pt.M);
+    UnitRange ur = unit_range(p, up.b, pt.M);
+    const int64_t row_start = (int64_t)up.pref * p.nheads_k;   // list position of unit (b, 0)
+    int kvh = (int)((pos - row_start) / ur.nchunks);
+    int offset = (int)((pos - row_start) - (int64_t)kvh * ur.nchunks);  // chunks into the unit
+    bool first = true;
+    while (pos < end) {
+        const int take = (int)min((int64_t)(ur.nchunks - offset), end - pos);
+        const bool whole = (offset == 0) && (take == ur.nchunks);
+        const int c_lo = ur.c0 + offset;
+        const int range_lo = max(ur.lo, c_lo * kChunk);
+        const int range_hi = min(ur.hi, (c_lo + take) * kChunk);
+        piece(up.b, kvh, ur, range_lo, range_hi, whole, worker * 2 + (first ? 0 : 1));
+        first = false;
+        pos += take;
+        offset = 0;
+        if (++kvh == p.nheads_k) {
+            kvh = 0;
+            do {
+                ++up.b;
+                if (up.b < p.batch) ur = unit_range(p, up.b, pt.M);
+            } while (up.b < p.batch && ur.nchunks == 0);
+            if (up.b >= p.batch) break;
+        }
+    }
+}
+
+// Units without a visible key belong to no share: workgroup g initialises units g, g + G, ...
+template <int DV> __device__ __forceinline__ void init_empty_units(const DecodeParams &p, const Partition &pt) {
+    if (!pt.any_empty) return;
+    const int units = p.batch * p.nheads_k;
+    for (int u = blockIdx.x; u < units; u += gridDim.x) {
+        const int b = u / p.nheads_k;
+        if (unit_range(p, b, pt.M).nchunks == 0) init_empty_unit<DV>(p, b, u - b * p.nheads_k);
+    }
+}
+
+// Workgroup-level worker: the share of workgroup blockIdx.x, then the empty-unit duty.
 template <int DV, typename PieceFn>
 __device__ __forceinline__ void balanced_driver(const DecodeParams &p, PieceFn piece) {
     __shared__ int s_pref[257];
-    const int seg = (p.batch + 255) / 256;
-    const int M = window_norm_m(p);
-    const bool any_empty = batch_chunk_prefix(p, s_pref, seg, M);
-    const int64_t W = (int64_t)s_pref[256] * p.nheads_k;
-    const int G = gridDim.x;
-    const int g = blockIdx.x;
-    const int64_t S = max((W + G - 1) / G, (int64_t)1);
-    int64_t pos = (int64_t)g * S;
-    const int64_t end = min(W, pos + S);
-
-    if (pos < end) {
-        UnitPos up = locate_row(p, s_pref, seg, pos, M);
-        UnitRange ur = unit_range(p, up.b, M);
-        const int64_t row_start = (int64_t)up.pref * p.nheads_k;   // list position of unit (b, 0)
-        int kvh = (int)((pos - row_start) / ur.nchunks);
-        int offset = (int)((pos - row_start) - (int64_t)kvh * ur.nchunks);  // chunks into the unit
-        bool first = true;
-        while (pos < end) {
-            const int take = (int)min((int64_t)(ur.nchunks - offset), end - pos);
-            const bool whole = (offset == 0) && (take == ur.nchunks);
-            const int c_lo = ur.c0 + offset;
-            const int range_lo = max(ur.lo, c_lo * kChunk);
-            const int range_hi = min(ur.hi, (c_lo + take) * kChunk);
-            UnitPieces pcs;
-            const int64_t u_start = pos - offset;
-            pcs.g_first = u_start / S;
-            pcs.ns = (int)((u_start + ur.nchunks - 1) / S - pcs.g_first + 1);
-            pcs.first_is_late = (u_start != pcs.g_first * S);
-            piece(up.b, kvh, ur, range_lo, range_hi, whole, (int64_t)g * 2 + (first ? 0 : 1), pcs);
-            first = false;
-            pos += take;
-            offset = 0;
-            if (++kvh == p.nheads_k) {
-                kvh = 0;
-                do {
-                    ++up.b;
-                    if (up.b < p.batch) ur = unit_range(p, up.b, M);
-                } while (up.b < p.batch && ur.nchunks == 0);
-                if (up.b >= p.batch) break;
-            }
-        }
-    }
-
-    if (any_empty) {
-        // rare: rows with no visible key
-        const int units = p.batch * p.nheads_k;
-        for (int u = g; u < units; u += G) {
-            const int b = u / p.nheads_k;
-            if (unit_range(p, b, M).nchunks == 0) init_empty_unit<DV>(p, b, u - b * p.nheads_k);
-        }
-    }
+    const Partition pt = make_partition(p, s_pref);
+    walk_share(p, pt, s_pref, blockIdx.x, piece);
+    init_empty_units<DV>(p, pt);
 }
 
 }  // namespace fa

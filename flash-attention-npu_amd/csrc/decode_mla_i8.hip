@@ -40,8 +40,8 @@ template <typename T> __device__ __forceinline__ void widen4(uint32_t w, uint32_
 template <typename T>
 __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, const int half, const UnitRange &ur,
                                           const int range_lo, const int range_hi, const bool write_final,
-                                          const int64_t slot, const UnitPieces &pieces, uint8_t (*s_k)[kMlaTileBytes],
-                                          float (*s_ks)[kChunk], float (*s_vs)[kChunk]) {
+                                          const int64_t slot, uint8_t (*s_k)[kMlaTileBytes], float (*s_ks)[kChunk],
+                                          float (*s_vs)[kChunk]) {
     constexpr int KSTEPS = kMlaDqk / 32;   // 18
     constexpr int CT = kMlaDv / 16;        // 32 column tiles
     const int tid = threadIdx.x;
@@ -259,9 +259,8 @@ template <typename T> __global__ void __launch_bounds__(256, 1) decode_mla_i8_ke
     __shared__ __attribute__((aligned(16))) uint8_t s_k[2][kMlaTileBytes];
     __shared__ __attribute__((aligned(16))) float s_ks[2][kChunk];
     __shared__ __attribute__((aligned(16))) float s_vs[2][kChunk];
-    balanced_driver<kMlaDv>(p, [&](int b, int half, const UnitRange &ur, int range_lo, int range_hi, bool whole, int64_t slot,
-                                   const UnitPieces &pcs) {
-        mla_piece<T>(p, b, half, ur, range_lo, range_hi, whole, slot, pcs, s_k, s_ks, s_vs);
+    balanced_driver<kMlaDv>(p, [&](int b, int half, const UnitRange &ur, int range_lo, int range_hi, bool whole, int64_t slot) {
+        mla_piece<T>(p, b, half, ur, range_lo, range_hi, whole, slot, s_k, s_ks, s_vs);
     });
 }
 

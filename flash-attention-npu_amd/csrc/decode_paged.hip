@@ -464,8 +464,7 @@ template <typename T, int D, int RT, int NW, bool SOFTCAP>
 __global__ void __launch_bounds__(NW * 64, (D <= 128 && RT <= 2) ? 2 : 1)
 decode_balanced_kernel(const DecodeParams p) {
     static_assert(NW == 4, "the batch scan assumes 256 threads");
-    balanced_driver<D>(p, [&](int b, int kvh, const UnitRange &ur, int range_lo, int range_hi, bool whole, int64_t slot,
-                              const UnitPieces &pcs) {
+    balanced_driver<D>(p, [&](int b, int kvh, const UnitRange &ur, int range_lo, int range_hi, bool whole, int64_t slot) {
         process_piece<T, D, RT, NW, SOFTCAP>(p, b, kvh, ur, range_lo, range_hi, whole, slot);
     });
 }
@@ -557,21 +556,11 @@ __global__ void __launch_bounds__(256) splitkv_combine_balanced_kernel(const Dec
     __shared__ int s_pref[257];
     const int kvh = blockIdx.y;
     const int b = blockIdx.z;
-    const int M = window_norm_m(p);
-    const int seg = (p.batch + 255) / 256;
-    batch_chunk_prefix(p, s_pref, seg, M);
-    const UnitRange ur = unit_range(p, b, M);
+    const Partition pt = make_partition(p, s_pref);
+    const UnitRange ur = unit_range(p, b, pt.M);
     if (ur.nchunks == 0) return;   // the decode kernel initialised this unit
-    const int64_t W = (int64_t)s_pref[256] * p.nheads_k;
-    const int64_t S = max((W + p.num_wgs - 1) / p.num_wgs, (int64_t)1);
-    const int t = b / seg;
-    int pref = s_pref[t];
-    for (int bb = t * seg; bb < b; ++bb) pref += unit_range(p, bb, M).nchunks;
-    const int64_t start = (int64_t)pref * p.nheads_k + (int64_t)kvh * ur.nchunks;
-    UnitPieces pcs;
-    pcs.g_first = start / S;
-    pcs.ns = (int)((start + ur.nchunks - 1) / S - pcs.g_first + 1);
-    pcs.first_is_late = (start != pcs.g_first * S);
+    const int64_t start = (int64_t)chunks_before(p, pt, s_pref, b) * p.nheads_k + (int64_t)kvh * ur.nchunks;
+    const UnitPieces pcs = unit_pieces(pt, start, ur.nchunks);
     if (pcs.ns == 1) return;       // written whole by one workgroup
     for (int row = blockIdx.x; row < p.rows; row += gridDim.x) combine_row_block<T, D>(p, b, kvh, row, pcs);
 }
@@ -614,6 +603,7 @@ template <typename T> static hipError_t launch_decode_t(const DecodeParams &p, i
 }
 
 hipError_t launch_decode_paged(const DecodeParams &p, int dtype, int headdim, hipStream_t stream) {
+    if (p.balanced && p.wave_workers) return launch_decode_wave(p, dtype, headdim, stream);
     return dtype == 0 ? launch_decode_t<BF16>(p, headdim, stream) : launch_decode_t<FP16>(p, headdim, stream);
 }
 

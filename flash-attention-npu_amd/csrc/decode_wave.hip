@@ -1,0 +1,369 @@
+// Paged GQA/MQA decode for gfx950 with the wavefront as the unit of work: every wave owns a
+// contiguous share of the balanced chunk list, streams it with its own running (max, sum, O) and
+// writes its own final rows or partials.  After the one block-level prefix scan at kernel start
+// there is no workgroup barrier: a wave that crosses from one (batch row, kv head) unit into the
+// next only restarts its own pipeline while the other waves of the compute unit keep streaming.
+//
+// Same arithmetic as decode_paged.hip (the reference's hot loop, csrc/ascend910/flash_attn_npu/
+// mha_fwd_kvcache.cpp:632-969): S^T = K Q^T and O^T = V^T P^T on the 16x16x32 MFMA with the query
+// row in lane column lane%16; K rows through a wave-private swizzled LDS tile, V rows loaded in
+// operand order and transposed with v_perm; P rounded to the I/O dtype before PV.  Used when the
+// query block (seqlen_q * group rows) fits one 16-row tile.
+#include "decode_common.h"
+
+namespace fa {
+
+template <int D> struct WaveCfg {
+    static constexpr int kLanesPerRow = D / 8;
+    static constexpr int kRowsPerLoad = 64 / kLanesPerRow;
+    static constexpr int kKLoads = kChunk / kRowsPerLoad;
+    static constexpr int kKSteps = D / 32;
+    static constexpr int kVW = (D >= 128) ? 8 : D / 16;
+    static constexpr int kVH = D / (16 * kVW);
+    static constexpr int kColTiles = D / 16;
+    static constexpr int kSwzMask = (kLanesPerRow >= 16) ? 15 : kLanesPerRow - 1;
+    static constexpr int kTileBytes = kChunk * D * 2;
+    static constexpr int kPiecesPerRow = D / 8;   // 16-byte pieces of a query row
+};
+
+// Stage the 16-row query tile of unit (b, kvh), rotated if requested, into this wave's LDS rows.
+// Work item = one 16-byte piece of one row; in the non-interleaved rotary region the item of a
+// first-half piece also produces its partner piece rot/2 elements further on.
+template <typename T, int D>
+__device__ __forceinline__ void stage_q_wave(const DecodeParams &p, int b, int kvh, int len_cache, uint16_t *sq) {
+    using Cfg = WaveCfg<D>;
+    const int lane = threadIdx.x & 63;
+    const uint16_t *qbase = reinterpret_cast<const uint16_t *>(p.q) + (int64_t)b * p.q_stride_b;
+    const uint16_t *cosT = reinterpret_cast<const uint16_t *>(p.rotary_cos);
+    const uint16_t *sinT = reinterpret_cast<const uint16_t *>(p.rotary_sin);
+    const int rot = (cosT != nullptr) ? p.rotary_dim : 0;
+    const int half = rot >> 1;
+    for (int item = lane; item < 16 * Cfg::kPiecesPerRow; item += 64) {
+        const int row = item / Cfg::kPiecesPerRow;
+        const int ci = item - row * Cfg::kPiecesPerRow;
+        const int d0 = ci * 8;
+        uint16_t *dst = sq + row * D + d0;
+        if (row >= p.rows) {
+            *reinterpret_cast<u32x4_t *>(dst) = u32x4_t{0, 0, 0, 0};
+            continue;
+        }
+        const int qi = row / p.group;
+        const int g = row - qi * p.group;
+        const uint16_t *src = qbase + (int64_t)qi * p.q_stride_s + (int64_t)(kvh * p.group + g) * p.q_stride_h;
+        if (d0 >= rot) {
+            *reinterpret_cast<u32x4_t *>(dst) = load16(src + d0);
+            continue;
+        }
+        int pos = len_cache + (p.rotary_per_token ? qi : 0);
+        pos = min(max(pos, 0), p.seqlen_ro - 1);
+        const uint16_t *cs = cosT + (int64_t)pos * half;
+        const uint16_t *sn = sinT + (int64_t)pos * half;
+        if (p.rotary_interleaved) {
+            // pairs (2c, 2c+1) live inside the piece: pair index d0/2 + j
+            alignas(16) uint16_t x[8];
+            alignas(16) uint16_t o[8];
+            *reinterpret_cast<u32x4_t *>(x) = load16(src + d0);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float c = to_float<T>(cs[d0 / 2 + j]), s = to_float<T>(sn[d0 / 2 + j]);
+                const float x1 = to_float<T>(x[2 * j]), x2 = to_float<T>(x[2 * j + 1]);
+                o[2 * j] = from_float<T>(__fsub_rn(__fmul_rn(x1, c), __fmul_rn(x2, s)));
+                o[2 * j + 1] = from_float<T>(__fadd_rn(__fmul_rn(x1, s), __fmul_rn(x2, c)));
+            }
+            *reinterpret_cast<u32x4_t *>(dst) = *reinterpret_cast<const u32x4_t *>(o);
+        } else if (d0 < half) {
+            // pairs (c, c + rot/2): this piece and its partner
+            alignas(16) uint16_t x1v[8];
+            alignas(16) uint16_t x2v[8];
+            alignas(16) uint16_t o1[8];
+            alignas(16) uint16_t o2[8];
+            *reinterpret_cast<u32x4_t *>(x1v) = load16(src + d0);
+            *reinterpret_cast<u32x4_t *>(x2v) = load16(src + d0 + half);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const float c = to_float<T>(cs[d0 + j]), s = to_float<T>(sn[d0 + j]);
+                const float x1 = to_float<T>(x1v[j]), x2 = to_float<T>(x2v[j]);
+                o1[j] = from_float<T>(__fsub_rn(__fmul_rn(x1, c), __fmul_rn(x2, s)));
+                o2[j] = from_float<T>(__fadd_rn(__fmul_rn(x1, s), __fmul_rn(x2, c)));
+            }
+            *reinterpret_cast<u32x4_t *>(dst) = *reinterpret_cast<const u32x4_t *>(o1);
+            *reinterpret_cast<u32x4_t *>(dst + half) = *reinterpret_cast<const u32x4_t *>(o2);
+        }
+        // second-half pieces of the non-interleaved region are written by their partner's item
+    }
+}
+
+template <typename T, int D, bool SOFTCAP>
+__device__ __forceinline__ void wave_piece(const DecodeParams &p, const int b, const int kvh, const UnitRange &ur,
+                                           const int range_lo, const int range_hi, const bool write_final,
+                                           const int64_t slot, uint8_t *ktile, uint16_t *sq) {
+    using Cfg = WaveCfg<D>;
+    const int lane = threadIdx.x & 63;
+    const int lq = lane >> 4;
+    const int ln = lane & 15;
+    const int Lk = ur.Lk;
+    const int Sq = p.seqlen_q;
+    const int off = Lk - Sq;
+
+    const uint8_t *kc_base = reinterpret_cast<const uint8_t *>(p.k_cache) + (int64_t)kvh * p.k_stride_h * 2;
+    const uint8_t *vc_base = reinterpret_cast<const uint8_t *>(p.v_cache) + (int64_t)kvh * p.v_stride_h * 2;
+    const int32_t *bt_row = p.block_table + (int64_t)b * p.bt_stride_b;
+    const int c_begin = range_lo / kChunk;
+    const int c_end = (range_hi + kChunk - 1) / kChunk;
+
+    u32x4_t kreg[Cfg::kKLoads];
+    uint32_t vreg[8][Cfg::kVH][Cfg::kVW / 2];
+    const uint32_t k_row_bytes = (uint32_t)p.k_stride_row * 2u;
+    const uint32_t v_row_bytes = (uint32_t)p.v_stride_row * 2u;
+    const int k_lane_row = lane / Cfg::kLanesPerRow;
+    const uint32_t k_lane_col = (uint32_t)(lane % Cfg::kLanesPerRow) * 16u;
+    const uint32_t v_lane_col = (uint32_t)(ln * Cfg::kVW) * 2u;
+    const uint32_t k_lane_off = (uint32_t)k_lane_row * k_row_bytes + k_lane_col;
+    const uint32_t v_lane_off = (uint32_t)(lq * 4) * v_row_bytes + v_lane_col;
+
+    auto fetch_blk = [&](int c) -> int {
+        if (c >= c_end) return 0;
+        int page = (c * kChunk) / p.page_size;
+        page = min(page, p.max_blocks - 1);
+        const int blk = __builtin_amdgcn_readfirstlane(bt_row[page]);
+        return min(max(blk, 0), p.num_blocks - 1);
+    };
+    auto load_v = [&](const uint8_t *s2, int e, int hh) {
+        if constexpr (Cfg::kVW == 8) {
+            const u32x4_t t4 = load16(s2);
+            vreg[e][hh][0] = t4[0];
+            vreg[e][hh][1] = t4[1];
+            vreg[e][hh][2] = t4[2];
+            vreg[e][hh][3] = t4[3];
+        } else if constexpr (Cfg::kVW == 4) {
+            const uint2 t2 = *reinterpret_cast<const uint2 *>(s2);
+            vreg[e][hh][0] = t2.x;
+            vreg[e][hh][1] = t2.y;
+        } else {
+            vreg[e][hh][0] = *reinterpret_cast<const uint32_t *>(s2);
+        }
+    };
+    auto issue_loads = [&](int c, int blk) {
+        const int key0 = c * kChunk;
+        const int inpage0 = key0 % p.page_size;
+        const int last = Lk - 1 - key0;  // last written key relative to the chunk (>= 0)
+        const uint8_t *kb = kc_base + (int64_t)blk * p.k_stride_block * 2 + (int64_t)inpage0 * k_row_bytes;
+        const uint8_t *vb = vc_base + (int64_t)blk * p.v_stride_block * 2 + (int64_t)inpage0 * v_row_bytes;
+        if (last >= kChunk - 1) {
+#pragma unroll
+            for (int j = 0; j < Cfg::kKLoads; ++j)
+                kreg[j] = load16(kb + (size_t)(j * Cfg::kRowsPerLoad) * k_row_bytes + k_lane_off);
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+#pragma unroll
+                for (int hh = 0; hh < Cfg::kVH; ++hh)
+                    load_v(vb + (size_t)((e >> 2) * 16 + (e & 3)) * v_row_bytes + hh * 256 + v_lane_off, e, hh);
+        } else {
+            // tail chunk: rows past the last written key re-read that key (their scores are masked)
+#pragma unroll
+            for (int j = 0; j < Cfg::kKLoads; ++j) {
+                const int row = min(j * Cfg::kRowsPerLoad + k_lane_row, last);
+                kreg[j] = load16(kb + (uint32_t)row * k_row_bytes + k_lane_col);
+            }
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const int row = min((e >> 2) * 16 + lq * 4 + (e & 3), last);
+#pragma unroll
+                for (int hh = 0; hh < Cfg::kVH; ++hh) load_v(vb + (uint32_t)row * v_row_bytes + v_lane_col + hh * 256, e, hh);
+            }
+        }
+    };
+
+    // first chunk in flight while Q is staged
+    int c = c_begin;
+    int blk_next = fetch_blk(c);
+    if (c < c_end) issue_loads(c, blk_next);
+    blk_next = fetch_blk(c + 1);
+
+    stage_q_wave<T, D>(p, b, kvh, ur.len_cache, sq);
+    __builtin_amdgcn_wave_barrier();
+    u32x4_t qreg[Cfg::kKSteps];
+#pragma unroll
+    for (int t = 0; t < Cfg::kKSteps; ++t) qreg[t] = *reinterpret_cast<const u32x4_t *>(&sq[ln * D + t * 32 + lq * 8]);
+
+    // visible key interval of query row ln, clipped to this piece
+    int row_lo = range_lo, row_hi = range_hi - 1;
+    {
+        const int qi = ln / p.group;
+        if (ur.wl >= 0) row_lo = max(row_lo, qi + off - ur.wl);
+        if (ur.wr >= 0) row_hi = min(row_hi, qi + off + ur.wr);
+        if (ln >= p.rows) row_hi = -1;
+    }
+
+    float m_run = -INFINITY, l_run = 0.f;
+    float4_t o_acc[Cfg::kColTiles];
+#pragma unroll
+    for (int t = 0; t < Cfg::kColTiles; ++t) o_acc[t] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+    while (c < c_end) {
+        // staged chunk: K -> swizzled LDS tile, V -> transposed operand registers
+#pragma unroll
+        for (int j = 0; j < Cfg::kKLoads; ++j) {
+            const int row = j * Cfg::kRowsPerLoad + k_lane_row;
+            const int ch = lane % Cfg::kLanesPerRow;
+            *reinterpret_cast<u32x4_t *>(ktile + row * (D * 2) + ((ch ^ (row & Cfg::kSwzMask)) << 4)) = kreg[j];
+        }
+        u32x4_t vt[Cfg::kColTiles];
+#pragma unroll
+        for (int hh = 0; hh < Cfg::kVH; ++hh)
+#pragma unroll
+            for (int w2 = 0; w2 < Cfg::kVW / 2; ++w2)
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const uint32_t a = vreg[2 * u][hh][w2];
+                    const uint32_t bb = vreg[2 * u + 1][hh][w2];
+                    vt[hh * Cfg::kVW + 2 * w2][u] = __builtin_amdgcn_perm(bb, a, 0x05040100u);
+                    vt[hh * Cfg::kVW + 2 * w2 + 1][u] = __builtin_amdgcn_perm(bb, a, 0x07060302u);
+                }
+        __builtin_amdgcn_wave_barrier();
+
+        const int cn = c + 1;
+        if (cn < c_end) issue_loads(cn, blk_next);
+        blk_next = fetch_blk(cn + 1);
+        __builtin_amdgcn_sched_barrier(0);
+
+        // S^T = K Q^T, two 16-key tiles
+        float4_t s[2] = {float4_t{0.f, 0.f, 0.f, 0.f}, float4_t{0.f, 0.f, 0.f, 0.f}};
+#pragma unroll
+        for (int t = 0; t < Cfg::kKSteps; ++t)
+#pragma unroll
+            for (int tt = 0; tt < 2; ++tt) {
+                const int row = tt * 16 + ln;
+                const u32x4_t a = *reinterpret_cast<const u32x4_t *>(
+                    ktile + row * (D * 2) + (((t * 4 + lq) ^ (row & Cfg::kSwzMask)) << 4));
+                s[tt] = mfma16<T>(a, qreg[t], s[tt]);
+            }
+
+        // online softmax of query row ln; register i of tile tt is key c*32 + tt*16 + lq*4 + i
+        const int key_base = c * kChunk + lq * 4;
+        float x[8];
+        float mloc = -INFINITY;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const int key = key_base + (e >> 2) * 16 + (e & 3);
+            float v = s[e >> 2][e & 3];
+            if constexpr (SOFTCAP) {
+                const float y = v * p.softcap_pre;
+                const float e2 = __expf(2.f * y);
+                v = p.softcap_post * (1.f - 2.f / (e2 + 1.f));
+            } else {
+                v *= p.scale_log2;
+            }
+            v = (key >= row_lo && key <= row_hi) ? v : -INFINITY;
+            x[e] = v;
+            mloc = fmaxf(mloc, v);
+        }
+        mloc = quad_rows_max(mloc);
+        const float m_new = fmaxf(m_run, mloc);
+        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+        const float alpha = fast_exp2(m_run - m_use);
+        m_run = m_new;
+        float psum = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            x[e] = fast_exp2(x[e] - m_use);
+            psum += x[e];
+        }
+        l_run = l_run * alpha + psum;
+        u32x4_t pk;
+        pk[0] = pack2<T>(x[0], x[1]);
+        pk[1] = pack2<T>(x[2], x[3]);
+        pk[2] = pack2<T>(x[4], x[5]);
+        pk[3] = pack2<T>(x[6], x[7]);
+#pragma unroll
+        for (int t = 0; t < Cfg::kColTiles; ++t) {
+            o_acc[t][0] *= alpha;
+            o_acc[t][1] *= alpha;
+            o_acc[t][2] *= alpha;
+            o_acc[t][3] *= alpha;
+        }
+#pragma unroll
+        for (int t = 0; t < Cfg::kColTiles; ++t) o_acc[t] = mfma16<T>(vt[t], pk, o_acc[t]);
+        c = cn;
+    }
+
+    // ---- write.  Register i of column tile t = hh*kVW + w is column hh*128 + (lq*4 + i)*kVW + w
+    //      of query row ln: kVW consecutive columns per (hh, i).
+    l_run = quad_rows_sum(l_run);
+    if (ln < p.rows) {
+        const float inv = (l_run > 0.f) ? 1.f / l_run : 0.f;
+        const int qi = ln / p.group;
+        const int head = kvh * p.group + (ln - qi * p.group);
+        if (write_final) {
+            uint16_t *dst = reinterpret_cast<uint16_t *>(p.out) + (int64_t)b * p.o_stride_b + (int64_t)qi * p.o_stride_s +
+                            (int64_t)head * p.o_stride_h;
+#pragma unroll
+            for (int hh = 0; hh < Cfg::kVH; ++hh)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    uint16_t *d2 = dst + hh * 128 + (lq * 4 + i) * Cfg::kVW;
+#pragma unroll
+                    for (int w = 0; w < Cfg::kVW; w += 2)
+                        *reinterpret_cast<uint32_t *>(d2 + w) =
+                            pack2<T>(o_acc[hh * Cfg::kVW + w][i] * inv, o_acc[hh * Cfg::kVW + w + 1][i] * inv);
+                }
+            if (lq == 0)
+                p.lse[((int64_t)b * p.nheads + head) * Sq + qi] = (l_run > 0.f) ? (m_run + fast_log2(l_run)) * kLn2 : INFINITY;
+        } else {
+            const int64_t srow = slot * p.rows + ln;
+            float *dst = p.o_partial + srow * D;
+#pragma unroll
+            for (int hh = 0; hh < Cfg::kVH; ++hh)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    float *d2 = dst + hh * 128 + (lq * 4 + i) * Cfg::kVW;
+#pragma unroll
+                    for (int w = 0; w < Cfg::kVW; w += 2)
+                        *reinterpret_cast<float2 *>(d2 + w) =
+                            make_float2(o_acc[hh * Cfg::kVW + w][i] * inv, o_acc[hh * Cfg::kVW + w + 1][i] * inv);
+                }
+            if (lq == 0) p.lse_partial[srow] = (l_run > 0.f) ? m_run + fast_log2(l_run) : -INFINITY;
+        }
+    }
+    __builtin_amdgcn_wave_barrier();   // the wave's LDS rows are reused by its next piece
+}
+
+template <typename T, int D, bool SOFTCAP>
+__global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) decode_wave_kernel(const DecodeParams p) {
+    using Cfg = WaveCfg<D>;
+    __shared__ int s_pref[257];
+    __shared__ __attribute__((aligned(16))) uint8_t s_k[4][Cfg::kTileBytes];
+    __shared__ __attribute__((aligned(16))) uint16_t s_q[4][16 * D];
+    const Partition pt = make_partition(p, s_pref);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    walk_share(p, pt, s_pref, (int64_t)blockIdx.x * 4 + wave,
+               [&](int b, int kvh, const UnitRange &ur, int range_lo, int range_hi, bool whole, int64_t slot) {
+                   wave_piece<T, D, SOFTCAP>(p, b, kvh, ur, range_lo, range_hi, whole, slot, s_k[wave], s_q[wave]);
+               });
+    init_empty_units<D>(p, pt);
+}
+
+template <typename T, int D> static hipError_t launch_wave_d(const DecodeParams &p, hipStream_t stream) {
+    dim3 grid(p.num_wgs), block(256);
+    if (p.softcap_post != 0.f)
+        hipLaunchKernelGGL((decode_wave_kernel<T, D, true>), grid, block, 0, stream, p);
+    else
+        hipLaunchKernelGGL((decode_wave_kernel<T, D, false>), grid, block, 0, stream, p);
+    return hipGetLastError();
+}
+
+template <typename T> static hipError_t launch_wave_t(const DecodeParams &p, int headdim, hipStream_t stream) {
+    switch (headdim) {
+        case 64: return launch_wave_d<T, 64>(p, stream);
+        case 128: return launch_wave_d<T, 128>(p, stream);
+        case 256: return launch_wave_d<T, 256>(p, stream);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+hipError_t launch_decode_wave(const DecodeParams &p, int dtype, int headdim, hipStream_t stream) {
+    if (p.rows > 16 || !p.balanced || !p.wave_workers || p.num_workers != p.num_wgs * 4) return hipErrorInvalidValue;
+    return dtype == 0 ? launch_wave_t<BF16>(p, headdim, stream) : launch_wave_t<FP16>(p, headdim, stream);
+}
+
+}  // namespace fa

@@ -37,7 +37,9 @@ struct DecodeParams {
     float softcap_post;    // softcap * log2(e)
     int32_t causal, window_left, window_right;
     int32_t nsplits, split_keys;   // grid mode: split slots per unit, keys per split
-    int32_t balanced, num_wgs;     // balanced mode: workgroups sharing the chunk list equally
+    int32_t balanced, num_wgs;     // balanced mode: workgroups launched
+    int32_t num_workers, min_share;  // workers sharing the chunk list (workgroups, or waves), least chunks per share
+    int32_t wave_workers;          // 1: every wave is a worker (num_workers = 4 * num_wgs)
 };
 
 struct AppendParams {
@@ -89,6 +91,7 @@ struct PrefillParams {
 // dtype: 0 = bf16, 1 = fp16 (enum fa_dtype).  All return hipError_t of the launch.
 hipError_t launch_append_kv(const AppendParams &p, int dtype, hipStream_t stream);
 hipError_t launch_decode_paged(const DecodeParams &p, int dtype, int headdim, hipStream_t stream);
+hipError_t launch_decode_wave(const DecodeParams &p, int dtype, int headdim, hipStream_t stream);
 hipError_t launch_splitkv_combine(const DecodeParams &p, int dtype, int headdim_v, hipStream_t stream);
 hipError_t launch_decode_mla_i8(const DecodeParams &p, int dtype, hipStream_t stream);
 hipError_t launch_prefill(const PrefillParams &p, int dtype, int headdim, hipStream_t stream);

@@ -71,6 +71,8 @@ size_t fa_rocm_sizeof_kvcache_args(void) { return sizeof(fa_kvcache_args); }
 
 size_t fa_rocm_sizeof_varlen_args(void) { return sizeof(fa_varlen_args); }
 
+size_t fa_rocm_sizeof_split_plan(void) { return sizeof(fa_split_plan); }
+
 int fa_rocm_num_cus(void) { return device_cus(); }
 
 int fa_rocm_kvcache_validate(const fa_kvcache_args *a) {
@@ -144,13 +146,20 @@ int fa_rocm_plan_kvcache(const fa_kvcache_args *a, int num_cus, fa_split_plan *p
         plan->nsplits = 1;
         const int per_cu = is_mla_i8(a) ? 1 : fa::decode_wgs_per_cu(a->headdim_qk, (int)rows);
         plan->num_wgs = num_cus * per_cu;
+        plan->min_share = 1;
         // tuning aid: FA_ROCM_DECODE_WGS overrides the workgroup count of the balanced partition
         if (const char *env = std::getenv("FA_ROCM_DECODE_WGS")) {
             const int v = std::atoi(env);
             if (v > 0) plan->num_wgs = v;
         }
-        // every workgroup writes at most two partials (the units cut at the two ends of its share)
-        plan->workspace_bytes = (size_t)plan->num_wgs * 2 * slot_bytes;
+        // Query blocks of one 16-row tile: every wave is a worker with its own contiguous share (no
+        // workgroup barrier anywhere in the stream); taller blocks and the latent kernel: the
+        // workgroup is the worker.
+        const bool wave_workers = !is_mla_i8(a) && rows <= 16 && !std::getenv("FA_ROCM_DECODE_BLOCK_WORKERS");
+        plan->num_workers = wave_workers ? plan->num_wgs * 4 : plan->num_wgs;
+        if (wave_workers) plan->min_share = 8;
+        // every worker writes at most two partials (the units cut at the two ends of its share)
+        plan->workspace_bytes = (size_t)plan->num_workers * 2 * slot_bytes;
         return FA_OK;
     }
     const int64_t bound = live_keys_bound(a);
@@ -372,6 +381,9 @@ static int fwd_kvcache_impl(const fa_kvcache_args *a, void *stream_, void *const
     p.split_keys = plan.split_keys > 0 ? plan.split_keys : 256;
     p.balanced = plan.mode == FA_SPLIT_BALANCED;
     p.num_wgs = plan.num_wgs;
+    p.num_workers = plan.num_workers;
+    p.min_share = plan.min_share;
+    p.wave_workers = plan.num_workers != plan.num_wgs;
     const bool needs_combine = need > 0;
     if (needs_combine) {
         const size_t slot_rows = need / (((size_t)a->headdim_v + 1) * sizeof(float));

@@ -50,7 +50,8 @@ class VarlenArgs(C.Structure):
 
 class SplitPlan(C.Structure):
     """Mirror of struct fa_split_plan (include/fa_rocm.h)."""
-    _fields_ = [("mode", _i32), ("nsplits", _i32), ("split_keys", _i32), ("num_wgs", _i32), ("workspace_bytes", _sz)]
+    _fields_ = [("mode", _i32), ("nsplits", _i32), ("split_keys", _i32), ("num_wgs", _i32), ("num_workers", _i32),
+                ("min_share", _i32), ("workspace_bytes", _sz)]
 
 
 EXPORTS = {
@@ -58,6 +59,7 @@ EXPORTS = {
     "fa_rocm_last_error": (C.c_char_p, []),
     "fa_rocm_sizeof_kvcache_args": (_sz, []),
     "fa_rocm_sizeof_varlen_args": (_sz, []),
+    "fa_rocm_sizeof_split_plan": (_sz, []),
     "fa_rocm_num_cus": (C.c_int, []),
     "fa_rocm_plan_kvcache": (C.c_int, [C.POINTER(KvcacheArgs), C.c_int, C.POINTER(SplitPlan)]),
     "fa_rocm_kvcache_workspace_bytes": (_sz, [C.POINTER(KvcacheArgs), C.c_int]),
@@ -88,7 +90,8 @@ def load() -> C.CDLL:
         if lib.fa_rocm_abi_version() != 1:
             raise RuntimeError("libfa_rocm.so ABI version mismatch")
         if (lib.fa_rocm_sizeof_kvcache_args() != C.sizeof(KvcacheArgs)
-                or lib.fa_rocm_sizeof_varlen_args() != C.sizeof(VarlenArgs)):
+                or lib.fa_rocm_sizeof_varlen_args() != C.sizeof(VarlenArgs)
+                or lib.fa_rocm_sizeof_split_plan() != C.sizeof(SplitPlan)):
             raise RuntimeError("libfa_rocm.so argument records do not match this binding")
         _lib = lib
     return _lib

@@ -128,6 +128,7 @@ const char *fa_rocm_last_error(void);
 /* sizeof the two argument records as this library was compiled (binding self-check). */
 size_t fa_rocm_sizeof_kvcache_args(void);
 size_t fa_rocm_sizeof_varlen_args(void);
+size_t fa_rocm_sizeof_split_plan(void);
 /* Compute units of the current HIP device (256 on MI355X); < 0 on error. */
 int fa_rocm_num_cus(void);
 
@@ -136,9 +137,10 @@ int fa_rocm_num_cus(void);
  * Stands in for the reference's flash-decode heuristic and partition
  * (csrc/ascend910/flash_attn_npu/flash_api.cpp:525-550, splitBN2S1GS2 :343-354; forced mode
  * csrc/ascend910/flash_attn_npu_3/fa_split.h:345-350).
- *   mode FA_SPLIT_BALANCED (num_splits == 0): `num_wgs` workgroups share the list of all 32-key
- *     chunks of all (batch row, kv head) units equally, cutting inside a unit where a share ends;
- *     the shares are computed on the device from cache_seqlens.
+ *   mode FA_SPLIT_BALANCED (num_splits == 0): `num_workers` workers (workgroups, or single waves
+ *     when the query block is one 16-row tile) share the list of all 32-key chunks of all
+ *     (batch row, kv head) units equally, cutting inside a unit where a share ends; the shares
+ *     are computed on the device from cache_seqlens.
  *   mode FA_SPLIT_GRID (num_splits >= 1): every unit is cut into at most `nsplits` ranges of
  *     `split_keys` keys (a multiple of 256); num_splits == 1 gives nsplits == 1 (no split).
  * Pure host integer code: needs no GPU.  `num_cus` <= 0 means 256.
@@ -149,6 +151,8 @@ typedef struct fa_split_plan {
     int32_t nsplits;          /* grid mode: split slots per unit (>= 1)          */
     int32_t split_keys;       /* grid mode: keys per split                       */
     int32_t num_wgs;          /* balanced mode: workgroups launched              */
+    int32_t num_workers;      /* balanced mode: workers sharing the chunk list (a workgroup, or each of its 4 waves) */
+    int32_t min_share;        /* balanced mode: least 32-key chunks per share    */
     size_t workspace_bytes;   /* fp32 partial outputs + LSEs the call needs      */
 } fa_split_plan;
 int fa_rocm_plan_kvcache(const fa_kvcache_args *args, int num_cus, fa_split_plan *plan);

@@ -33,6 +33,7 @@ def test_record_sizes_and_version():
     assert lib.fa_rocm_abi_version() == 1
     assert lib.fa_rocm_sizeof_kvcache_args() == C.sizeof(_lib.KvcacheArgs)
     assert lib.fa_rocm_sizeof_varlen_args() == C.sizeof(_lib.VarlenArgs)
+    assert lib.fa_rocm_sizeof_split_plan() == C.sizeof(_lib.SplitPlan)
 
 
 def good_args():
@@ -94,8 +95,13 @@ def test_split_plan_invariants():
     a = good_args()
     assert lib.fa_rocm_plan_kvcache(C.byref(a), 256, C.byref(plan)) == 0
     assert plan.mode == 1 and plan.num_wgs == 512                      # balanced: two workgroups per CU
+    assert plan.num_workers == 2048 and plan.min_share == 8            # one 16-row tile: every wave is a worker
     rows = 4
-    assert plan.workspace_bytes == 512 * 2 * rows * (128 + 1) * 4 == lib.fa_rocm_kvcache_workspace_bytes(C.byref(a), 256)
+    assert plan.workspace_bytes == 2048 * 2 * rows * (128 + 1) * 4 == lib.fa_rocm_kvcache_workspace_bytes(C.byref(a), 256)
+    a.seqlen_q = 5                                                      # 20 rows: two tiles, the workgroup is the worker
+    lib.fa_rocm_plan_kvcache(C.byref(a), 256, C.byref(plan))
+    assert plan.num_workers == plan.num_wgs == 512 and plan.workspace_bytes == 512 * 2 * 20 * 129 * 4
+    a.seqlen_q = 1
     a.num_splits = 1
     lib.fa_rocm_plan_kvcache(C.byref(a), 256, C.byref(plan))
     assert plan.mode == 0 and plan.nsplits == 1 and plan.workspace_bytes == 0 and plan.split_keys >= 33 * 256
