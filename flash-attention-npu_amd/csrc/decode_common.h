@@ -88,8 +88,9 @@ struct UnitPos {
 };
 
 // batch row whose units contain list position `pos` (0 <= pos < Hk * total)
-__device__ __forceinline__ UnitPos locate_row(const DecodeParams &p, const int *s_pref, int seg, int64_t pos, int M) {
-    const int target = (int)(pos / p.nheads_k);  // rows with pref <= target < pref + n
+__device__ __forceinline__ UnitPos locate_row(const DecodeParams &p, const int *s_pref, int seg, int64_t pos, int M,
+                                              int list_heads) {
+    const int target = (int)(pos / list_heads);  // rows with pref <= target < pref + n
     int lo = 0, hi = 256;                        // segment t with s_pref[t] <= target < s_pref[t+1]
     while (hi - lo > 1) {
         const int mid = (lo + hi) >> 1;
@@ -108,14 +109,17 @@ __device__ __forceinline__ UnitPos locate_row(const DecodeParams &p, const int *
 }
 
 
-// Where a unit's pieces live: it is cut over workgroups g_first .. g_first + ns - 1; piece s sits
-// in slot 2*(g_first + s), except that piece 0 sits in the odd slot when its workgroup's share
-// started in an earlier unit.
+// Where a unit's pieces live: it is cut over shares g_first .. g_first + ns - 1; piece s sits in
+// slot 2*worker of its share's worker, except that piece 0 sits in the odd slot when its worker's
+// share started in an earlier unit.
 struct UnitPieces {
     int ns;
     int64_t g_first;
     bool first_is_late;
-    __device__ __forceinline__ int64_t slot(int s) const { return (g_first + s) * 2 + ((s == 0 && first_is_late) ? 1 : 0); }
+    int stride, offset;   // worker of share g: g * stride + offset
+    __device__ __forceinline__ int64_t slot(int s) const {
+        return ((g_first + s) * stride + offset) * 2 + ((s == 0 && first_is_late) ? 1 : 0);
+    }
 };
 
 // Split-KV merge of one query row by one wave (CombineScale.hpp:166-194,249-316):
@@ -172,11 +176,20 @@ template <int DV> __device__ __forceinline__ void init_empty_unit(const DecodePa
 }
 
 // The balanced partition of a launch: W chunks in the list, S chunks per worker share.
+// Two list orders.  Plain: units (b, kvh) with kvh inner, a share is any contiguous run of the
+// whole list.  Head-interleaved (p.head_interleave): the list holds the chunks of ONE kv head
+// (they are the same for every head); worker w streams share w / Hk of it for kv head w % Hk, so
+// Hk neighbouring workers read the same token range of all heads at the same time - adjacent
+// 256-byte pieces of the same cache rows.
 struct Partition {
     int M;          // window normalisation key count
     int seg;        // batch rows per prefix segment
+    int list_heads; // kv heads inside the list: nheads_k (plain) or 1 (head-interleaved)
     int64_t W, S;
     bool any_empty; // some batch row has no visible key
+    __device__ __forceinline__ int64_t worker_of(int64_t share, int kvh, int hk) const {
+        return list_heads == 1 ? share * hk + kvh : share;
+    }
 };
 
 // Block-level (256 threads, contains barriers): prefix sums into s_pref[257], share size for
@@ -186,8 +199,10 @@ __device__ __forceinline__ Partition make_partition(const DecodeParams &p, int *
     pt.seg = (p.batch + 255) / 256;
     pt.M = window_norm_m(p);
     pt.any_empty = batch_chunk_prefix(p, s_pref, pt.seg, pt.M);
-    pt.W = (int64_t)s_pref[256] * p.nheads_k;
-    pt.S = max((pt.W + p.num_workers - 1) / p.num_workers, (int64_t)max(p.min_share, 1));
+    pt.list_heads = p.head_interleave ? 1 : p.nheads_k;
+    pt.W = (int64_t)s_pref[256] * pt.list_heads;
+    const int64_t shares = p.head_interleave ? max(p.num_workers / p.nheads_k, 1) : p.num_workers;
+    pt.S = max((pt.W + shares - 1) / shares, (int64_t)max(p.min_share, 1));
     return pt;
 }
 
@@ -199,11 +214,13 @@ __device__ __forceinline__ int chunks_before(const DecodeParams &p, const Partit
     return pref;
 }
 
-__device__ __forceinline__ UnitPieces unit_pieces(const Partition &pt, int64_t unit_start, int nchunks) {
+__device__ __forceinline__ UnitPieces unit_pieces(const Partition &pt, int64_t unit_start, int nchunks, int kvh, int hk) {
     UnitPieces pcs;
     pcs.g_first = unit_start / pt.S;
     pcs.ns = (int)((unit_start + nchunks - 1) / pt.S - pcs.g_first + 1);
     pcs.first_is_late = (unit_start != pcs.g_first * pt.S);
+    pcs.stride = (pt.list_heads == 1) ? hk : 1;
+    pcs.offset = (pt.list_heads == 1) ? kvh : 0;
     return pcs;
 }
 
@@ -214,12 +231,15 @@ __device__ __forceinline__ UnitPieces unit_pieces(const Partition &pt, int64_t u
 template <typename PieceFn>
 __device__ __forceinline__ void walk_share(const DecodeParams &p, const Partition &pt, const int *s_pref, int64_t worker,
                                            PieceFn piece) {
-    int64_t pos = worker * pt.S;
+    const bool inter = pt.list_heads == 1;
+    const int64_t share = inter ? worker / p.nheads_k : worker;
+    const int fixed_kvh = inter ? (int)(worker - share * p.nheads_k) : 0;
+    int64_t pos = share * pt.S;
     const int64_t end = min(pt.W, pos + pt.S);
     if (pos >= end) return;
-    UnitPos up = locate_row(p, s_pref, pt.seg, pos, pt.M);
+    UnitPos up = locate_row(p, s_pref, pt.seg, pos, pt.M, pt.list_heads);
     UnitRange ur = unit_range(p, up.b, pt.M);
-    const int64_t row_start = (int64_t)up.pref * p.nheads_k;   // list position of unit (b, 0)
+    const int64_t row_start = (int64_t)up.pref * pt.list_heads;   // list position of unit (b, 0)
     int kvh = (int)((pos - row_start) / ur.nchunks);
     int offset = (int)((pos - row_start) - (int64_t)kvh * ur.nchunks);  // chunks into the unit
     bool first = true;
@@ -229,11 +249,11 @@ __device__ __forceinline__ void walk_share(const DecodeParams &p, const Partitio
         const int c_lo = ur.c0 + offset;
         const int range_lo = max(ur.lo, c_lo * kChunk);
         const int range_hi = min(ur.hi, (c_lo + take) * kChunk);
-        piece(up.b, kvh, ur, range_lo, range_hi, whole, worker * 2 + (first ? 0 : 1));
+        piece(up.b, inter ? fixed_kvh : kvh, ur, range_lo, range_hi, whole, worker * 2 + (first ? 0 : 1));
         first = false;
         pos += take;
         offset = 0;
-        if (++kvh == p.nheads_k) {
+        if (++kvh == pt.list_heads) {
             kvh = 0;
             do {
                 ++up.b;

@@ -559,9 +559,17 @@ __global__ void __launch_bounds__(256) splitkv_combine_balanced_kernel(const Dec
     const Partition pt = make_partition(p, s_pref);
     const UnitRange ur = unit_range(p, b, pt.M);
     if (ur.nchunks == 0) return;   // the decode kernel initialised this unit
-    const int64_t start = (int64_t)chunks_before(p, pt, s_pref, b) * p.nheads_k + (int64_t)kvh * ur.nchunks;
-    const UnitPieces pcs = unit_pieces(pt, start, ur.nchunks);
-    if (pcs.ns == 1) return;       // written whole by one workgroup
+    const int64_t start = (int64_t)chunks_before(p, pt, s_pref, b) * pt.list_heads +
+                          (pt.list_heads == 1 ? 0 : (int64_t)kvh * ur.nchunks);
+    const UnitPieces pcs = unit_pieces(pt, start, ur.nchunks, kvh, p.nheads_k);
+    if (pcs.ns == 1) return;       // written whole by one worker
+    if (gridDim.x == 1 && pcs.ns <= 16) {
+        // one workgroup for the whole unit and few pieces: the four waves merge rows side by side
+        const int wave = threadIdx.x >> 6;
+        for (int row = wave; row < p.rows; row += 4)
+            combine_row_wave<T, D>(p, b, kvh, row, pcs.ns, [&](int s) { return pcs.slot(s); });
+        return;
+    }
     for (int row = blockIdx.x; row < p.rows; row += gridDim.x) combine_row_block<T, D>(p, b, kvh, row, pcs);
 }
 

@@ -93,6 +93,59 @@ __device__ __forceinline__ void stage_q_wave(const DecodeParams &p, int b, int k
     }
 }
 
+// In-place append of the new rows whose positions fall into [range_lo, range_hi), by the wave that
+// is about to stream that range: same arithmetic as append_kv_kernel (separately rounded fp32
+// products and sum, round-to-nearest-even), so the written bytes are identical.
+template <typename T, int D>
+__device__ __forceinline__ void append_rows_wave(const DecodeParams &p, int b, int kvh, int len_cache, int range_lo,
+                                                 int range_hi) {
+    const int lane = threadIdx.x & 63;
+    const uint16_t *cosT = reinterpret_cast<const uint16_t *>(p.rotary_cos);
+    const uint16_t *sinT = reinterpret_cast<const uint16_t *>(p.rotary_sin);
+    const int rot = (cosT != nullptr) ? p.rotary_dim : 0;
+    const int half = rot >> 1;
+    for (int t = max(0, range_lo - len_cache); t < min(p.seqlen_new, range_hi - len_cache); ++t) {
+        const int pos = len_cache + t;
+        const int page = pos / p.page_size;
+        if (page >= p.max_blocks) continue;
+        const int blk = p.block_table[(int64_t)b * p.bt_stride_b + page];
+        if (blk < 0 || blk >= p.num_blocks) continue;
+        const int inpage = pos - page * p.page_size;
+        uint16_t *kdst = const_cast<uint16_t *>(reinterpret_cast<const uint16_t *>(p.k_cache)) + (int64_t)blk * p.k_stride_block +
+                         (int64_t)inpage * p.k_stride_row + (int64_t)kvh * p.k_stride_h;
+        uint16_t *vdst = const_cast<uint16_t *>(reinterpret_cast<const uint16_t *>(p.v_cache)) + (int64_t)blk * p.v_stride_block +
+                         (int64_t)inpage * p.v_stride_row + (int64_t)kvh * p.v_stride_h;
+        const uint16_t *ksrc = reinterpret_cast<const uint16_t *>(p.k_new) + (int64_t)b * p.kn_stride_b +
+                               (int64_t)t * p.kn_stride_s + (int64_t)kvh * p.kn_stride_h;
+        const uint16_t *vsrc = reinterpret_cast<const uint16_t *>(p.v_new) + (int64_t)b * p.vn_stride_b +
+                               (int64_t)t * p.vn_stride_s + (int64_t)kvh * p.vn_stride_h;
+        const int rpos = min(pos, p.seqlen_ro - 1);
+        for (int c = lane; c < D / 2; c += 64) {
+            int d1, d2;
+            if (c < half) {
+                d1 = p.rotary_interleaved ? 2 * c : c;
+                d2 = p.rotary_interleaved ? 2 * c + 1 : c + half;
+            } else {
+                d1 = rot + 2 * (c - half);
+                d2 = d1 + 1;
+            }
+            uint16_t o1 = ksrc[d1], o2 = ksrc[d2];
+            if (c < half) {
+                const float cs = to_float<T>(cosT[(int64_t)rpos * half + c]);
+                const float sn = to_float<T>(sinT[(int64_t)rpos * half + c]);
+                const float x1 = to_float<T>(o1), x2 = to_float<T>(o2);
+                o1 = from_float<T>(__fsub_rn(__fmul_rn(x1, cs), __fmul_rn(x2, sn)));
+                o2 = from_float<T>(__fadd_rn(__fmul_rn(x1, sn), __fmul_rn(x2, cs)));
+            }
+            kdst[d1] = o1;
+            kdst[d2] = o2;
+        }
+        for (int d = lane; d < D; d += 64) vdst[d] = vsrc[d];
+    }
+    // the wave's own later loads of these rows must find them
+    __threadfence_block();
+}
+
 template <typename T, int D, bool SOFTCAP>
 __device__ __forceinline__ void wave_piece(const DecodeParams &p, const int b, const int kvh, const UnitRange &ur,
                                            const int range_lo, const int range_hi, const bool write_final,
@@ -173,6 +226,8 @@ __device__ __forceinline__ void wave_piece(const DecodeParams &p, const int b, c
             }
         }
     };
+
+    if (p.k_new != nullptr && range_hi > ur.len_cache) append_rows_wave<T, D>(p, b, kvh, ur.len_cache, range_lo, range_hi);
 
     // first chunk in flight while Q is staged
     int c = c_begin;

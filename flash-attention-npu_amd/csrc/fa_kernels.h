@@ -17,6 +17,8 @@ struct DecodeParams {
     const void *v_cache;
     const float *k_scale;
     const float *v_scale;
+    const void *k_new;      // fused append (wave-level kernel): rows written by the wave that owns their chunk
+    const void *v_new;
     const void *rotary_cos;
     const void *rotary_sin;
     const int32_t *cache_seqlens;
@@ -31,6 +33,8 @@ struct DecodeParams {
     int64_t k_stride_block, k_stride_row, k_stride_h;
     int64_t v_stride_block, v_stride_row, v_stride_h;
     int64_t ks_stride_block, ks_stride_row;
+    int64_t kn_stride_b, kn_stride_s, kn_stride_h;
+    int64_t vn_stride_b, vn_stride_s, vn_stride_h;
     int64_t bt_stride_b;
     float scale_log2;      // softmax_scale * log2(e)            (softcap off)
     float softcap_pre;     // softmax_scale / softcap            (softcap on)
@@ -40,6 +44,7 @@ struct DecodeParams {
     int32_t balanced, num_wgs;     // balanced mode: workgroups launched
     int32_t num_workers, min_share;  // workers sharing the chunk list (workgroups, or waves), least chunks per share
     int32_t wave_workers;          // 1: every wave is a worker (num_workers = 4 * num_wgs)
+    int32_t head_interleave;       // 1: worker w streams share w / Hk of the per-head list for kv head w % Hk
 };
 
 struct AppendParams {

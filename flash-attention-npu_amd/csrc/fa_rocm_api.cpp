@@ -384,6 +384,9 @@ static int fwd_kvcache_impl(const fa_kvcache_args *a, void *stream_, void *const
     p.num_workers = plan.num_workers;
     p.min_share = plan.min_share;
     p.wave_workers = plan.num_workers != plan.num_wgs;
+    // wave workers of neighbouring kv heads walk the same token range together
+    p.head_interleave = p.wave_workers && a->nheads_k > 1 && plan.num_workers % a->nheads_k == 0 &&
+                        !std::getenv("FA_ROCM_NO_HEAD_INTERLEAVE");
     const bool needs_combine = need > 0;
     if (needs_combine) {
         const size_t slot_rows = need / (((size_t)a->headdim_v + 1) * sizeof(float));
@@ -391,7 +394,22 @@ static int fwd_kvcache_impl(const fa_kvcache_args *a, void *stream_, void *const
         p.lse_partial = p.o_partial + slot_rows * a->headdim_v;
     }
 
-    if (a->k_new) {
+    // The wave-level kernel appends on the fly when every new position is certain to be visible
+    // (and so owned by exactly one wave): causal or no right bound, and no left bound that could
+    // exclude the oldest new key.  Otherwise the rows are written by their own kernel first.
+    const bool fuse_append = a->k_new && p.balanced && p.wave_workers && (a->causal || a->window_right < 0) &&
+                             (a->window_left < 0 || (int64_t)a->seqlen_q + a->window_left >= a->seqlen_new) &&
+                             !std::getenv("FA_ROCM_SEPARATE_APPEND");
+    if (fuse_append) {
+        p.k_new = a->k_new;
+        p.v_new = a->v_new;
+        p.kn_stride_b = a->kn_stride_b;
+        p.kn_stride_s = a->kn_stride_s;
+        p.kn_stride_h = a->kn_stride_h;
+        p.vn_stride_b = a->vn_stride_b;
+        p.vn_stride_s = a->vn_stride_s;
+        p.vn_stride_h = a->vn_stride_h;
+    } else if (a->k_new) {
         rc = fa_rocm_append_kv(a, stream_);
         if (rc != FA_OK) return rc;
     }
