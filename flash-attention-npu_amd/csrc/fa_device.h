@@ -43,9 +43,18 @@ template <> __device__ __forceinline__ uint16_t from_float<FP16>(float f) {
     return b;
 }
 
-// two floats -> one dword holding (lo = a, hi = b) in the 16-bit type
-template <typename T> __device__ __forceinline__ uint32_t pack2(float a, float b) {
-    return static_cast<uint32_t>(from_float<T>(a)) | (static_cast<uint32_t>(from_float<T>(b)) << 16);
+// two floats -> one dword holding (lo = a, hi = b) in the 16-bit type, round-to-nearest-even
+// (bf16: one v_cvt_pk_bf16_f32)
+typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2_t;
+typedef __attribute__((__vector_size__(2 * sizeof(_Float16)))) _Float16 half2_t;
+template <typename T> __device__ __forceinline__ uint32_t pack2(float a, float b);
+template <> __device__ __forceinline__ uint32_t pack2<BF16>(float a, float b) {
+    const bf16x2_t v = {static_cast<__bf16>(a), static_cast<__bf16>(b)};
+    return __builtin_bit_cast(uint32_t, v);
+}
+template <> __device__ __forceinline__ uint32_t pack2<FP16>(float a, float b) {
+    const half2_t v = {static_cast<_Float16>(a), static_cast<_Float16>(b)};
+    return __builtin_bit_cast(uint32_t, v);
 }
 
 // ---- MFMA 16x16x32: D(16x16) += A(16x32) * B(32x16), 16-bit inputs, fp32 accumulate -------

@@ -201,38 +201,62 @@ __global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) prefill_kernel(const 
         //      kt*64 + tt*32 + 8*(r/4) + 4*lh + r%4
         const int tile0 = kt * kBN;
         const bool need_mask = (tile0 < wave_klo_max) || (tile0 + kBN - 1 > wave_khi_min);
+        // Fast path (no softcap, no element masks, positive scale): the maximum is taken on the raw
+        // scores and the scale rides in the exponent's fused multiply-add.
+        const bool raw_path = !SOFTCAP && !need_mask && p.scale_log2 > 0.f;
         float mloc = -INFINITY;
+        if (raw_path) {
 #pragma unroll
-        for (int tt = 0; tt < 2; ++tt)
+            for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                float v = s[tt][r];
-                if constexpr (SOFTCAP) {
-                    const float y = v * p.softcap_pre;
-                    const float e2 = __expf(2.f * y);
-                    v = p.softcap_post * (1.f - 2.f / (e2 + 1.f));
-                } else {
-                    v *= p.scale_log2;
+                for (int r = 0; r < 16; ++r) mloc = fmaxf(mloc, s[tt][r]);
+            mloc *= p.scale_log2;
+        } else {
+#pragma unroll
+            for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    float v = s[tt][r];
+                    if constexpr (SOFTCAP) {
+                        const float y = v * p.softcap_pre;
+                        const float e2 = __expf(2.f * y);
+                        v = p.softcap_post * (1.f - 2.f / (e2 + 1.f));
+                    } else {
+                        v *= p.scale_log2;
+                    }
+                    if (need_mask) {
+                        const int key = tile0 + tt * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
+                        v = (key >= klo_r && key <= khi_r) ? v : -INFINITY;
+                    }
+                    s[tt][r] = v;
+                    mloc = fmaxf(mloc, v);
                 }
-                if (need_mask) {
-                    const int key = tile0 + tt * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
-                    v = (key >= klo_r && key <= khi_r) ? v : -INFINITY;
-                }
-                s[tt][r] = v;
-                mloc = fmaxf(mloc, v);
-            }
+        }
         mloc = fmaxf(mloc, xor_shuffle(mloc, 32));
-        const float m_new = fmaxf(m_run, mloc);
-        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-        const float alpha = fast_exp2(m_run - m_use);
-        m_run = m_new;
+        // The accumulator rescale is skipped for the whole wave when no row of it saw a new maximum
+        // (most tiles once a row is a few hundred keys in).  m_run stays the exact running maximum,
+        // so the largest P of a row is exactly 1 as in the reference's golden.
+        const bool bump = mloc > m_run;   // false for fully hidden tiles
+        if (__any(bump)) {
+            const float m_new = bump ? mloc : m_run;
+            const float m_new_use = (m_new == -INFINITY) ? 0.f : m_new;
+            const float alpha = bump ? fast_exp2(m_run - m_new_use) : 1.f;
+            m_run = m_new;
+            l_run *= alpha;
+#pragma unroll
+            for (int t = 0; t < Cfg::kMT; ++t)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) o_acc[t][r] *= alpha;
+        }
+        const float m_use = (m_run == -INFINITY) ? 0.f : m_run;
         float psum = 0.f;
         u32x4_t pk[2][2];
 #pragma unroll
         for (int tt = 0; tt < 2; ++tt) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                s[tt][r] = fast_exp2(s[tt][r] - m_use);
+                const float e = raw_path ? __builtin_fmaf(s[tt][r], p.scale_log2, -m_use) : s[tt][r] - m_use;
+                s[tt][r] = fast_exp2(e);
                 psum += s[tt][r];
             }
 #pragma unroll
@@ -240,11 +264,7 @@ __global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) prefill_kernel(const 
 #pragma unroll
                 for (int u = 0; u < 4; ++u) pk[tt][ks][u] = pack2<T>(s[tt][8 * ks + 2 * u], s[tt][8 * ks + 2 * u + 1]);
         }
-        l_run = l_run * alpha + psum;
-#pragma unroll
-        for (int t = 0; t < Cfg::kMT; ++t)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) o_acc[t][r] *= alpha;
+        l_run += psum;
 
         // ---- O^T += V^T P^T, 16 keys per step; V rows read whole and transposed in registers
 #pragma unroll
