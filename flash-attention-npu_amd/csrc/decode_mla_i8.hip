@@ -11,9 +11,11 @@
 // unit list (same balanced partition as the bf16 decode kernel): every 32-key chunk is fetched
 // once as int8 with 16-byte loads, widened to the 16-bit type on the way into LDS (a code is an
 // integer of magnitude <= 127, exact in bf16 and fp16) and shared by the four waves, each of
-// which owns 16 heads: S^T = K Q^T with Q^T resident in registers, per-token scale folded into
-// the scores (K side) and into P (V side), O^T += V^T P^T with V rows read whole from the same
-// LDS tile and transposed in registers.
+// which owns 16 heads for the scores: S^T = K Q^T with Q^T resident in registers, per-token scale
+// folded into the scores (K side) and into P (V side).  For O^T += V^T P^T the waves trade places:
+// P of all 64 heads goes through LDS and every wave owns a 128-column slice of V for all heads,
+// so each transposed V operand (rows read whole from the same LDS tile, v_perm in registers)
+// feeds four MFMAs and is read from LDS once per workgroup instead of once per wave.
 #include "decode_common.h"
 
 namespace fa {
@@ -37,19 +39,27 @@ template <typename T> __device__ __forceinline__ void widen4(uint32_t w, uint32_
     hi = pack2<T>(f2, f3);
 }
 
+struct MlaShared {
+    __attribute__((aligned(16))) uint8_t k[2][kMlaTileBytes];   // widened key tiles
+    __attribute__((aligned(16))) float ks[2][kChunk];            // per-token scales, K side
+    __attribute__((aligned(16))) float vs[2][kChunk];            // per-token scales, V side
+    __attribute__((aligned(16))) u32x4_t pk[4][64];              // P^T operands of the four head groups
+    float alpha[kMlaHeadsPerUnit];                               // accumulator rescale per head
+    float m[kMlaHeadsPerUnit], l[kMlaHeadsPerUnit];              // final max / sum per head
+    int bump[4];                                                 // head group saw a new maximum
+};
+
 template <typename T>
 __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, const int half, const UnitRange &ur,
                                           const int range_lo, const int range_hi, const bool write_final,
-                                          const int64_t slot, uint8_t (*s_k)[kMlaTileBytes], float (*s_ks)[kChunk],
-                                          float (*s_vs)[kChunk]) {
+                                          const int64_t slot, MlaShared &sh) {
     constexpr int KSTEPS = kMlaDqk / 32;   // 18
-    constexpr int CT = kMlaDv / 16;        // 32 column tiles
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lq = lane >> 4;
     const int ln = lane & 15;
-    const int head = half * kMlaHeadsPerUnit + wave * 16 + ln;   // query head of this lane column
+    const int head = half * kMlaHeadsPerUnit + wave * 16 + ln;   // query head whose scores this lane column holds
     const int Lk = ur.Lk;
 
     // Q^T operand (seqlen_q == 1): lane (lq, ln) holds head `head`, elements t*32 + lq*8 .. +7
@@ -62,9 +72,12 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
     }
 
     float m_run = -INFINITY, l_run = 0.f;
-    float4_t o_acc[CT];
+    // o_acc[g][t]: head group g (16 heads), column tile t of this wave's 128-column slice
+    float4_t o_acc[4][8];
 #pragma unroll
-    for (int t = 0; t < CT; ++t) o_acc[t] = float4_t{0.f, 0.f, 0.f, 0.f};
+    for (int g = 0; g < 4; ++g)
+#pragma unroll
+        for (int t = 0; t < 8; ++t) o_acc[g][t] = float4_t{0.f, 0.f, 0.f, 0.f};
 
     const int8_t *kc = reinterpret_cast<const int8_t *>(p.k_cache);
     const int32_t *bt_row = p.block_table + (int64_t)b * p.bt_stride_b;
@@ -113,14 +126,14 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
                 widen4<T>(st[i][3], w[6], w[7]);
                 const u32x4_t a = {w[0], w[1], w[2], w[3]};
                 const u32x4_t bq = {w[4], w[5], w[6], w[7]};
-                uint8_t *dst = &s_k[buf][row * kMlaRowBytes + c16 * 32];
+                uint8_t *dst = &sh.k[buf][row * kMlaRowBytes + c16 * 32];
                 *reinterpret_cast<u32x4_t *>(dst) = a;
                 *reinterpret_cast<u32x4_t *>(dst + 16) = bq;
             }
         }
         if (tid < kChunk) {
-            s_ks[buf][tid] = st_ks;
-            s_vs[buf][tid] = st_vs;
+            sh.ks[buf][tid] = st_ks;
+            sh.vs[buf][tid] = st_vs;
         }
     };
 
@@ -137,24 +150,34 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
         __builtin_amdgcn_sched_barrier(0);
 
         // ---- S^T = K Q^T : two 16-key tiles x this wave's 16 heads
+        // operand reads run kPf k-steps ahead of the MFMAs that use them (one wave per SIMD here:
+        // nothing else hides the LDS latency)
+        constexpr int kPf = 4;
         float4_t s[2] = {float4_t{0.f, 0.f, 0.f, 0.f}, float4_t{0.f, 0.f, 0.f, 0.f}};
+        u32x4_t ka[KSTEPS][2];
+        auto read_k = [&](int t) {
 #pragma unroll
-        for (int t = 0; t < KSTEPS; ++t)
+            for (int tt = 0; tt < 2; ++tt)
+                ka[t][tt] = *reinterpret_cast<const u32x4_t *>(&sh.k[cur][(tt * 16 + ln) * kMlaRowBytes + (t * 4 + lq) * 16]);
+        };
 #pragma unroll
-            for (int tt = 0; tt < 2; ++tt) {
-                const u32x4_t a = *reinterpret_cast<const u32x4_t *>(
-                    &s_k[cur][(tt * 16 + ln) * kMlaRowBytes + (t * 4 + lq) * 16]);
-                s[tt] = mfma16<T>(a, qreg[t], s[tt]);
-            }
+        for (int t = 0; t < kPf; ++t) read_k(t);
+#pragma unroll
+        for (int t = 0; t < KSTEPS; ++t) {
+            if (t + kPf < KSTEPS) read_k(t + kPf);
+            s[0] = mfma16<T>(ka[t][0], qreg[t], s[0]);
+            s[1] = mfma16<T>(ka[t][1], qreg[t], s[1]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
 
-        // ---- softmax; register i of tile tt is key c*32 + tt*16 + lq*4 + i
+        // ---- softmax of this wave's heads; register i of tile tt is key c*32 + tt*16 + lq*4 + i
         const int key_base = c * kChunk + lq * 4;
         float x[8], vs[8];
         float mloc = -INFINITY;
 #pragma unroll
         for (int tt = 0; tt < 2; ++tt) {
-            const float4 ks4 = *reinterpret_cast<const float4 *>(&s_ks[cur][tt * 16 + lq * 4]);
-            const float4 vs4 = *reinterpret_cast<const float4 *>(&s_vs[cur][tt * 16 + lq * 4]);
+            const float4 ks4 = *reinterpret_cast<const float4 *>(&sh.ks[cur][tt * 16 + lq * 4]);
+            const float4 vs4 = *reinterpret_cast<const float4 *>(&sh.vs[cur][tt * 16 + lq * 4]);
             const float ksv[4] = {ks4.x, ks4.y, ks4.z, ks4.w};
             const float vsv[4] = {vs4.x, vs4.y, vs4.z, vs4.w};
 #pragma unroll
@@ -168,9 +191,10 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
             }
         }
         mloc = quad_rows_max(mloc);
-        const float m_new = fmaxf(m_run, mloc);
+        const bool bump = mloc > m_run;
+        const float m_new = bump ? mloc : m_run;
         const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-        const float alpha = fast_exp2(m_run - m_use);
+        const float alpha = bump ? fast_exp2(m_run - m_use) : 1.f;
         m_run = m_new;
         float psum = 0.f;
 #pragma unroll
@@ -185,82 +209,108 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
         pk[1] = pack2<T>(x[2], x[3]);
         pk[2] = pack2<T>(x[4], x[5]);
         pk[3] = pack2<T>(x[6], x[7]);
-#pragma unroll
-        for (int t = 0; t < CT; ++t) {
-            o_acc[t][0] *= alpha;
-            o_acc[t][1] *= alpha;
-            o_acc[t][2] *= alpha;
-            o_acc[t][3] *= alpha;
-        }
+        sh.pk[wave][lane] = pk;
+        if (lq == 0) sh.alpha[wave * 16 + ln] = alpha;
+        const int wave_bump = __any(bump) ? 1 : 0;
+        if (lane == 0) sh.bump[wave] = wave_bump;
+        __syncthreads();   // P, alpha of all 64 heads are in LDS
 
-        // ---- O^T += V^T P^T : 4 passes of 128 columns; lane (lq, ln) reads 8 key rows x 8 columns
+        // ---- O^T += V^T P^T on this wave's 128-column slice, all four head groups
+        u32x4_t pkg[4];
 #pragma unroll
-        for (int hh = 0; hh < 4; ++hh) {
-            u32x4_t vr[8];
+        for (int g = 0; g < 4; ++g) {
+            pkg[g] = sh.pk[g][lane];
+            if (sh.bump[g]) {
+                const float ag = sh.alpha[g * 16 + ln];
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const int row = (e >> 2) * 16 + lq * 4 + (e & 3);
-                vr[e] = *reinterpret_cast<const u32x4_t *>(&s_k[cur][row * kMlaRowBytes + (hh * 128 + ln * 8) * 2]);
-            }
-#pragma unroll
-            for (int w2 = 0; w2 < 4; ++w2) {
-                u32x4_t a_lo, a_hi;
-#pragma unroll
-                for (int u = 0; u < 4; ++u) {
-                    a_lo[u] = __builtin_amdgcn_perm(vr[2 * u + 1][w2], vr[2 * u][w2], 0x05040100u);
-                    a_hi[u] = __builtin_amdgcn_perm(vr[2 * u + 1][w2], vr[2 * u][w2], 0x07060302u);
+                for (int t = 0; t < 8; ++t) {
+                    o_acc[g][t][0] *= ag;
+                    o_acc[g][t][1] *= ag;
+                    o_acc[g][t][2] *= ag;
+                    o_acc[g][t][3] *= ag;
                 }
-                o_acc[hh * 8 + 2 * w2] = mfma16<T>(a_lo, pk, o_acc[hh * 8 + 2 * w2]);
-                o_acc[hh * 8 + 2 * w2 + 1] = mfma16<T>(a_hi, pk, o_acc[hh * 8 + 2 * w2 + 1]);
+            }
+        }
+        u32x4_t vr[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const int row = (e >> 2) * 16 + lq * 4 + (e & 3);
+            vr[e] = *reinterpret_cast<const u32x4_t *>(&sh.k[cur][row * kMlaRowBytes + (wave * 128 + ln * 8) * 2]);
+        }
+#pragma unroll
+        for (int w2 = 0; w2 < 4; ++w2) {
+            u32x4_t a_lo, a_hi;
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                a_lo[u] = __builtin_amdgcn_perm(vr[2 * u + 1][w2], vr[2 * u][w2], 0x05040100u);
+                a_hi[u] = __builtin_amdgcn_perm(vr[2 * u + 1][w2], vr[2 * u][w2], 0x07060302u);
+            }
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                o_acc[g][2 * w2] = mfma16<T>(a_lo, pkg[g], o_acc[g][2 * w2]);
+                o_acc[g][2 * w2 + 1] = mfma16<T>(a_hi, pkg[g], o_acc[g][2 * w2 + 1]);
             }
         }
 
+        // keep the widening of the prefetched tile behind the products: it waits for the loads
+        __builtin_amdgcn_sched_barrier(0);
         if (more) stash(cur ^ 1);
-        __syncthreads();
+        __syncthreads();   // next tile staged; P buffer free again
         cur ^= 1;
     }
 
-    // ---- write.  Register i of column tile t = hh*8 + w is column hh*128 + (lq*4 + i)*8 + w.
+    // ---- write.  The score-owning waves publish max and sum; every wave then stores its column
+    //      slice: register i of tile t of group g is column wave*128 + (lq*4 + i)*8 + t of head g*16 + ln.
     l_run = quad_rows_sum(l_run);
-    const float inv = (l_run > 0.f) ? 1.f / l_run : 0.f;
-    const int row = wave * 16 + ln;   // row of the unit (0..63)
-    if (write_final) {
-        uint16_t *dst = reinterpret_cast<uint16_t *>(p.out) + (int64_t)b * p.o_stride_b + (int64_t)head * p.o_stride_h;
+    if (lq == 0) {
+        sh.m[wave * 16 + ln] = m_run;
+        sh.l[wave * 16 + ln] = l_run;
+    }
+    __syncthreads();
 #pragma unroll
-        for (int hh = 0; hh < 4; ++hh)
+    for (int g = 0; g < 4; ++g) {
+        const int row = g * 16 + ln;   // row of the unit (0..63)
+        const int hd = half * kMlaHeadsPerUnit + row;
+        const float lg = sh.l[row];
+        const float inv = (lg > 0.f) ? 1.f / lg : 0.f;
+        if (write_final) {
+            uint16_t *dst = reinterpret_cast<uint16_t *>(p.out) + (int64_t)b * p.o_stride_b + (int64_t)hd * p.o_stride_h +
+                            wave * 128;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 u32x4_t o4;
 #pragma unroll
-                for (int u = 0; u < 4; ++u)
-                    o4[u] = pack2<T>(o_acc[hh * 8 + 2 * u][i] * inv, o_acc[hh * 8 + 2 * u + 1][i] * inv);
-                store16(dst + hh * 128 + (lq * 4 + i) * 8, o4);
+                for (int u = 0; u < 4; ++u) o4[u] = pack2<T>(o_acc[g][2 * u][i] * inv, o_acc[g][2 * u + 1][i] * inv);
+                store16(dst + (lq * 4 + i) * 8, o4);
             }
-        if (lq == 0) p.lse[(int64_t)b * p.nheads + head] = (l_run > 0.f) ? (m_run + fast_log2(l_run)) * kLn2 : INFINITY;
-    } else {
-        const int64_t srow = slot * p.rows + row;
-        float *dst = p.o_partial + srow * kMlaDv;
-#pragma unroll
-        for (int hh = 0; hh < 4; ++hh)
+        } else {
+            const int64_t srow = slot * p.rows + row;
+            float *dst = p.o_partial + srow * kMlaDv + wave * 128;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                float *d2 = dst + hh * 128 + (lq * 4 + i) * 8;
-                *reinterpret_cast<float4 *>(d2) = make_float4(o_acc[hh * 8 + 0][i] * inv, o_acc[hh * 8 + 1][i] * inv,
-                                                              o_acc[hh * 8 + 2][i] * inv, o_acc[hh * 8 + 3][i] * inv);
-                *reinterpret_cast<float4 *>(d2 + 4) = make_float4(o_acc[hh * 8 + 4][i] * inv, o_acc[hh * 8 + 5][i] * inv,
-                                                                  o_acc[hh * 8 + 6][i] * inv, o_acc[hh * 8 + 7][i] * inv);
+                float *d2 = dst + (lq * 4 + i) * 8;
+                *reinterpret_cast<float4 *>(d2) = make_float4(o_acc[g][0][i] * inv, o_acc[g][1][i] * inv, o_acc[g][2][i] * inv,
+                                                              o_acc[g][3][i] * inv);
+                *reinterpret_cast<float4 *>(d2 + 4) = make_float4(o_acc[g][4][i] * inv, o_acc[g][5][i] * inv,
+                                                                  o_acc[g][6][i] * inv, o_acc[g][7][i] * inv);
             }
-        if (lq == 0) p.lse_partial[srow] = (l_run > 0.f) ? m_run + fast_log2(l_run) : -INFINITY;
+        }
+    }
+    if (lq == 0) {
+        // this lane column's own head: LSE (final) or partial LSE
+        const int row = wave * 16 + ln;
+        if (write_final)
+            p.lse[(int64_t)b * p.nheads + head] = (l_run > 0.f) ? (m_run + fast_log2(l_run)) * kLn2 : INFINITY;
+        else
+            p.lse_partial[slot * p.rows + row] = (l_run > 0.f) ? m_run + fast_log2(l_run) : -INFINITY;
     }
     __syncthreads();   // the LDS tiles are reused by the next piece
 }
 
 template <typename T> __global__ void __launch_bounds__(256, 1) decode_mla_i8_kernel(const DecodeParams p) {
-    __shared__ __attribute__((aligned(16))) uint8_t s_k[2][kMlaTileBytes];
-    __shared__ __attribute__((aligned(16))) float s_ks[2][kChunk];
-    __shared__ __attribute__((aligned(16))) float s_vs[2][kChunk];
+    __shared__ MlaShared sh;
     balanced_driver<kMlaDv>(p, [&](int b, int half, const UnitRange &ur, int range_lo, int range_hi, bool whole, int64_t slot) {
-        mla_piece<T>(p, b, half, ur, range_lo, range_hi, whole, slot, s_k, s_ks, s_vs);
+        mla_piece<T>(p, b, half, ur, range_lo, range_hi, whole, slot, sh);
     });
 }
 

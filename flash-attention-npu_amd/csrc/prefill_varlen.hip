@@ -11,7 +11,7 @@
 //     double-buffered in LDS (K rows XOR-swizzled so MFMA operand reads are conflict free);
 //   * S^T = K Q^T and O^T = V^T P^T on the 32x32x16 MFMA: a query row is one lane column in both
 //     products, so the running max / sum / rescale never leave the lane (one xor-32 exchange);
-//   * V operands are read as whole rows and transposed in registers with v_perm;
+//   * V^T operands come straight from the transposing LDS read (ds_read_b64_tr_b16);
 //   * key tiles outside the causal / window range of the 128-row block are never loaded.
 #include "fa_device.h"
 #include "fa_kernels.h"
@@ -28,6 +28,8 @@ template <int D> struct PrefillCfg {
     static constexpr int kChunks = D / 8;         // 16-byte pieces per row
     static constexpr int kSwz = (kChunks >= 16) ? 15 : kChunks - 1;
     static constexpr int kTileBytes = kBN * D * 2;
+    static constexpr int kVRowBytes = D * 2 + 64;        // padded V rows: transposing reads spread over all banks
+    static constexpr int kVTileBytes = kBN * kVRowBytes;
     static constexpr int kPieces = kBN * kChunks / 256;  // 16-byte pieces per thread per tile
 };
 
@@ -35,7 +37,7 @@ template <typename T, int D, bool PAGED, bool SOFTCAP>
 __global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) prefill_kernel(const PrefillParams p) {
     using Cfg = PrefillCfg<D>;
     __shared__ __attribute__((aligned(16))) uint8_t s_k[2][Cfg::kTileBytes];
-    __shared__ __attribute__((aligned(16))) uint8_t s_v[2][Cfg::kTileBytes];
+    __shared__ __attribute__((aligned(16))) uint8_t s_v[2][Cfg::kVTileBytes];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -128,7 +130,25 @@ __global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) prefill_kernel(const 
     const int32_t *bt_row = PAGED ? p.block_table + (int64_t)b * p.bt_stride_b : nullptr;
 
     u32x4_t kst[Cfg::kPieces], vst[Cfg::kPieces];
+    // dense K/V: a thread's pieces of one tile are 256/kChunks rows apart, tiles are kBN rows apart,
+    // so one per-thread offset plus wave-uniform terms addresses every load of an interior tile
+    const int t_row = tid / Cfg::kChunks;
+    const int t_ch = tid % Cfg::kChunks;
+    const int64_t k_thread_off = (int64_t)(k0 + t_row) * p.k_stride_t + t_ch * 8;
+    const int64_t v_thread_off = (int64_t)(k0 + t_row) * p.v_stride_t + t_ch * 8;
     auto fetch_tile = [&](int kt) {
+        if constexpr (!PAGED) {
+            if (kt * kBN + kBN <= Sk) {
+                const uint16_t *kb = kbase + (int64_t)kt * kBN * p.k_stride_t;
+                const uint16_t *vb = vbase + (int64_t)kt * kBN * p.v_stride_t;
+#pragma unroll
+                for (int i = 0; i < Cfg::kPieces; ++i) {
+                    kst[i] = load16(kb + (int64_t)i * (256 / Cfg::kChunks) * p.k_stride_t + k_thread_off);
+                    vst[i] = load16(vb + (int64_t)i * (256 / Cfg::kChunks) * p.v_stride_t + v_thread_off);
+                }
+                return;
+            }
+        }
 #pragma unroll
         for (int i = 0; i < Cfg::kPieces; ++i) {
             const int piece = tid + 256 * i;
@@ -158,7 +178,7 @@ __global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) prefill_kernel(const 
             const int row = piece / Cfg::kChunks;
             const int ch = piece % Cfg::kChunks;
             *reinterpret_cast<u32x4_t *>(&s_k[buf][row * (D * 2) + ((ch ^ (row & Cfg::kSwz)) << 4)]) = kst[i];
-            *reinterpret_cast<u32x4_t *>(&s_v[buf][row * (D * 2) + (ch << 4)]) = vst[i];
+            *reinterpret_cast<u32x4_t *>(&s_v[buf][row * Cfg::kVRowBytes + (ch << 4)]) = vst[i];
         }
     };
 
@@ -187,20 +207,32 @@ __global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) prefill_kernel(const 
         for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
             for (int r = 0; r < 16; ++r) s[tt][r] = 0.f;
-#pragma unroll
-        for (int t = 0; t < Cfg::kKSteps; ++t)
+        // operand reads run kPf k-steps ahead of the MFMAs that use them
+        constexpr int kPf = 2;
+        u32x4_t ka[Cfg::kKSteps][2];
+        auto read_k = [&](int t) {
 #pragma unroll
             for (int tt = 0; tt < 2; ++tt) {
                 const int row = tt * 32 + ln;
-                const u32x4_t a = *reinterpret_cast<const u32x4_t *>(
+                ka[t][tt] = *reinterpret_cast<const u32x4_t *>(
                     &s_k[cur][row * (D * 2) + (((t * 2 + lh) ^ (row & Cfg::kSwz)) << 4)]);
-                s[tt] = mfma32<T>(a, qreg[t], s[tt]);
             }
+        };
+#pragma unroll
+        for (int t = 0; t < kPf; ++t) read_k(t);
+#pragma unroll
+        for (int t = 0; t < Cfg::kKSteps; ++t) {
+            if (t + kPf < Cfg::kKSteps) read_k(t + kPf);
+            s[0] = mfma32<T>(ka[t][0], qreg[t], s[0]);
+            s[1] = mfma32<T>(ka[t][1], qreg[t], s[1]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
 
         // ---- online softmax; lane column = query row, register r of half tt = key
         //      kt*64 + tt*32 + 8*(r/4) + 4*lh + r%4
         const int tile0 = kt * kBN;
-        const bool need_mask = (tile0 < wave_klo_max) || (tile0 + kBN - 1 > wave_khi_min);
+        // wave-uniform by construction; made scalar so the two softmax paths stay separate branches
+        const bool need_mask = __builtin_amdgcn_readfirstlane((tile0 < wave_klo_max) || (tile0 + kBN - 1 > wave_khi_min));
         // Fast path (no softcap, no element masks, positive scale): the maximum is taken on the raw
         // scores and the scale rides in the exponent's fused multiply-add.
         const bool raw_path = !SOFTCAP && !need_mask && p.scale_log2 > 0.f;
@@ -251,14 +283,21 @@ __global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) prefill_kernel(const 
         const float m_use = (m_run == -INFINITY) ? 0.f : m_run;
         float psum = 0.f;
         u32x4_t pk[2][2];
+        if (raw_path) {
+#pragma unroll
+            for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) s[tt][r] = fast_exp2(__builtin_fmaf(s[tt][r], p.scale_log2, -m_use));
+        } else {
+#pragma unroll
+            for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) s[tt][r] = fast_exp2(s[tt][r] - m_use);
+        }
 #pragma unroll
         for (int tt = 0; tt < 2; ++tt) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const float e = raw_path ? __builtin_fmaf(s[tt][r], p.scale_log2, -m_use) : s[tt][r] - m_use;
-                s[tt][r] = fast_exp2(e);
-                psum += s[tt][r];
-            }
+            for (int r = 0; r < 16; ++r) psum += s[tt][r];
 #pragma unroll
             for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
@@ -266,37 +305,31 @@ __global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) prefill_kernel(const 
         }
         l_run += psum;
 
-        // ---- O^T += V^T P^T, 16 keys per step; V rows read whole and transposed in registers
+        // ---- O^T += V^T P^T, 16 keys per step.  The V^T operand comes from the transposing LDS read
+        //      (ds_read_b64_tr_b16): in every 16-lane group, lane s points at 4 columns of key row
+        //      s/4 and receives column s (of the group's 16) for the group's 4 key rows.  Column tile
+        //      t is V columns t*32 .. t*32+31 in lane order.
+        typedef short v4s_t __attribute__((ext_vector_type(4)));
+        const int tr_row = 4 * lh + ((lane & 15) >> 2);
+        const int tr_col = ((lane >> 4) & 1) * 16 + (lane & 3) * 4;
 #pragma unroll
         for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
             for (int ks = 0; ks < 2; ++ks) {
-                uint32_t vr[8][Cfg::kCPL / 2 > 0 ? Cfg::kCPL / 2 : 1];
+                u32x4_t va[Cfg::kMT];
 #pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const int row = tt * 32 + 16 * ks + 8 * (e >> 2) + 4 * lh + (e & 3);
-                    const uint8_t *src = &s_v[cur][row * (D * 2) + ln * (Cfg::kCPL * 2)];
-                    if constexpr (Cfg::kCPL == 8) {
-                        const u32x4_t t4 = *reinterpret_cast<const u32x4_t *>(src);
-                        vr[e][0] = t4[0]; vr[e][1] = t4[1]; vr[e][2] = t4[2]; vr[e][3] = t4[3];
-                    } else if constexpr (Cfg::kCPL == 4) {
-                        const uint2 t2 = *reinterpret_cast<const uint2 *>(src);
-                        vr[e][0] = t2.x; vr[e][1] = t2.y;
-                    } else {
-                        vr[e][0] = *reinterpret_cast<const uint32_t *>(src);
+                for (int t = 0; t < Cfg::kMT; ++t)
+#pragma unroll
+                    for (int hv = 0; hv < 2; ++hv) {
+                        const int row = tt * 32 + 16 * ks + 8 * hv + tr_row;
+                        const v4s_t r4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                            (__attribute__((address_space(3))) v4s_t *)(&s_v[cur][row * Cfg::kVRowBytes + (t * 32 + tr_col) * 2]));
+                        const uint2 r2 = __builtin_bit_cast(uint2, r4);
+                        va[t][2 * hv] = r2.x;
+                        va[t][2 * hv + 1] = r2.y;
                     }
-                }
 #pragma unroll
-                for (int w2 = 0; w2 < Cfg::kCPL / 2; ++w2) {
-                    u32x4_t a_lo, a_hi;
-#pragma unroll
-                    for (int u = 0; u < 4; ++u) {
-                        a_lo[u] = __builtin_amdgcn_perm(vr[2 * u + 1][w2], vr[2 * u][w2], 0x05040100u);
-                        a_hi[u] = __builtin_amdgcn_perm(vr[2 * u + 1][w2], vr[2 * u][w2], 0x07060302u);
-                    }
-                    o_acc[2 * w2] = mfma32<T>(a_lo, pk[tt][ks], o_acc[2 * w2]);
-                    o_acc[2 * w2 + 1] = mfma32<T>(a_hi, pk[tt][ks], o_acc[2 * w2 + 1]);
-                }
+                for (int t = 0; t < Cfg::kMT; ++t) o_acc[t] = mfma32<T>(va[t], pk[tt][ks], o_acc[t]);
             }
 
         if (more) stash_tile(cur ^ 1);
@@ -305,30 +338,20 @@ __global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) prefill_kernel(const 
     }
 
     // ---- epilogue: O^T / l, store.  Register r of column tile t is V column
-    //      (8*(r/4) + 4*lh + r%4) * kCPL + t of query row ln.
+    //      t*32 + 8*(r/4) + 4*lh + r%4 of query row ln: four consecutive columns per (t, r/4).
     l_run += xor_shuffle(l_run, 32);
     const float inv = (l_run > 0.f) ? 1.f / l_run : 0.f;
     if (row_ok) {
         uint16_t *dst = ob + (int64_t)(q0 + my_row) * p.o_stride_t;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int col = (8 * (r >> 2) + 4 * lh + (r & 3)) * Cfg::kCPL;
-            if constexpr (Cfg::kCPL == 4) {
+        for (int t = 0; t < Cfg::kMT; ++t)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
                 uint2 o2;
-                o2.x = pack2<T>(o_acc[0][r] * inv, o_acc[1][r] * inv);
-                o2.y = pack2<T>(o_acc[2][r] * inv, o_acc[3][r] * inv);
-                *reinterpret_cast<uint2 *>(dst + col) = o2;
-            } else if constexpr (Cfg::kCPL == 8) {
-                u32x4_t o4;
-                o4[0] = pack2<T>(o_acc[0][r] * inv, o_acc[1][r] * inv);
-                o4[1] = pack2<T>(o_acc[2][r] * inv, o_acc[3][r] * inv);
-                o4[2] = pack2<T>(o_acc[4][r] * inv, o_acc[5][r] * inv);
-                o4[3] = pack2<T>(o_acc[6][r] * inv, o_acc[7][r] * inv);
-                store16(dst + col, o4);
-            } else {
-                *reinterpret_cast<uint32_t *>(dst + col) = pack2<T>(o_acc[0][r] * inv, o_acc[1][r] * inv);
+                o2.x = pack2<T>(o_acc[t][4 * j] * inv, o_acc[t][4 * j + 1] * inv);
+                o2.y = pack2<T>(o_acc[t][4 * j + 2] * inv, o_acc[t][4 * j + 3] * inv);
+                *reinterpret_cast<uint2 *>(dst + t * 32 + 8 * j + 4 * lh) = o2;
             }
-        }
         if (lh == 0) lse_b[q0 + my_row] = (l_run > 0.f) ? (m_run + fast_log2(l_run)) * kLn2 : INFINITY;
     }
 }
