@@ -87,13 +87,16 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
     // ---- staging: int8 rows -> registers -> widened LDS tile --------------------------------
     u32x4_t st[kMlaRounds];
     float st_ks = 0.f, st_vs = 0.f;
-    auto fetch = [&](int c) {
-        const int key0 = c * kChunk;
-        int page = key0 / p.page_size;
+    // page id of chunk c, fetched one chunk before the loads that need it
+    auto fetch_blk = [&](int c) -> int {
+        if (c >= c_end) return 0;
+        int page = (c * kChunk) / p.page_size;
         page = min(page, p.max_blocks - 1);
-        int blk = bt_row[page];
-        blk = min(max(blk, 0), p.num_blocks - 1);
-        const int inpage0 = key0 - page * p.page_size;
+        return min(max(bt_row[page], 0), p.num_blocks - 1);
+    };
+    auto fetch = [&](int c, int blk) {
+        const int key0 = c * kChunk;
+        const int inpage0 = key0 % p.page_size;
         const int last = Lk - 1 - key0;
         const int8_t *base = kc + (int64_t)blk * p.k_stride_block;
 #pragma unroll
@@ -137,8 +140,10 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
         }
     };
 
+    int blk_next = fetch_blk(c_begin);
     if (c_begin < c_end) {
-        fetch(c_begin);
+        fetch(c_begin, blk_next);
+        blk_next = fetch_blk(c_begin + 1);
         stash(0);
     }
     __syncthreads();
@@ -146,7 +151,8 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
     int cur = 0;
     for (int c = c_begin; c < c_end; ++c) {
         const bool more = c + 1 < c_end;
-        if (more) fetch(c + 1);
+        if (more) fetch(c + 1, blk_next);
+        blk_next = fetch_blk(c + 2);
         __builtin_amdgcn_sched_barrier(0);
 
         // ---- S^T = K Q^T : two 16-key tiles x this wave's 16 heads

@@ -26,7 +26,9 @@ template <int D> struct PrefillCfg {
     static constexpr int kMT = D / 32;            // 32-column tiles of O^T
     static constexpr int kCPL = D / 32;           // V columns a lane owns per key row
     static constexpr int kChunks = D / 8;         // 16-byte pieces per row
-    static constexpr int kSwz = (kChunks >= 16) ? 15 : kChunks - 1;
+    // XOR swizzle of the 16-byte pieces of a K row; the mask must not see the row step of the
+    // tile stores (256 / kChunks rows), so it is 7 for D = 256
+    static constexpr int kSwz = (kChunks == 16) ? 15 : 7;
     static constexpr int kTileBytes = kBN * D * 2;
     static constexpr int kVRowBytes = D * 2 + 64;        // padded V rows: transposing reads spread over all banks
     static constexpr int kVTileBytes = kBN * kVRowBytes;
@@ -130,30 +132,33 @@ __global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) prefill_kernel(const 
     const int32_t *bt_row = PAGED ? p.block_table + (int64_t)b * p.bt_stride_b : nullptr;
 
     u32x4_t kst[Cfg::kPieces], vst[Cfg::kPieces];
-    // dense K/V: a thread's pieces of one tile are 256/kChunks rows apart, tiles are kBN rows apart,
-    // so one per-thread offset plus wave-uniform terms addresses every load of an interior tile
+    // A thread's pieces of one tile sit 256/kChunks rows apart and tiles kBN rows apart, so one small
+    // per-thread byte offset plus wave-uniform (scalar) terms addresses every load of an interior
+    // tile of dense K/V, and one per-thread LDS offset plus constants every store.
+    constexpr int kRowsPerPass = 256 / Cfg::kChunks;
     const int t_row = tid / Cfg::kChunks;
     const int t_ch = tid % Cfg::kChunks;
-    const int64_t k_thread_off = (int64_t)(k0 + t_row) * p.k_stride_t + t_ch * 8;
-    const int64_t v_thread_off = (int64_t)(k0 + t_row) * p.v_stride_t + t_ch * 8;
+    const uint32_t k_thread_off = (uint32_t)t_row * (uint32_t)p.k_stride_t * 2u + t_ch * 16;
+    const uint32_t v_thread_off = (uint32_t)t_row * (uint32_t)p.v_stride_t * 2u + t_ch * 16;
+    const uint32_t k_lds_off = t_row * (D * 2) + ((t_ch ^ (t_row & Cfg::kSwz)) << 4);   // row + 16*i keeps row & 15
+    const uint32_t v_lds_off = t_row * Cfg::kVRowBytes + (t_ch << 4);
+    static_assert(kRowsPerPass % (Cfg::kSwz + 1) == 0 && Cfg::kSwz < Cfg::kChunks, "swizzle must survive the row step");
     auto fetch_tile = [&](int kt) {
         if constexpr (!PAGED) {
             if (kt * kBN + kBN <= Sk) {
-                const uint16_t *kb = kbase + (int64_t)kt * kBN * p.k_stride_t;
-                const uint16_t *vb = vbase + (int64_t)kt * kBN * p.v_stride_t;
+                const uint8_t *kb = reinterpret_cast<const uint8_t *>(kbase) + (int64_t)(k0 + kt * kBN) * p.k_stride_t * 2;
+                const uint8_t *vb = reinterpret_cast<const uint8_t *>(vbase) + (int64_t)(k0 + kt * kBN) * p.v_stride_t * 2;
 #pragma unroll
                 for (int i = 0; i < Cfg::kPieces; ++i) {
-                    kst[i] = load16(kb + (int64_t)i * (256 / Cfg::kChunks) * p.k_stride_t + k_thread_off);
-                    vst[i] = load16(vb + (int64_t)i * (256 / Cfg::kChunks) * p.v_stride_t + v_thread_off);
+                    kst[i] = load16(kb + (int64_t)i * kRowsPerPass * p.k_stride_t * 2 + k_thread_off);
+                    vst[i] = load16(vb + (int64_t)i * kRowsPerPass * p.v_stride_t * 2 + v_thread_off);
                 }
                 return;
             }
         }
 #pragma unroll
         for (int i = 0; i < Cfg::kPieces; ++i) {
-            const int piece = tid + 256 * i;
-            const int row = piece / Cfg::kChunks;
-            const int ch = piece % Cfg::kChunks;
+            const int row = t_row + kRowsPerPass * i;
             const int key = min(kt * kBN + row, Sk - 1);
             int64_t koff, voff;
             if constexpr (PAGED) {
@@ -167,18 +172,15 @@ __global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) prefill_kernel(const 
                 koff = (int64_t)(k0 + key) * p.k_stride_t;
                 voff = (int64_t)(k0 + key) * p.v_stride_t;
             }
-            kst[i] = load16(kbase + koff + ch * 8);
-            vst[i] = load16(vbase + voff + ch * 8);
+            kst[i] = load16(kbase + koff + t_ch * 8);
+            vst[i] = load16(vbase + voff + t_ch * 8);
         }
     };
     auto stash_tile = [&](int buf) {
 #pragma unroll
         for (int i = 0; i < Cfg::kPieces; ++i) {
-            const int piece = tid + 256 * i;
-            const int row = piece / Cfg::kChunks;
-            const int ch = piece % Cfg::kChunks;
-            *reinterpret_cast<u32x4_t *>(&s_k[buf][row * (D * 2) + ((ch ^ (row & Cfg::kSwz)) << 4)]) = kst[i];
-            *reinterpret_cast<u32x4_t *>(&s_v[buf][row * Cfg::kVRowBytes + (ch << 4)]) = vst[i];
+            *reinterpret_cast<u32x4_t *>(&s_k[buf][k_lds_off + i * kRowsPerPass * (D * 2)]) = kst[i];
+            *reinterpret_cast<u32x4_t *>(&s_v[buf][v_lds_off + i * kRowsPerPass * Cfg::kVRowBytes]) = vst[i];
         }
     };
 
