@@ -54,8 +54,8 @@ __device__ __forceinline__ UnitRange unit_range(const DecodeParams &p, int b, in
 }
 
 // exclusive prefix of per-row chunk counts over 256 equal segments of the batch: s_pref[t] =
-// chunks of rows [0, t*seg); s_pref[256] = total.  All threads of a 256-thread block must call.
-// Returns whether some batch row has no visible key at all.
+// chunks of rows [0, t*seg); s_pref[256] = total.  All threads of the block must call (256 or more
+// threads; the first 256 do the work).  Returns whether some batch row has no visible key at all.
 __device__ __forceinline__ bool batch_chunk_prefix(const DecodeParams &p, int *s_pref, int seg, int M) {
     __shared__ int s_wave[4];
     const int tid = threadIdx.x;
@@ -72,11 +72,13 @@ __device__ __forceinline__ bool batch_chunk_prefix(const DecodeParams &p, int *s
         const int v = __shfl_up(inc, d, 64);
         if ((tid & 63) >= d) inc += v;
     }
-    if ((tid & 63) == 63) s_wave[tid >> 6] = inc;
+    if ((tid & 63) == 63 && tid < 256) s_wave[tid >> 6] = inc;
     const bool any_empty = __syncthreads_or(empty_row ? 1 : 0) != 0;
-    int base = 0;
-    for (int w = 0; w < (tid >> 6); ++w) base += s_wave[w];
-    s_pref[tid + 1] = base + inc;
+    if (tid < 256) {
+        int base = 0;
+        for (int w = 0; w < (tid >> 6); ++w) base += s_wave[w];
+        s_pref[tid + 1] = base + inc;
+    }
     if (tid == 0) s_pref[0] = 0;
     __syncthreads();
     return any_empty;

@@ -7,27 +7,34 @@
 // the same as the bf16 decode kernel's (mha_fwd_kvcache.cpp:632-969 in the reference) applied to
 // K^ = code * scale[token].
 //
-// A work unit is (batch row, 64-head half).  The 256-thread workgroup streams its share of the
+// A work unit is (batch row, 64-head half).  The 512-thread workgroup (two waves per SIMD, so one
+// wave's matrix products cover the other's conversions and LDS waits) streams its share of the
 // unit list (same balanced partition as the bf16 decode kernel): every 32-key chunk is fetched
-// once as int8 with 16-byte loads, widened to the 16-bit type on the way into LDS (a code is an
-// integer of magnitude <= 127, exact in bf16 and fp16) and shared by the four waves, each of
-// which owns 16 heads for the scores: S^T = K Q^T with Q^T resident in registers, per-token scale
-// folded into the scores (K side) and into P (V side).  For O^T += V^T P^T the waves trade places:
-// P of all 64 heads goes through LDS and every wave owns a 128-column slice of V for all heads,
-// so each transposed V operand (rows read whole from the same LDS tile, v_perm in registers)
-// feeds four MFMAs and is read from LDS once per workgroup instead of once per wave.
+// once as int8 with 12-byte loads, widened to the 16-bit type on the way into LDS (a code is an
+// integer of magnitude <= 127, exact in bf16 and fp16) and shared by the eight waves.
+//   scores : wave (g, t) owns head group g (16 heads, Q^T resident in registers) and the 16-key
+//            tile t of the chunk: S^T = K Q^T, per-token scale folded into the scores; the chunk
+//            maximum of a head group is exchanged between its two waves through LDS;
+//   output : the waves trade places: P of all 64 heads goes through LDS and every wave owns a
+//            64-column slice of V for all heads, so each transposed V operand (rows read whole
+//            from the same LDS tile, v_perm in registers) feeds four MFMAs; the V side of the
+//            dequantisation is folded into P.
+// Two barriers per chunk; the widening of the next chunk sits between them.
 #include "decode_common.h"
 
 namespace fa {
 
 constexpr int kMlaDqk = 576;
 constexpr int kMlaDv = 512;
+constexpr int kMlaThreads = 512;
 constexpr int kMlaRowBytes = kMlaDqk * 2 + 16;           // padded LDS row: conflict-free operand reads
 constexpr int kMlaTileBytes = kChunk * kMlaRowBytes;     // 37376
-constexpr int kMlaPiecesPerRow = kMlaDqk / 16;           // 36 16-byte int8 pieces per key
-constexpr int kMlaPieces = kChunk * kMlaPiecesPerRow;    // 1152 per chunk
-constexpr int kMlaRounds = (kMlaPieces + 255) / 256;     // 5 (last one half full)
+constexpr int kMlaPiecesPerRow = kMlaDqk / 12;           // 48 12-byte int8 pieces per key
+constexpr int kMlaRounds = kChunk * kMlaPiecesPerRow / kMlaThreads;   // 3 pieces per thread per chunk
 constexpr int kMlaHeadsPerUnit = 64;
+static_assert(kChunk * kMlaPiecesPerRow == kMlaRounds * kMlaThreads, "chunk must split evenly over the threads");
+
+struct __attribute__((aligned(4))) MlaCodes12 { uint32_t w[3]; };
 
 // 4 signed bytes -> two dwords of 16-bit floats (lo = bytes 0,1 ; hi = bytes 2,3)
 template <typename T> __device__ __forceinline__ void widen4(uint32_t w, uint32_t &lo, uint32_t &hi) {
@@ -43,10 +50,12 @@ struct MlaShared {
     __attribute__((aligned(16))) uint8_t k[2][kMlaTileBytes];   // widened key tiles
     __attribute__((aligned(16))) float ks[2][kChunk];            // per-token scales, K side
     __attribute__((aligned(16))) float vs[2][kChunk];            // per-token scales, V side
-    __attribute__((aligned(16))) u32x4_t pk[4][64];              // P^T operands of the four head groups
-    float alpha[kMlaHeadsPerUnit];                               // accumulator rescale per head
-    float m[kMlaHeadsPerUnit], l[kMlaHeadsPerUnit];              // final max / sum per head
-    int bump[4];                                                 // head group saw a new maximum
+    __attribute__((aligned(16))) uint2 pk[4][64][2];             // P^T operands of the four head groups, by key tile
+    // per head, indexed [head group][head in group] so the group is a constant address offset
+    float mx[2][4][16];                                          // chunk maximum per key tile
+    float alpha[4][16];                                          // accumulator rescale
+    float m[4][16], l[2][4][16];                                 // final max, sum per key tile
+    __attribute__((aligned(4))) uint8_t bump[4];                 // head group saw a new maximum
 };
 
 template <typename T>
@@ -57,9 +66,11 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int g = wave & 3;    // head group of the score phase
+    const int kt = wave >> 2;  // 16-key tile of the score phase
     const int lq = lane >> 4;
     const int ln = lane & 15;
-    const int head = half * kMlaHeadsPerUnit + wave * 16 + ln;   // query head whose scores this lane column holds
+    const int head = half * kMlaHeadsPerUnit + g * 16 + ln;   // query head whose scores this lane column holds
     const int Lk = ur.Lk;
 
     // Q^T operand (seqlen_q == 1): lane (lq, ln) holds head `head`, elements t*32 + lq*8 .. +7
@@ -72,131 +83,135 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
     }
 
     float m_run = -INFINITY, l_run = 0.f;
-    // o_acc[g][t]: head group g (16 heads), column tile t of this wave's 128-column slice
-    float4_t o_acc[4][8];
+    // o_acc[hg][t]: head group hg (16 heads), column tile t of this wave's 64-column slice
+    float4_t o_acc[4][4];
 #pragma unroll
-    for (int g = 0; g < 4; ++g)
+    for (int hg = 0; hg < 4; ++hg)
 #pragma unroll
-        for (int t = 0; t < 8; ++t) o_acc[g][t] = float4_t{0.f, 0.f, 0.f, 0.f};
+        for (int t = 0; t < 4; ++t) o_acc[hg][t] = float4_t{0.f, 0.f, 0.f, 0.f};
 
     const int8_t *kc = reinterpret_cast<const int8_t *>(p.k_cache);
     const int32_t *bt_row = p.block_table + (int64_t)b * p.bt_stride_b;
     const int c_begin = range_lo / kChunk;
     const int c_end = (range_hi + kChunk - 1) / kChunk;
 
-    // ---- staging: int8 rows -> registers -> widened LDS tile --------------------------------
-    u32x4_t st[kMlaRounds];
-    float st_ks = 0.f, st_vs = 0.f;
-    // page id of chunk c, fetched one chunk before the loads that need it
+    // ---- staging: int8 rows -> registers -> widened LDS tile.  Loads run two chunks ahead of the
+    //      products (register sets st[0], st[1] by chunk parity within the piece): one chunk of
+    //      arithmetic is shorter than a trip to memory.
+    MlaCodes12 st[2][kMlaRounds];
+    float st_ks[2] = {0.f, 0.f}, st_vs[2] = {0.f, 0.f};
     auto fetch_blk = [&](int c) -> int {
         if (c >= c_end) return 0;
         int page = (c * kChunk) / p.page_size;
         page = min(page, p.max_blocks - 1);
         return min(max(bt_row[page], 0), p.num_blocks - 1);
     };
-    auto fetch = [&](int c, int blk) {
+    // thread -> (key row, 12-byte column) of the chunk: 16 threads per row, three pieces 192 bytes
+    // apart each, so one address per chunk serves all three loads and one LDS address all stores
+    static_assert(kMlaThreads / 16 == kChunk && kMlaRounds * 16 == kMlaPiecesPerRow, "thread map of the staging");
+    // (the thread index comes in as an argument: the chunk loop passes a copy the compiler cannot
+    //  see through, so these few address terms are recomputed per chunk instead of held in registers)
+    auto fetch = [&](int c, int blk, int set, int th) {
+        const int t_row = th >> 4;
+        const int t_sub = th & 15;
         const int key0 = c * kChunk;
         const int inpage0 = key0 % p.page_size;
         const int last = Lk - 1 - key0;
-        const int8_t *base = kc + (int64_t)blk * p.k_stride_block;
+        // wave-uniform 64-bit base + 32-bit per-thread offset
+        const int8_t *src = kc + (int64_t)blk * p.k_stride_block + (int64_t)inpage0 * p.k_stride_row;
+        const uint32_t voff = (uint32_t)min(t_row, last) * (uint32_t)p.k_stride_row + t_sub * 12;
 #pragma unroll
-        for (int i = 0; i < kMlaRounds; ++i) {
-            const int piece = tid + 256 * i;
-            if (piece < kMlaPieces) {
-                const int row = min(piece / kMlaPiecesPerRow, last);
-                const int c16 = piece % kMlaPiecesPerRow;
-                st[i] = load16(base + (int64_t)(inpage0 + row) * p.k_stride_row + c16 * 16);
-            }
-        }
-        if (tid < kChunk) {
-            const int row = min(tid, last);
-            const int64_t so = (int64_t)blk * p.ks_stride_block + (int64_t)(inpage0 + row) * p.ks_stride_row;
-            st_ks = p.k_scale[so];
-            st_vs = p.v_scale[so];
-        }
+        for (int i = 0; i < kMlaRounds; ++i) st[set][i] = *reinterpret_cast<const MlaCodes12 *>(src + voff + i * 192);
+        // every thread loads a scale (no branch around a load: the waits stay counted in order)
+        const int64_t so = (int64_t)blk * p.ks_stride_block + (int64_t)inpage0 * p.ks_stride_row;
+        const uint32_t soff = (uint32_t)min(th & (kChunk - 1), last) * (uint32_t)p.ks_stride_row;
+        st_ks[set] = (p.k_scale + so)[soff];
+        st_vs[set] = (p.v_scale + so)[soff];
     };
-    auto stash = [&](int buf) {
+    auto stash = [&](int buf, int set, int th) {
+        uint8_t *dst = &sh.k[buf][(th >> 4) * kMlaRowBytes + (th & 15) * 24];
 #pragma unroll
         for (int i = 0; i < kMlaRounds; ++i) {
-            const int piece = tid + 256 * i;
-            if (piece < kMlaPieces) {
-                const int row = piece / kMlaPiecesPerRow;
-                const int c16 = piece % kMlaPiecesPerRow;
-                uint32_t w[8];
-                widen4<T>(st[i][0], w[0], w[1]);
-                widen4<T>(st[i][1], w[2], w[3]);
-                widen4<T>(st[i][2], w[4], w[5]);
-                widen4<T>(st[i][3], w[6], w[7]);
-                const u32x4_t a = {w[0], w[1], w[2], w[3]};
-                const u32x4_t bq = {w[4], w[5], w[6], w[7]};
-                uint8_t *dst = &sh.k[buf][row * kMlaRowBytes + c16 * 32];
-                *reinterpret_cast<u32x4_t *>(dst) = a;
-                *reinterpret_cast<u32x4_t *>(dst + 16) = bq;
+#pragma unroll
+            for (int j = 0; j < 3; ++j) {
+                uint2 w;
+                widen4<T>(st[set][i].w[j], w.x, w.y);
+                *reinterpret_cast<uint2 *>(dst + i * 384 + j * 8) = w;
             }
         }
-        if (tid < kChunk) {
-            sh.ks[buf][tid] = st_ks;
-            sh.vs[buf][tid] = st_vs;
+        if (th < kChunk) {
+            sh.ks[buf][th] = st_ks[set];
+            sh.vs[buf][th] = st_vs[set];
         }
     };
 
-    int blk_next = fetch_blk(c_begin);
+    // page ids are loaded one step before the loads that use them and always ahead of that step's
+    // tile loads, so waiting for a page id never waits for younger tile loads
+    int blk_next = 0;
     if (c_begin < c_end) {
-        fetch(c_begin, blk_next);
+        fetch(c_begin, fetch_blk(c_begin), 0, tid);
         blk_next = fetch_blk(c_begin + 1);
-        stash(0);
+        stash(0, 0, tid);
+        const int blk2 = fetch_blk(c_begin + 2);
+        if (c_begin + 1 < c_end) fetch(c_begin + 1, blk_next, 1, tid);
+        blk_next = blk2;
     }
     __syncthreads();
 
-    int cur = 0;
-    for (int c = c_begin; c < c_end; ++c) {
+    // one chunk; `set` = parity of the chunk within the piece (compile-time in the unrolled loop)
+    auto chunk_step = [&](const int c, const int set) {
+        const int cur = set;
         const bool more = c + 1 < c_end;
-        if (more) fetch(c + 1, blk_next);
-        blk_next = fetch_blk(c + 2);
+        // lane-derived LDS addresses are recomputed in every step (a few adds) instead of being kept
+        // in registers across the whole piece, which the register budget cannot afford
+        int tid_here = tid;
+        asm volatile("" : "+v"(tid_here));
+        const int lane = tid_here & 63;
+        const int lq = lane >> 4;
+        const int ln = lane & 15;
+        {
+            const int blk3 = fetch_blk(c + 3);
+            if (c + 2 < c_end) fetch(c + 2, blk_next, set, tid_here);
+            blk_next = blk3;
+        }
         __builtin_amdgcn_sched_barrier(0);
 
-        // ---- S^T = K Q^T : two 16-key tiles x this wave's 16 heads
-        // operand reads run kPf k-steps ahead of the MFMAs that use them (one wave per SIMD here:
-        // nothing else hides the LDS latency)
+        // ---- S^T = K Q^T : this wave's 16-key tile x 16 heads; operand reads run kPf k-steps
+        //      ahead of the MFMAs that use them, two accumulators break the dependency chain
         constexpr int kPf = 4;
-        float4_t s[2] = {float4_t{0.f, 0.f, 0.f, 0.f}, float4_t{0.f, 0.f, 0.f, 0.f}};
-        u32x4_t ka[KSTEPS][2];
-        auto read_k = [&](int t) {
+        float4_t s2[2] = {float4_t{0.f, 0.f, 0.f, 0.f}, float4_t{0.f, 0.f, 0.f, 0.f}};
+        u32x4_t ka[KSTEPS];
+        const uint8_t *k_rd = &sh.k[cur][(kt * 16 + ln) * kMlaRowBytes + lq * 16];
 #pragma unroll
-            for (int tt = 0; tt < 2; ++tt)
-                ka[t][tt] = *reinterpret_cast<const u32x4_t *>(&sh.k[cur][(tt * 16 + ln) * kMlaRowBytes + (t * 4 + lq) * 16]);
-        };
-#pragma unroll
-        for (int t = 0; t < kPf; ++t) read_k(t);
+        for (int t = 0; t < kPf; ++t) ka[t] = *reinterpret_cast<const u32x4_t *>(k_rd + t * 64);
 #pragma unroll
         for (int t = 0; t < KSTEPS; ++t) {
-            if (t + kPf < KSTEPS) read_k(t + kPf);
-            s[0] = mfma16<T>(ka[t][0], qreg[t], s[0]);
-            s[1] = mfma16<T>(ka[t][1], qreg[t], s[1]);
+            if (t + kPf < KSTEPS) ka[t + kPf] = *reinterpret_cast<const u32x4_t *>(k_rd + (t + kPf) * 64);
+            s2[t & 1] = mfma16<T>(ka[t], qreg[t], s2[t & 1]);
             __builtin_amdgcn_sched_barrier(0);
         }
 
-        // ---- softmax of this wave's heads; register i of tile tt is key c*32 + tt*16 + lq*4 + i
-        const int key_base = c * kChunk + lq * 4;
-        float x[8], vs[8];
+        // ---- softmax; register i is key c*32 + kt*16 + lq*4 + i of head `head`
+        const int key_base = c * kChunk + kt * 16 + lq * 4;
+        const float4 ks4 = *reinterpret_cast<const float4 *>(&sh.ks[cur][kt * 16 + lq * 4]);
+        const float4 vs4 = *reinterpret_cast<const float4 *>(&sh.vs[cur][kt * 16 + lq * 4]);
+        const float ksv[4] = {ks4.x, ks4.y, ks4.z, ks4.w};
+        const float vsv[4] = {vs4.x, vs4.y, vs4.z, vs4.w};
+        float x[4];
         float mloc = -INFINITY;
 #pragma unroll
-        for (int tt = 0; tt < 2; ++tt) {
-            const float4 ks4 = *reinterpret_cast<const float4 *>(&sh.ks[cur][tt * 16 + lq * 4]);
-            const float4 vs4 = *reinterpret_cast<const float4 *>(&sh.vs[cur][tt * 16 + lq * 4]);
-            const float ksv[4] = {ks4.x, ks4.y, ks4.z, ks4.w};
-            const float vsv[4] = {vs4.x, vs4.y, vs4.z, vs4.w};
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int key = key_base + tt * 16 + i;
-                float v = s[tt][i] * ksv[i] * p.scale_log2;
-                v = (key >= range_lo && key < range_hi) ? v : -INFINITY;
-                x[tt * 4 + i] = v;
-                vs[tt * 4 + i] = vsv[i];
-                mloc = fmaxf(mloc, v);
-            }
+        for (int i = 0; i < 4; ++i) {
+            const int key = key_base + i;
+            float v = (s2[0][i] + s2[1][i]) * ksv[i] * p.scale_log2;
+            v = (key >= range_lo && key < range_hi) ? v : -INFINITY;
+            x[i] = v;
+            mloc = fmaxf(mloc, v);
         }
         mloc = quad_rows_max(mloc);
+        if (lq == 0) sh.mx[kt][g][ln] = mloc;
+        __syncthreads();   // both key tiles' maxima are in LDS (and the previous chunk's products are done)
+
+        mloc = fmaxf(mloc, sh.mx[kt ^ 1][g][ln]);
         const bool bump = mloc > m_run;
         const float m_new = bump ? mloc : m_run;
         const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
@@ -204,116 +219,113 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
         m_run = m_new;
         float psum = 0.f;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const float pe = fast_exp2(x[e] - m_use);
+        for (int i = 0; i < 4; ++i) {
+            const float pe = fast_exp2(x[i] - m_use);
             psum += pe;
-            x[e] = pe * vs[e];   // V side of the dequantisation folded into P
+            x[i] = pe * vsv[i];   // V side of the dequantisation folded into P
         }
         l_run = l_run * alpha + psum;
-        u32x4_t pk;
-        pk[0] = pack2<T>(x[0], x[1]);
-        pk[1] = pack2<T>(x[2], x[3]);
-        pk[2] = pack2<T>(x[4], x[5]);
-        pk[3] = pack2<T>(x[6], x[7]);
-        sh.pk[wave][lane] = pk;
-        if (lq == 0) sh.alpha[wave * 16 + ln] = alpha;
-        const int wave_bump = __any(bump) ? 1 : 0;
-        if (lane == 0) sh.bump[wave] = wave_bump;
-        __syncthreads();   // P, alpha of all 64 heads are in LDS
-
-        // ---- O^T += V^T P^T on this wave's 128-column slice, all four head groups
-        u32x4_t pkg[4];
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            pkg[g] = sh.pk[g][lane];
-            if (sh.bump[g]) {
-                const float ag = sh.alpha[g * 16 + ln];
-#pragma unroll
-                for (int t = 0; t < 8; ++t) {
-                    o_acc[g][t][0] *= ag;
-                    o_acc[g][t][1] *= ag;
-                    o_acc[g][t][2] *= ag;
-                    o_acc[g][t][3] *= ag;
-                }
-            }
+        sh.pk[g][lane][kt] = make_uint2(pack2<T>(x[0], x[1]), pack2<T>(x[2], x[3]));
+        if (kt == 0) {
+            if (lq == 0) sh.alpha[g][ln] = alpha;
+            const int wave_bump = __any(bump) ? 1 : 0;
+            if (lane == 0) sh.bump[g] = (uint8_t)wave_bump;
         }
-        u32x4_t vr[8];
+        // widening of the prefetched tile: its buffer was last read by the previous chunk's products
+        if (more) stash(cur ^ 1, set ^ 1, tid_here);
+        __syncthreads();   // P, alpha of all 64 heads and the next tile are in LDS
+
+        // ---- O^T += V^T P^T on this wave's 64-column slice, all four head groups.
+        //      k slot 8*lq + e of the MFMA is key (e >> 2) * 16 + lq * 4 + (e & 3) of the chunk.
+        uint2 vr[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
             const int row = (e >> 2) * 16 + lq * 4 + (e & 3);
-            vr[e] = *reinterpret_cast<const u32x4_t *>(&sh.k[cur][row * kMlaRowBytes + (wave * 128 + ln * 8) * 2]);
+            vr[e] = *reinterpret_cast<const uint2 *>(&sh.k[cur][row * kMlaRowBytes + (wave * 64 + ln * 4) * 2]);
+        }
+        u32x4_t pkg[4];
+        const uint32_t bumps = *reinterpret_cast<const uint32_t *>(sh.bump);
+#pragma unroll
+        for (int hg = 0; hg < 4; ++hg) {
+            pkg[hg] = *reinterpret_cast<const u32x4_t *>(&sh.pk[hg][lane][0]);
+            if ((bumps >> (8 * hg)) & 0xffu) {
+                const float ag = sh.alpha[hg][ln];
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    o_acc[hg][t][0] *= ag;
+                    o_acc[hg][t][1] *= ag;
+                    o_acc[hg][t][2] *= ag;
+                    o_acc[hg][t][3] *= ag;
+                }
+            }
         }
 #pragma unroll
-        for (int w2 = 0; w2 < 4; ++w2) {
+        for (int w2 = 0; w2 < 2; ++w2) {
             u32x4_t a_lo, a_hi;
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
-                a_lo[u] = __builtin_amdgcn_perm(vr[2 * u + 1][w2], vr[2 * u][w2], 0x05040100u);
-                a_hi[u] = __builtin_amdgcn_perm(vr[2 * u + 1][w2], vr[2 * u][w2], 0x07060302u);
+                const uint32_t e0 = w2 ? vr[2 * u].y : vr[2 * u].x;
+                const uint32_t e1 = w2 ? vr[2 * u + 1].y : vr[2 * u + 1].x;
+                a_lo[u] = __builtin_amdgcn_perm(e1, e0, 0x05040100u);
+                a_hi[u] = __builtin_amdgcn_perm(e1, e0, 0x07060302u);
             }
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                o_acc[g][2 * w2] = mfma16<T>(a_lo, pkg[g], o_acc[g][2 * w2]);
-                o_acc[g][2 * w2 + 1] = mfma16<T>(a_hi, pkg[g], o_acc[g][2 * w2 + 1]);
+            for (int hg = 0; hg < 4; ++hg) {
+                o_acc[hg][2 * w2] = mfma16<T>(a_lo, pkg[hg], o_acc[hg][2 * w2]);
+                o_acc[hg][2 * w2 + 1] = mfma16<T>(a_hi, pkg[hg], o_acc[hg][2 * w2 + 1]);
             }
         }
-
-        // keep the widening of the prefetched tile behind the products: it waits for the loads
-        __builtin_amdgcn_sched_barrier(0);
-        if (more) stash(cur ^ 1);
-        __syncthreads();   // next tile staged; P buffer free again
-        cur ^= 1;
+    };
+    for (int c = c_begin; c < c_end; c += 2) {
+        chunk_step(c, 0);
+        if (c + 1 < c_end) chunk_step(c + 1, 1);
     }
 
     // ---- write.  The score-owning waves publish max and sum; every wave then stores its column
-    //      slice: register i of tile t of group g is column wave*128 + (lq*4 + i)*8 + t of head g*16 + ln.
+    //      slice: register i of tile t of group hg is column wave*64 + (lq*4 + i)*4 + t of head hg*16 + ln.
     l_run = quad_rows_sum(l_run);
     if (lq == 0) {
-        sh.m[wave * 16 + ln] = m_run;
-        sh.l[wave * 16 + ln] = l_run;
+        sh.m[g][ln] = m_run;      // identical in both key-tile waves
+        sh.l[kt][g][ln] = l_run;
     }
     __syncthreads();
 #pragma unroll
-    for (int g = 0; g < 4; ++g) {
-        const int row = g * 16 + ln;   // row of the unit (0..63)
+    for (int hg = 0; hg < 4; ++hg) {
+        const int row = hg * 16 + ln;   // row of the unit (0..63)
         const int hd = half * kMlaHeadsPerUnit + row;
-        const float lg = sh.l[row];
+        const float lg = sh.l[0][hg][ln] + sh.l[1][hg][ln];
         const float inv = (lg > 0.f) ? 1.f / lg : 0.f;
         if (write_final) {
             uint16_t *dst = reinterpret_cast<uint16_t *>(p.out) + (int64_t)b * p.o_stride_b + (int64_t)hd * p.o_stride_h +
-                            wave * 128;
+                            wave * 64;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                u32x4_t o4;
-#pragma unroll
-                for (int u = 0; u < 4; ++u) o4[u] = pack2<T>(o_acc[g][2 * u][i] * inv, o_acc[g][2 * u + 1][i] * inv);
-                store16(dst + (lq * 4 + i) * 8, o4);
+                const uint2 o2 = make_uint2(pack2<T>(o_acc[hg][0][i] * inv, o_acc[hg][1][i] * inv),
+                                            pack2<T>(o_acc[hg][2][i] * inv, o_acc[hg][3][i] * inv));
+                *reinterpret_cast<uint2 *>(dst + (lq * 4 + i) * 4) = o2;
             }
         } else {
             const int64_t srow = slot * p.rows + row;
-            float *dst = p.o_partial + srow * kMlaDv + wave * 128;
+            float *dst = p.o_partial + srow * kMlaDv + wave * 64;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                float *d2 = dst + (lq * 4 + i) * 8;
-                *reinterpret_cast<float4 *>(d2) = make_float4(o_acc[g][0][i] * inv, o_acc[g][1][i] * inv, o_acc[g][2][i] * inv,
-                                                              o_acc[g][3][i] * inv);
-                *reinterpret_cast<float4 *>(d2 + 4) = make_float4(o_acc[g][4][i] * inv, o_acc[g][5][i] * inv,
-                                                                  o_acc[g][6][i] * inv, o_acc[g][7][i] * inv);
-            }
+            for (int i = 0; i < 4; ++i)
+                *reinterpret_cast<float4 *>(dst + (lq * 4 + i) * 4) =
+                    make_float4(o_acc[hg][0][i] * inv, o_acc[hg][1][i] * inv, o_acc[hg][2][i] * inv, o_acc[hg][3][i] * inv);
         }
     }
-    if (lq == 0) {
+    if (kt == 0 && lq == 0) {
         // this lane column's own head: LSE (final) or partial LSE
-        const int row = wave * 16 + ln;
+        const int row = g * 16 + ln;
+        const float lg = sh.l[0][g][ln] + sh.l[1][g][ln];
         if (write_final)
-            p.lse[(int64_t)b * p.nheads + head] = (l_run > 0.f) ? (m_run + fast_log2(l_run)) * kLn2 : INFINITY;
+            p.lse[(int64_t)b * p.nheads + head] = (lg > 0.f) ? (m_run + fast_log2(lg)) * kLn2 : INFINITY;
         else
-            p.lse_partial[slot * p.rows + row] = (l_run > 0.f) ? m_run + fast_log2(l_run) : -INFINITY;
+            p.lse_partial[slot * p.rows + row] = (lg > 0.f) ? m_run + fast_log2(lg) : -INFINITY;
     }
     __syncthreads();   // the LDS tiles are reused by the next piece
 }
 
-template <typename T> __global__ void __launch_bounds__(256, 1) decode_mla_i8_kernel(const DecodeParams p) {
+template <typename T> __global__ void __launch_bounds__(kMlaThreads) decode_mla_i8_kernel(const DecodeParams p) {
     __shared__ MlaShared sh;
     balanced_driver<kMlaDv>(p, [&](int b, int half, const UnitRange &ur, int range_lo, int range_hi, bool whole, int64_t slot) {
         mla_piece<T>(p, b, half, ur, range_lo, range_hi, whole, slot, sh);
@@ -324,7 +336,7 @@ template <typename T> __global__ void __launch_bounds__(256, 1) decode_mla_i8_ke
 hipError_t launch_decode_mla_i8(const DecodeParams &p, int dtype, hipStream_t stream) {
     if (p.seqlen_q != 1 || p.rows != kMlaHeadsPerUnit || p.group != kMlaHeadsPerUnit || !p.balanced)
         return hipErrorInvalidValue;
-    dim3 grid(p.num_wgs), block(256);
+    dim3 grid(p.num_wgs), block(kMlaThreads);
     if (dtype == 0)
         hipLaunchKernelGGL(decode_mla_i8_kernel<BF16>, grid, block, 0, stream, p);
     else
