@@ -7,19 +7,22 @@
 // the same as the bf16 decode kernel's (mha_fwd_kvcache.cpp:632-969 in the reference) applied to
 // K^ = code * scale[token].
 //
-// A work unit is (batch row, 64-head half).  The 512-thread workgroup (two waves per SIMD, so one
-// wave's matrix products cover the other's conversions and LDS waits) streams its share of the
+// A work unit is (batch row, 64-head half).  The 512-thread workgroup streams its share of the
 // unit list (same balanced partition as the bf16 decode kernel): every 32-key chunk is fetched
 // once as int8 with 12-byte loads, widened to the 16-bit type on the way into LDS (a code is an
-// integer of magnitude <= 127, exact in bf16 and fp16) and shared by the eight waves.
-//   scores : wave (g, t) owns head group g (16 heads, Q^T resident in registers) and the 16-key
-//            tile t of the chunk: S^T = K Q^T, per-token scale folded into the scores; the chunk
-//            maximum of a head group is exchanged between its two waves through LDS;
-//   output : the waves trade places: P of all 64 heads goes through LDS and every wave owns a
-//            64-column slice of V for all heads, so each transposed V operand (rows read whole
-//            from the same LDS tile, v_perm in registers) feeds four MFMAs; the V side of the
-//            dequantisation is folded into P.
-// Two barriers per chunk; the widening of the next chunk sits between them.
+// integer of magnitude <= 127, exact in bf16 and fp16) and shared by the eight waves, which come
+// in two kinds, one of each per SIMD:
+//   score waves  (0-3): they also stage the cache (loads two chunks ahead, the widening of chunk
+//            c+2 interleaved with the products of chunk c+1); wave w owns heads 16w..16w+15 with
+//            Q^T resident in registers: S^T = K Q^T over the chunk, per-token scale folded into
+//            the scores, online softmax local to the lane column; P, the rescale factor and a
+//            "new maximum" flag go to LDS;
+//   output waves (4-7): wave w owns a 128-column slice of V for all 64 heads: O^T += V^T P^T, each
+//            transposed V operand (rows read whole from the same LDS tile, v_perm in registers)
+//            feeding four MFMAs; the V side of the dequantisation is folded into P.
+// The kinds run one chunk apart (scores of chunk c+1 beside the output of chunk c), so the
+// LDS-heavy score products, the conversions and the output products of one SIMD overlap instead
+// of taking turns, with one barrier per chunk.
 #include "decode_common.h"
 
 namespace fa {
@@ -30,9 +33,10 @@ constexpr int kMlaThreads = 512;
 constexpr int kMlaRowBytes = kMlaDqk * 2 + 16;           // padded LDS row: conflict-free operand reads
 constexpr int kMlaTileBytes = kChunk * kMlaRowBytes;     // 37376
 constexpr int kMlaPiecesPerRow = kMlaDqk / 12;           // 48 12-byte int8 pieces per key
-constexpr int kMlaRounds = kChunk * kMlaPiecesPerRow / kMlaThreads;   // 3 pieces per thread per chunk
+constexpr int kMlaStagers = 256;                         // threads of the score waves
+constexpr int kMlaRounds = kChunk * kMlaPiecesPerRow / kMlaStagers;   // 6 pieces per staging thread per chunk
 constexpr int kMlaHeadsPerUnit = 64;
-static_assert(kChunk * kMlaPiecesPerRow == kMlaRounds * kMlaThreads, "chunk must split evenly over the threads");
+static_assert(kChunk * kMlaPiecesPerRow == kMlaRounds * kMlaStagers, "chunk must split evenly over the staging threads");
 
 struct __attribute__((aligned(4))) MlaCodes12 { uint32_t w[3]; };
 
@@ -47,15 +51,13 @@ template <typename T> __device__ __forceinline__ void widen4(uint32_t w, uint32_
 }
 
 struct MlaShared {
-    __attribute__((aligned(16))) uint8_t k[2][kMlaTileBytes];   // widened key tiles
-    __attribute__((aligned(16))) float ks[2][kChunk];            // per-token scales, K side
-    __attribute__((aligned(16))) float vs[2][kChunk];            // per-token scales, V side
-    __attribute__((aligned(16))) uint2 pk[4][64][2];             // P^T operands of the four head groups, by key tile
-    // per head, indexed [head group][head in group] so the group is a constant address offset
-    float mx[2][4][16];                                          // chunk maximum per key tile
-    float alpha[4][16];                                          // accumulator rescale
-    float m[4][16], l[2][4][16];                                 // final max, sum per key tile
-    __attribute__((aligned(4))) uint8_t bump[4];                 // head group saw a new maximum
+    __attribute__((aligned(16))) uint8_t k[3][kMlaTileBytes];   // widened key tiles: scores, output, being filled
+    __attribute__((aligned(16))) float ks[3][kChunk];            // per-token scales, K side
+    __attribute__((aligned(16))) float vs[3][kChunk];            // per-token scales, V side
+    __attribute__((aligned(16))) u32x4_t pk[2][4][64];           // P^T operands of the four head groups, two chunks
+    float alpha[2][4][16];                                       // accumulator rescale per head
+    __attribute__((aligned(4))) uint8_t bump[2][4];              // head group saw a new maximum
+    float l[4][16];                                              // final sum per head
 };
 
 template <typename T>
@@ -64,265 +66,309 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
                                           const int64_t slot, MlaShared &sh) {
     constexpr int KSTEPS = kMlaDqk / 32;   // 18
     const int tid = threadIdx.x;
-    const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int g = wave & 3;    // head group of the score phase
-    const int kt = wave >> 2;  // 16-key tile of the score phase
-    const int lq = lane >> 4;
-    const int ln = lane & 15;
-    const int head = half * kMlaHeadsPerUnit + g * 16 + ln;   // query head whose scores this lane column holds
+    const int role = wave >> 2;   // 0: scores, 1: output
+    const int w4 = wave & 3;      // head group (scores) or 128-column slice (output)
     const int Lk = ur.Lk;
-
-    // Q^T operand (seqlen_q == 1): lane (lq, ln) holds head `head`, elements t*32 + lq*8 .. +7
-    u32x4_t qreg[KSTEPS];
-    {
-        const uint16_t *src = reinterpret_cast<const uint16_t *>(p.q) + (int64_t)b * p.q_stride_b +
-                              (int64_t)head * p.q_stride_h + lq * 8;
-#pragma unroll
-        for (int t = 0; t < KSTEPS; ++t) qreg[t] = load16(src + t * 32);
-    }
-
-    float m_run = -INFINITY, l_run = 0.f;
-    // o_acc[hg][t]: head group hg (16 heads), column tile t of this wave's 64-column slice
-    float4_t o_acc[4][4];
-#pragma unroll
-    for (int hg = 0; hg < 4; ++hg)
-#pragma unroll
-        for (int t = 0; t < 4; ++t) o_acc[hg][t] = float4_t{0.f, 0.f, 0.f, 0.f};
 
     const int8_t *kc = reinterpret_cast<const int8_t *>(p.k_cache);
     const int32_t *bt_row = p.block_table + (int64_t)b * p.bt_stride_b;
     const int c_begin = range_lo / kChunk;
-    const int c_end = (range_hi + kChunk - 1) / kChunk;
+    const int n = (range_hi + kChunk - 1) / kChunk - c_begin;   // chunks of this piece
 
-    // ---- staging: int8 rows -> registers -> widened LDS tile.  Loads run two chunks ahead of the
-    //      products (register sets st[0], st[1] by chunk parity within the piece): one chunk of
-    //      arithmetic is shorter than a trip to memory.
-    MlaCodes12 st[2][kMlaRounds];
-    float st_ks[2] = {0.f, 0.f}, st_vs[2] = {0.f, 0.f};
-    auto fetch_blk = [&](int c) -> int {
-        if (c >= c_end) return 0;
-        int page = (c * kChunk) / p.page_size;
-        page = min(page, p.max_blocks - 1);
-        return min(max(bt_row[page], 0), p.num_blocks - 1);
-    };
-    // thread -> (key row, 12-byte column) of the chunk: 16 threads per row, three pieces 192 bytes
-    // apart each, so one address per chunk serves all three loads and one LDS address all stores
-    static_assert(kMlaThreads / 16 == kChunk && kMlaRounds * 16 == kMlaPiecesPerRow, "thread map of the staging");
-    // (the thread index comes in as an argument: the chunk loop passes a copy the compiler cannot
-    //  see through, so these few address terms are recomputed per chunk instead of held in registers)
-    auto fetch = [&](int c, int blk, int set, int th) {
-        const int t_row = th >> 4;
-        const int t_sub = th & 15;
-        const int key0 = c * kChunk;
-        const int inpage0 = key0 % p.page_size;
-        const int last = Lk - 1 - key0;
-        // wave-uniform 64-bit base + 32-bit per-thread offset
-        const int8_t *src = kc + (int64_t)blk * p.k_stride_block + (int64_t)inpage0 * p.k_stride_row;
-        const uint32_t voff = (uint32_t)min(t_row, last) * (uint32_t)p.k_stride_row + t_sub * 12;
+    // Step j of a piece (j = 0 .. n + 1): chunk j is widened into tile j % 3 and chunk j + 2 loaded;
+    // the score waves work on chunk j - 1 (tile (j + 2) % 3), the output waves on chunk j - 2
+    // (tile (j + 1) % 3); one barrier ends the step.
+    if (role == 0) {
+        // =========================== score waves ===========================================
+        const int lane0 = tid & 63;
+        const int head = half * kMlaHeadsPerUnit + w4 * 16 + (lane0 & 15);   // head of this lane column
+        // Q^T operand (seqlen_q == 1): lane (lq, ln) holds head `head`, elements t*32 + lq*8 .. +7
+        u32x4_t qreg[KSTEPS];
+        {
+            const uint16_t *src = reinterpret_cast<const uint16_t *>(p.q) + (int64_t)b * p.q_stride_b +
+                                  (int64_t)head * p.q_stride_h + (lane0 >> 4) * 8;
 #pragma unroll
-        for (int i = 0; i < kMlaRounds; ++i) st[set][i] = *reinterpret_cast<const MlaCodes12 *>(src + voff + i * 192);
-        // every thread loads a scale (no branch around a load: the waits stay counted in order)
-        const int64_t so = (int64_t)blk * p.ks_stride_block + (int64_t)inpage0 * p.ks_stride_row;
-        const uint32_t soff = (uint32_t)min(th & (kChunk - 1), last) * (uint32_t)p.ks_stride_row;
-        st_ks[set] = (p.k_scale + so)[soff];
-        st_vs[set] = (p.v_scale + so)[soff];
-    };
-    auto stash = [&](int buf, int set, int th) {
-        uint8_t *dst = &sh.k[buf][(th >> 4) * kMlaRowBytes + (th & 15) * 24];
+            for (int t = 0; t < KSTEPS; ++t) qreg[t] = load16(src + t * 32);
+        }
+        // ---- staging: int8 rows -> registers -> widened LDS tile.  Chunk j of the piece is loaded
+        //      into register set j & 1 two steps before it is widened.  Thread -> (key row, 12-byte
+        //      column): 8 threads per row, six pieces 96 bytes apart each, so one address per chunk
+        //      serves all loads and one LDS address all stores.  Past the end of the piece the last
+        //      chunk is named again: every step issues the same loads, so the compiler counts the
+        //      loads in flight instead of waiting for all of them.  Page ids are loaded one step
+        //      before the tile loads that use them and ahead of that step's tile loads, so waiting
+        //      for a page id never waits for younger tile loads.  The thread index comes in as an
+        //      argument: the step loop passes a copy the compiler cannot see through, so the few
+        //      address terms are recomputed per chunk instead of held in registers.
+        static_assert(kMlaStagers / 8 == kChunk && kMlaRounds * 8 == kMlaPiecesPerRow, "thread map of the staging");
+        MlaCodes12 st[2][kMlaRounds];
+        float st_ks[2] = {0.f, 0.f}, st_vs[2] = {0.f, 0.f};
+        auto fetch_blk = [&](int j) -> int {
+            int page = ((c_begin + min(j, n - 1)) * kChunk) / p.page_size;
+            page = min(page, p.max_blocks - 1);
+            return min(max(bt_row[page], 0), p.num_blocks - 1);
+        };
+        auto fetch = [&](int j_any, int blk, int set, int th) {
+            const int j = min(j_any, n - 1);
+            const int t_row = th >> 3;
+            const int t_sub = th & 7;
+            const int key0 = (c_begin + j) * kChunk;
+            const int inpage0 = key0 % p.page_size;
+            const int last = Lk - 1 - key0;
+            // wave-uniform 64-bit base + 32-bit per-thread offset
+            const int8_t *src = kc + (int64_t)blk * p.k_stride_block + (int64_t)inpage0 * p.k_stride_row;
+            const uint32_t voff = (uint32_t)min(t_row, last) * (uint32_t)p.k_stride_row + t_sub * 12;
 #pragma unroll
-        for (int i = 0; i < kMlaRounds; ++i) {
+            for (int i = 0; i < kMlaRounds; ++i) st[set][i] = *reinterpret_cast<const MlaCodes12 *>(src + voff + i * 96);
+            const int64_t so = (int64_t)blk * p.ks_stride_block + (int64_t)inpage0 * p.ks_stride_row;
+            const uint32_t soff = (uint32_t)min(th & (kChunk - 1), last) * (uint32_t)p.ks_stride_row;
+            st_ks[set] = (p.k_scale + so)[soff];
+            st_vs[set] = (p.v_scale + so)[soff];
+        };
+        // word t (0..17) of the staged chunk: four codes -> four 16-bit floats -> LDS
+        auto widen_word = [&](int tile, int set, int th, int t) {
+            uint8_t *dst = &sh.k[tile][(th >> 3) * kMlaRowBytes + (th & 7) * 24];
+            uint2 w;
+            widen4<T>(st[set][t / 3].w[t % 3], w.x, w.y);
+            *reinterpret_cast<uint2 *>(dst + (t / 3) * 192 + (t % 3) * 8) = w;
+        };
+        auto stash_scales = [&](int tile, int set, int th) {
+            if (th < kChunk) {
+                sh.ks[tile][th] = st_ks[set];
+                sh.vs[tile][th] = st_vs[set];
+            }
+        };
+        int blk_next;
+        {
+            const int b0 = fetch_blk(0), b1 = fetch_blk(1);
+            blk_next = fetch_blk(2);
+            fetch(0, b0, 0, tid);
+            fetch(1, b1, 1, tid);
+        }
+        float m_run = -INFINITY, l_run = 0.f;
+
+        auto score_step = [&](const int j, const int set, const int tile_j) {
+            int th = tid;
+            asm volatile("" : "+v"(th));
+            const int lane = th & 63;
+            const int lq = lane >> 4;
+            const int ln = lane & 15;
+            const bool do_stash = j < n;
+            const bool do_score = j >= 1 && j <= n;
+            const int tile = (tile_j == 0) ? 2 : tile_j - 1;   // (j + 2) % 3: tile of the scores
+            float4_t s[2] = {float4_t{0.f, 0.f, 0.f, 0.f}, float4_t{0.f, 0.f, 0.f, 0.f}};
+            if (do_score) {
+                // ---- S^T = K Q^T : two 16-key tiles x this wave's 16 heads; operand reads run kPf
+                //      k-steps ahead of the MFMAs that use them; one word of the next-but-one chunk
+                //      is widened beside every k-step (in the last score step that is the last chunk
+                //      once more, into a tile nobody reads: no branch inside the product loop)
+                constexpr int kPf = 4;
+                u32x4_t ka[KSTEPS][2];
+                const uint8_t *k_rd = &sh.k[tile][ln * kMlaRowBytes + lq * 16];
+                auto read_k = [&](int t) {
+                    ka[t][0] = *reinterpret_cast<const u32x4_t *>(k_rd + t * 64);
+                    ka[t][1] = *reinterpret_cast<const u32x4_t *>(k_rd + 16 * kMlaRowBytes + t * 64);
+                };
 #pragma unroll
-            for (int j = 0; j < 3; ++j) {
-                uint2 w;
-                widen4<T>(st[set][i].w[j], w.x, w.y);
-                *reinterpret_cast<uint2 *>(dst + i * 384 + j * 8) = w;
+                for (int t = 0; t < kPf; ++t) read_k(t);
+#pragma unroll
+                for (int t = 0; t < KSTEPS; ++t) {
+                    if (t + kPf < KSTEPS) read_k(t + kPf);
+                    s[0] = mfma16<T>(ka[t][0], qreg[t], s[0]);
+                    widen_word(tile_j, set, th, t);
+                    s[1] = mfma16<T>(ka[t][1], qreg[t], s[1]);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            } else if (do_stash) {
+#pragma unroll
+                for (int t = 0; t < KSTEPS; ++t) widen_word(tile_j, set, th, t);
+            }
+            if (do_stash) stash_scales(tile_j, set, th);
+            {
+                const int blk_after = fetch_blk(j + 3);
+                fetch(j + 2, blk_next, set, th);
+                blk_next = blk_after;
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            if (do_score) {
+                const int c = c_begin + j - 1;
+                const int pb = set ^ 1;                              // (j - 1) & 1
+                // ---- softmax; register i of tile tt is key c*32 + tt*16 + lq*4 + i
+                const int key_base = c * kChunk + lq * 4;
+                float x[8], vsc[8];
+                float mloc = -INFINITY;
+#pragma unroll
+                for (int tt = 0; tt < 2; ++tt) {
+                    const float4 ks4 = *reinterpret_cast<const float4 *>(&sh.ks[tile][tt * 16 + lq * 4]);
+                    const float4 vs4 = *reinterpret_cast<const float4 *>(&sh.vs[tile][tt * 16 + lq * 4]);
+                    const float ksv[4] = {ks4.x, ks4.y, ks4.z, ks4.w};
+                    const float vsv[4] = {vs4.x, vs4.y, vs4.z, vs4.w};
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int key = key_base + tt * 16 + i;
+                        float v = s[tt][i] * ksv[i] * p.scale_log2;
+                        v = (key >= range_lo && key < range_hi) ? v : -INFINITY;
+                        x[tt * 4 + i] = v;
+                        vsc[tt * 4 + i] = vsv[i];
+                        mloc = fmaxf(mloc, v);
+                    }
+                }
+                mloc = quad_rows_max(mloc);
+                const bool bump = mloc > m_run;
+                const float m_new = bump ? mloc : m_run;
+                const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+                const float alpha = bump ? fast_exp2(m_run - m_use) : 1.f;
+                m_run = m_new;
+                float psum = 0.f;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float pe = fast_exp2(x[e] - m_use);
+                    psum += pe;
+                    x[e] = pe * vsc[e];   // V side of the dequantisation folded into P
+                }
+                l_run = l_run * alpha + psum;
+                u32x4_t pk;
+                pk[0] = pack2<T>(x[0], x[1]);
+                pk[1] = pack2<T>(x[2], x[3]);
+                pk[2] = pack2<T>(x[4], x[5]);
+                pk[3] = pack2<T>(x[6], x[7]);
+                sh.pk[pb][w4][lane] = pk;
+                if (lq == 0) sh.alpha[pb][w4][ln] = alpha;
+                const int wave_bump = __any(bump) ? 1 : 0;
+                if (lane == 0) sh.bump[pb][w4] = (uint8_t)wave_bump;
+            }
+            __syncthreads();
+        };
+        int tile_j = 0;
+        for (int j = 0; j <= n + 1; j += 2) {
+            score_step(j, 0, tile_j);
+            tile_j = (tile_j == 2) ? 0 : tile_j + 1;
+            if (j + 1 <= n + 1) {
+                score_step(j + 1, 1, tile_j);
+                tile_j = (tile_j == 2) ? 0 : tile_j + 1;
             }
         }
-        if (th < kChunk) {
-            sh.ks[buf][th] = st_ks[set];
-            sh.vs[buf][th] = st_vs[set];
+
+        // ---- publish the sums, write the LSE
+        l_run = quad_rows_sum(l_run);
+        const int lane = tid & 63;
+        const int ln = lane & 15;
+        if ((lane >> 4) == 0) {
+            sh.l[w4][ln] = l_run;
+            const int row = w4 * 16 + ln;
+            if (write_final)
+                p.lse[(int64_t)b * p.nheads + head] = (l_run > 0.f) ? (m_run + fast_log2(l_run)) * kLn2 : INFINITY;
+            else
+                p.lse_partial[slot * p.rows + row] = (l_run > 0.f) ? m_run + fast_log2(l_run) : -INFINITY;
         }
-    };
+        __syncthreads();
+    } else {
+        // =========================== output waves ==========================================
+        // o_acc[hg][t]: head group hg (16 heads), column tile t of this wave's 128-column slice
+        float4_t o_acc[4][8];
+#pragma unroll
+        for (int hg = 0; hg < 4; ++hg)
+#pragma unroll
+            for (int t = 0; t < 8; ++t) o_acc[hg][t] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-    // page ids are loaded one step before the loads that use them and always ahead of that step's
-    // tile loads, so waiting for a page id never waits for younger tile loads
-    int blk_next = 0;
-    if (c_begin < c_end) {
-        fetch(c_begin, fetch_blk(c_begin), 0, tid);
-        blk_next = fetch_blk(c_begin + 1);
-        stash(0, 0, tid);
-        const int blk2 = fetch_blk(c_begin + 2);
-        if (c_begin + 1 < c_end) fetch(c_begin + 1, blk_next, 1, tid);
-        blk_next = blk2;
-    }
-    __syncthreads();
+        auto output_step = [&](const int j, const int set, const int tile_j) {
+            int th = tid;
+            asm volatile("" : "+v"(th));
+            const int lane = th & 63;
+            const int lq = lane >> 4;
+            const int ln = lane & 15;
+            if (j >= 2) {
+                const int tile = (tile_j == 2) ? 0 : tile_j + 1;   // (j + 1) % 3
+                const int pb = set;                                  // (j - 2) & 1
+                // ---- O^T += V^T P^T on this wave's 128-column slice, all four head groups.
+                //      k slot 8*lq + e of the MFMA is key (e >> 2) * 16 + lq * 4 + (e & 3) of the chunk.
+                u32x4_t vr[8];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const int row = (e >> 2) * 16 + lq * 4 + (e & 3);
+                    vr[e] = *reinterpret_cast<const u32x4_t *>(&sh.k[tile][row * kMlaRowBytes + (w4 * 128 + ln * 8) * 2]);
+                }
+                u32x4_t pkg[4];
+                const uint32_t bumps = *reinterpret_cast<const uint32_t *>(sh.bump[pb]);
+#pragma unroll
+                for (int hg = 0; hg < 4; ++hg) {
+                    pkg[hg] = sh.pk[pb][hg][lane];
+                    if ((bumps >> (8 * hg)) & 0xffu) {
+                        const float ag = sh.alpha[pb][hg][ln];
+#pragma unroll
+                        for (int t = 0; t < 8; ++t) {
+                            o_acc[hg][t][0] *= ag;
+                            o_acc[hg][t][1] *= ag;
+                            o_acc[hg][t][2] *= ag;
+                            o_acc[hg][t][3] *= ag;
+                        }
+                    }
+                }
+#pragma unroll
+                for (int w2 = 0; w2 < 4; ++w2) {
+                    u32x4_t a_lo, a_hi;
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        a_lo[u] = __builtin_amdgcn_perm(vr[2 * u + 1][w2], vr[2 * u][w2], 0x05040100u);
+                        a_hi[u] = __builtin_amdgcn_perm(vr[2 * u + 1][w2], vr[2 * u][w2], 0x07060302u);
+                    }
+#pragma unroll
+                    for (int hg = 0; hg < 4; ++hg) {
+                        o_acc[hg][2 * w2] = mfma16<T>(a_lo, pkg[hg], o_acc[hg][2 * w2]);
+                        o_acc[hg][2 * w2 + 1] = mfma16<T>(a_hi, pkg[hg], o_acc[hg][2 * w2 + 1]);
+                    }
+                }
+            }
+            __syncthreads();
+        };
+        int tile_j = 0;
+        for (int j = 0; j <= n + 1; j += 2) {
+            output_step(j, 0, tile_j);
+            tile_j = (tile_j == 2) ? 0 : tile_j + 1;
+            if (j + 1 <= n + 1) {
+                output_step(j + 1, 1, tile_j);
+                tile_j = (tile_j == 2) ? 0 : tile_j + 1;
+            }
+        }
 
-    // one chunk; `set` = parity of the chunk within the piece (compile-time in the unrolled loop)
-    auto chunk_step = [&](const int c, const int set) {
-        const int cur = set;
-        const bool more = c + 1 < c_end;
-        // lane-derived LDS addresses are recomputed in every step (a few adds) instead of being kept
-        // in registers across the whole piece, which the register budget cannot afford
-        int tid_here = tid;
-        asm volatile("" : "+v"(tid_here));
-        const int lane = tid_here & 63;
+        // ---- write the column slice: register i of tile t of group hg is column
+        //      w4*128 + (lq*4 + i)*8 + t of head hg*16 + ln
+        __syncthreads();   // sums of all heads are in LDS
+        const int lane = tid & 63;
         const int lq = lane >> 4;
         const int ln = lane & 15;
-        {
-            const int blk3 = fetch_blk(c + 3);
-            if (c + 2 < c_end) fetch(c + 2, blk_next, set, tid_here);
-            blk_next = blk3;
-        }
-        __builtin_amdgcn_sched_barrier(0);
-
-        // ---- S^T = K Q^T : this wave's 16-key tile x 16 heads; operand reads run kPf k-steps
-        //      ahead of the MFMAs that use them, two accumulators break the dependency chain
-        constexpr int kPf = 4;
-        float4_t s2[2] = {float4_t{0.f, 0.f, 0.f, 0.f}, float4_t{0.f, 0.f, 0.f, 0.f}};
-        u32x4_t ka[KSTEPS];
-        const uint8_t *k_rd = &sh.k[cur][(kt * 16 + ln) * kMlaRowBytes + lq * 16];
-#pragma unroll
-        for (int t = 0; t < kPf; ++t) ka[t] = *reinterpret_cast<const u32x4_t *>(k_rd + t * 64);
-#pragma unroll
-        for (int t = 0; t < KSTEPS; ++t) {
-            if (t + kPf < KSTEPS) ka[t + kPf] = *reinterpret_cast<const u32x4_t *>(k_rd + (t + kPf) * 64);
-            s2[t & 1] = mfma16<T>(ka[t], qreg[t], s2[t & 1]);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-
-        // ---- softmax; register i is key c*32 + kt*16 + lq*4 + i of head `head`
-        const int key_base = c * kChunk + kt * 16 + lq * 4;
-        const float4 ks4 = *reinterpret_cast<const float4 *>(&sh.ks[cur][kt * 16 + lq * 4]);
-        const float4 vs4 = *reinterpret_cast<const float4 *>(&sh.vs[cur][kt * 16 + lq * 4]);
-        const float ksv[4] = {ks4.x, ks4.y, ks4.z, ks4.w};
-        const float vsv[4] = {vs4.x, vs4.y, vs4.z, vs4.w};
-        float x[4];
-        float mloc = -INFINITY;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int key = key_base + i;
-            float v = (s2[0][i] + s2[1][i]) * ksv[i] * p.scale_log2;
-            v = (key >= range_lo && key < range_hi) ? v : -INFINITY;
-            x[i] = v;
-            mloc = fmaxf(mloc, v);
-        }
-        mloc = quad_rows_max(mloc);
-        if (lq == 0) sh.mx[kt][g][ln] = mloc;
-        __syncthreads();   // both key tiles' maxima are in LDS (and the previous chunk's products are done)
-
-        mloc = fmaxf(mloc, sh.mx[kt ^ 1][g][ln]);
-        const bool bump = mloc > m_run;
-        const float m_new = bump ? mloc : m_run;
-        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-        const float alpha = bump ? fast_exp2(m_run - m_use) : 1.f;
-        m_run = m_new;
-        float psum = 0.f;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const float pe = fast_exp2(x[i] - m_use);
-            psum += pe;
-            x[i] = pe * vsv[i];   // V side of the dequantisation folded into P
-        }
-        l_run = l_run * alpha + psum;
-        sh.pk[g][lane][kt] = make_uint2(pack2<T>(x[0], x[1]), pack2<T>(x[2], x[3]));
-        if (kt == 0) {
-            if (lq == 0) sh.alpha[g][ln] = alpha;
-            const int wave_bump = __any(bump) ? 1 : 0;
-            if (lane == 0) sh.bump[g] = (uint8_t)wave_bump;
-        }
-        // widening of the prefetched tile: its buffer was last read by the previous chunk's products
-        if (more) stash(cur ^ 1, set ^ 1, tid_here);
-        __syncthreads();   // P, alpha of all 64 heads and the next tile are in LDS
-
-        // ---- O^T += V^T P^T on this wave's 64-column slice, all four head groups.
-        //      k slot 8*lq + e of the MFMA is key (e >> 2) * 16 + lq * 4 + (e & 3) of the chunk.
-        uint2 vr[8];
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const int row = (e >> 2) * 16 + lq * 4 + (e & 3);
-            vr[e] = *reinterpret_cast<const uint2 *>(&sh.k[cur][row * kMlaRowBytes + (wave * 64 + ln * 4) * 2]);
-        }
-        u32x4_t pkg[4];
-        const uint32_t bumps = *reinterpret_cast<const uint32_t *>(sh.bump);
 #pragma unroll
         for (int hg = 0; hg < 4; ++hg) {
-            pkg[hg] = *reinterpret_cast<const u32x4_t *>(&sh.pk[hg][lane][0]);
-            if ((bumps >> (8 * hg)) & 0xffu) {
-                const float ag = sh.alpha[hg][ln];
+            const int row = hg * 16 + ln;   // row of the unit (0..63)
+            const int hd = half * kMlaHeadsPerUnit + row;
+            const float lg = sh.l[hg][ln];
+            const float inv = (lg > 0.f) ? 1.f / lg : 0.f;
+            if (write_final) {
+                uint16_t *dst = reinterpret_cast<uint16_t *>(p.out) + (int64_t)b * p.o_stride_b + (int64_t)hd * p.o_stride_h +
+                                w4 * 128;
 #pragma unroll
-                for (int t = 0; t < 4; ++t) {
-                    o_acc[hg][t][0] *= ag;
-                    o_acc[hg][t][1] *= ag;
-                    o_acc[hg][t][2] *= ag;
-                    o_acc[hg][t][3] *= ag;
+                for (int i = 0; i < 4; ++i) {
+                    u32x4_t o4;
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) o4[u] = pack2<T>(o_acc[hg][2 * u][i] * inv, o_acc[hg][2 * u + 1][i] * inv);
+                    store16(dst + (lq * 4 + i) * 8, o4);
+                }
+            } else {
+                const int64_t srow = slot * p.rows + row;
+                float *dst = p.o_partial + srow * kMlaDv + w4 * 128;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    float *d2 = dst + (lq * 4 + i) * 8;
+                    *reinterpret_cast<float4 *>(d2) = make_float4(o_acc[hg][0][i] * inv, o_acc[hg][1][i] * inv,
+                                                                  o_acc[hg][2][i] * inv, o_acc[hg][3][i] * inv);
+                    *reinterpret_cast<float4 *>(d2 + 4) = make_float4(o_acc[hg][4][i] * inv, o_acc[hg][5][i] * inv,
+                                                                      o_acc[hg][6][i] * inv, o_acc[hg][7][i] * inv);
                 }
             }
         }
-#pragma unroll
-        for (int w2 = 0; w2 < 2; ++w2) {
-            u32x4_t a_lo, a_hi;
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                const uint32_t e0 = w2 ? vr[2 * u].y : vr[2 * u].x;
-                const uint32_t e1 = w2 ? vr[2 * u + 1].y : vr[2 * u + 1].x;
-                a_lo[u] = __builtin_amdgcn_perm(e1, e0, 0x05040100u);
-                a_hi[u] = __builtin_amdgcn_perm(e1, e0, 0x07060302u);
-            }
-#pragma unroll
-            for (int hg = 0; hg < 4; ++hg) {
-                o_acc[hg][2 * w2] = mfma16<T>(a_lo, pkg[hg], o_acc[hg][2 * w2]);
-                o_acc[hg][2 * w2 + 1] = mfma16<T>(a_hi, pkg[hg], o_acc[hg][2 * w2 + 1]);
-            }
-        }
-    };
-    for (int c = c_begin; c < c_end; c += 2) {
-        chunk_step(c, 0);
-        if (c + 1 < c_end) chunk_step(c + 1, 1);
     }
-
-    // ---- write.  The score-owning waves publish max and sum; every wave then stores its column
-    //      slice: register i of tile t of group hg is column wave*64 + (lq*4 + i)*4 + t of head hg*16 + ln.
-    l_run = quad_rows_sum(l_run);
-    if (lq == 0) {
-        sh.m[g][ln] = m_run;      // identical in both key-tile waves
-        sh.l[kt][g][ln] = l_run;
-    }
-    __syncthreads();
-#pragma unroll
-    for (int hg = 0; hg < 4; ++hg) {
-        const int row = hg * 16 + ln;   // row of the unit (0..63)
-        const int hd = half * kMlaHeadsPerUnit + row;
-        const float lg = sh.l[0][hg][ln] + sh.l[1][hg][ln];
-        const float inv = (lg > 0.f) ? 1.f / lg : 0.f;
-        if (write_final) {
-            uint16_t *dst = reinterpret_cast<uint16_t *>(p.out) + (int64_t)b * p.o_stride_b + (int64_t)hd * p.o_stride_h +
-                            wave * 64;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const uint2 o2 = make_uint2(pack2<T>(o_acc[hg][0][i] * inv, o_acc[hg][1][i] * inv),
-                                            pack2<T>(o_acc[hg][2][i] * inv, o_acc[hg][3][i] * inv));
-                *reinterpret_cast<uint2 *>(dst + (lq * 4 + i) * 4) = o2;
-            }
-        } else {
-            const int64_t srow = slot * p.rows + row;
-            float *dst = p.o_partial + srow * kMlaDv + wave * 64;
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-                *reinterpret_cast<float4 *>(dst + (lq * 4 + i) * 4) =
-                    make_float4(o_acc[hg][0][i] * inv, o_acc[hg][1][i] * inv, o_acc[hg][2][i] * inv, o_acc[hg][3][i] * inv);
-        }
-    }
-    if (kt == 0 && lq == 0) {
-        // this lane column's own head: LSE (final) or partial LSE
-        const int row = g * 16 + ln;
-        const float lg = sh.l[0][g][ln] + sh.l[1][g][ln];
-        if (write_final)
-            p.lse[(int64_t)b * p.nheads + head] = (lg > 0.f) ? (m_run + fast_log2(lg)) * kLn2 : INFINITY;
-        else
-            p.lse_partial[slot * p.rows + row] = (lg > 0.f) ? m_run + fast_log2(lg) : -INFINITY;
-    }
-    __syncthreads();   // the LDS tiles are reused by the next piece
+    __syncthreads();   // the LDS tiles and sums are reused by the next piece
 }
 
 template <typename T> __global__ void __launch_bounds__(kMlaThreads) decode_mla_i8_kernel(const DecodeParams p) {
