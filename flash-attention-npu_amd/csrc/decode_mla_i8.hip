@@ -158,12 +158,19 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
             const bool do_score = j >= 1 && j <= n;
             const int tile = (tile_j == 0) ? 2 : tile_j - 1;   // (j + 2) % 3: tile of the scores
             float4_t s[2] = {float4_t{0.f, 0.f, 0.f, 0.f}, float4_t{0.f, 0.f, 0.f, 0.f}};
+            // per-token scales of the score chunk, read ahead of the products
+            float4 ks4[2], vs4[2];
+#pragma unroll
+            for (int tt = 0; tt < 2; ++tt) {
+                ks4[tt] = *reinterpret_cast<const float4 *>(&sh.ks[tile][tt * 16 + lq * 4]);
+                vs4[tt] = *reinterpret_cast<const float4 *>(&sh.vs[tile][tt * 16 + lq * 4]);
+            }
             if (do_score) {
                 // ---- S^T = K Q^T : two 16-key tiles x this wave's 16 heads; operand reads run kPf
                 //      k-steps ahead of the MFMAs that use them; one word of the next-but-one chunk
                 //      is widened beside every k-step (in the last score step that is the last chunk
                 //      once more, into a tile nobody reads: no branch inside the product loop)
-                constexpr int kPf = 4;
+                constexpr int kPf = 8;
                 u32x4_t ka[KSTEPS][2];
                 const uint8_t *k_rd = &sh.k[tile][ln * kMlaRowBytes + lq * 16];
                 auto read_k = [&](int t) {
@@ -200,10 +207,8 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
                 float mloc = -INFINITY;
 #pragma unroll
                 for (int tt = 0; tt < 2; ++tt) {
-                    const float4 ks4 = *reinterpret_cast<const float4 *>(&sh.ks[tile][tt * 16 + lq * 4]);
-                    const float4 vs4 = *reinterpret_cast<const float4 *>(&sh.vs[tile][tt * 16 + lq * 4]);
-                    const float ksv[4] = {ks4.x, ks4.y, ks4.z, ks4.w};
-                    const float vsv[4] = {vs4.x, vs4.y, vs4.z, vs4.w};
+                    const float ksv[4] = {ks4[tt].x, ks4[tt].y, ks4[tt].z, ks4[tt].w};
+                    const float vsv[4] = {vs4[tt].x, vs4[tt].y, vs4[tt].z, vs4[tt].w};
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
                         const int key = key_base + tt * 16 + i;

@@ -91,16 +91,30 @@ __device__ __forceinline__ float16_t mfma32<FP16>(const u32x4_t &a, const u32x4_
 // ---- wave-level exchanges -------------------------------------------------------------------
 __device__ __forceinline__ float xor_shuffle(float v, int lane_mask) { return __shfl_xor(v, lane_mask, 64); }
 
-// max / sum over the four lanes {n, n+16, n+32, n+48}
+// max / sum over the four lanes {n, n+16, n+32, n+48}, in the vector ALU: the gfx950 permlane
+// swaps trade rows (16 lanes) and halves (32 lanes) between two registers, so with both operands
+// the same value the two results hold v[lane] and v[lane ^ 16] (resp. ^ 32) in some order -
+// enough for a symmetric reduction, and without the LDS round trip of a bpermute
 __device__ __forceinline__ float quad_rows_max(float v) {
-    v = fmaxf(v, xor_shuffle(v, 16));
-    v = fmaxf(v, xor_shuffle(v, 32));
-    return v;
+    auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+    r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+// max / sum over the two lanes {n, n ^ 32}
+__device__ __forceinline__ float halves_max(float v) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float halves_sum(float v) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 __device__ __forceinline__ float quad_rows_sum(float v) {
-    v += xor_shuffle(v, 16);
-    v += xor_shuffle(v, 32);
-    return v;
+    auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = __uint_as_float(r[0]) + __uint_as_float(r[1]);
+    r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }

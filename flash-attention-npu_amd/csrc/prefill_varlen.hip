@@ -266,7 +266,7 @@ __global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) prefill_kernel(const 
                     mloc = fmaxf(mloc, v);
                 }
         }
-        mloc = fmaxf(mloc, xor_shuffle(mloc, 32));
+        mloc = halves_max(mloc);
         // The accumulator rescale is skipped for the whole wave when no row of it saw a new maximum
         // (most tiles once a row is a few hundred keys in).  m_run stays the exact running maximum,
         // so the largest P of a row is exactly 1 as in the reference's golden.
@@ -341,7 +341,7 @@ __global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) prefill_kernel(const 
 
     // ---- epilogue: O^T / l, store.  Register r of column tile t is V column
     //      t*32 + 8*(r/4) + 4*lh + r%4 of query row ln: four consecutive columns per (t, r/4).
-    l_run += xor_shuffle(l_run, 32);
+    l_run = halves_sum(l_run);
     const float inv = (l_run > 0.f) ? 1.f / l_run : 0.f;
     if (row_ok) {
         uint16_t *dst = ob + (int64_t)(q0 + my_row) * p.o_stride_t;
