@@ -9,7 +9,7 @@
 //
 // A work unit is (batch row, 64-head half).  The 512-thread workgroup streams its share of the
 // unit list (same balanced partition as the bf16 decode kernel): every 32-key chunk is fetched
-// once as int8 with 12-byte loads, widened to the 16-bit type on the way into LDS (a code is an
+// once as int8 with 8-byte loads, widened to the 16-bit type on the way into LDS (a code is an
 // integer of magnitude <= 127, exact in bf16 and fp16) and shared by the eight waves, which come
 // in two kinds, one of each per SIMD:
 //   score waves  (0-3): they also stage the cache (loads two chunks ahead, the widening of chunk
@@ -30,15 +30,20 @@ namespace fa {
 constexpr int kMlaDqk = 576;
 constexpr int kMlaDv = 512;
 constexpr int kMlaThreads = 512;
-constexpr int kMlaRowBytes = kMlaDqk * 2 + 16;           // padded LDS row: conflict-free operand reads
-constexpr int kMlaTileBytes = kChunk * kMlaRowBytes;     // 37376
-constexpr int kMlaPiecesPerRow = kMlaDqk / 12;           // 48 12-byte int8 pieces per key
+// LDS key rows are unpadded; the 16-byte units of a row are XOR-swizzled with (row & 7) inside
+// their aligned groups of eight.  The LDS serves 16-byte reads eight lanes at a time and two
+// neighbouring groups of eight lanes overlap in time, so any 16 consecutive lanes (from a
+// multiple of 8) must hit 16 different units modulo 256 bytes: rows are 1152 = 4.5 * 256 bytes,
+// so odd and even rows sit half a bank cycle apart and the swizzle spreads rows of equal parity.
+constexpr int kMlaRowBytes = kMlaDqk * 2;                // 1152
+constexpr int kMlaTileBytes = kChunk * kMlaRowBytes;     // 36864
+constexpr int kMlaPiecesPerRow = kMlaDqk / 8;            // 72 8-byte int8 pieces per key = 16-byte units once widened
 constexpr int kMlaStagers = 256;                         // threads of the score waves
-constexpr int kMlaRounds = kChunk * kMlaPiecesPerRow / kMlaStagers;   // 6 pieces per staging thread per chunk
+constexpr int kMlaRounds = kChunk * kMlaPiecesPerRow / kMlaStagers;   // 9 pieces per staging thread per chunk
 constexpr int kMlaHeadsPerUnit = 64;
 static_assert(kChunk * kMlaPiecesPerRow == kMlaRounds * kMlaStagers, "chunk must split evenly over the staging threads");
 
-struct __attribute__((aligned(4))) MlaCodes12 { uint32_t w[3]; };
+struct __attribute__((aligned(4))) MlaCodes8 { uint32_t w[2]; };
 
 // 4 signed bytes -> two dwords of 16-bit floats (lo = bytes 0,1 ; hi = bytes 2,3)
 template <typename T> __device__ __forceinline__ void widen4(uint32_t w, uint32_t &lo, uint32_t &hi) {
@@ -92,9 +97,10 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
             for (int t = 0; t < KSTEPS; ++t) qreg[t] = load16(src + t * 32);
         }
         // ---- staging: int8 rows -> registers -> widened LDS tile.  Chunk j of the piece is loaded
-        //      into register set j & 1 two steps before it is widened.  Thread -> (key row, 12-byte
-        //      column): 8 threads per row, six pieces 96 bytes apart each, so one address per chunk
-        //      serves all loads and one LDS address all stores.  Past the end of the piece the last
+        //      into register set j & 1 two steps before it is widened.  Thread -> (key row, 8-byte
+        //      column): 8 threads per row, nine pieces 64 bytes apart each, so one address per chunk
+        //      serves all loads and one LDS address all stores (the swizzle stays inside a group of
+        //      eight units, the pieces of a thread are eight units apart).  Past the end of the piece the last
         //      chunk is named again: every step issues the same loads, so the compiler counts the
         //      loads in flight instead of waiting for all of them.  Page ids are loaded one step
         //      before the tile loads that use them and ahead of that step's tile loads, so waiting
@@ -102,7 +108,7 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
         //      argument: the step loop passes a copy the compiler cannot see through, so the few
         //      address terms are recomputed per chunk instead of held in registers.
         static_assert(kMlaStagers / 8 == kChunk && kMlaRounds * 8 == kMlaPiecesPerRow, "thread map of the staging");
-        MlaCodes12 st[2][kMlaRounds];
+        MlaCodes8 st[2][kMlaRounds];
         float st_ks[2] = {0.f, 0.f}, st_vs[2] = {0.f, 0.f};
         auto fetch_blk = [&](int j) -> int {
             int page = ((c_begin + min(j, n - 1)) * kChunk) / p.page_size;
@@ -118,20 +124,25 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
             const int last = Lk - 1 - key0;
             // wave-uniform 64-bit base + 32-bit per-thread offset
             const int8_t *src = kc + (int64_t)blk * p.k_stride_block + (int64_t)inpage0 * p.k_stride_row;
-            const uint32_t voff = (uint32_t)min(t_row, last) * (uint32_t)p.k_stride_row + t_sub * 12;
+            const uint32_t voff = (uint32_t)min(t_row, last) * (uint32_t)p.k_stride_row + t_sub * 8;
 #pragma unroll
-            for (int i = 0; i < kMlaRounds; ++i) st[set][i] = *reinterpret_cast<const MlaCodes12 *>(src + voff + i * 96);
+            for (int i = 0; i < kMlaRounds; ++i) st[set][i] = *reinterpret_cast<const MlaCodes8 *>(src + voff + i * 64);
             const int64_t so = (int64_t)blk * p.ks_stride_block + (int64_t)inpage0 * p.ks_stride_row;
             const uint32_t soff = (uint32_t)min(th & (kChunk - 1), last) * (uint32_t)p.ks_stride_row;
             st_ks[set] = (p.k_scale + so)[soff];
             st_vs[set] = (p.v_scale + so)[soff];
         };
-        // word t (0..17) of the staged chunk: four codes -> four 16-bit floats -> LDS
-        auto widen_word = [&](int tile, int set, int th, int t) {
-            uint8_t *dst = &sh.k[tile][(th >> 3) * kMlaRowBytes + (th & 7) * 24];
-            uint2 w;
-            widen4<T>(st[set][t / 3].w[t % 3], w.x, w.y);
-            *reinterpret_cast<uint2 *>(dst + (t / 3) * 192 + (t % 3) * 8) = w;
+        // piece i (0..8) of the staged chunk: eight codes -> eight 16-bit floats -> one LDS unit
+        auto widen_piece = [&](int tile, int set, int th, int i) {
+            const int row = th >> 3;
+            uint8_t *dst = &sh.k[tile][row * kMlaRowBytes + (((th & 7) ^ (row & 7)) << 4)];
+            u32x4_t w;
+            uint32_t lo, hi;
+            widen4<T>(st[set][i].w[0], lo, hi);
+            w[0] = lo, w[1] = hi;
+            widen4<T>(st[set][i].w[1], lo, hi);
+            w[2] = lo, w[3] = hi;
+            *reinterpret_cast<u32x4_t *>(dst + i * 128) = w;
         };
         auto stash_scales = [&](int tile, int set, int th) {
             if (th < kChunk) {
@@ -167,15 +178,17 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
             }
             if (do_score) {
                 // ---- S^T = K Q^T : two 16-key tiles x this wave's 16 heads; operand reads run kPf
-                //      k-steps ahead of the MFMAs that use them; one word of the next-but-one chunk
-                //      is widened beside every k-step (in the last score step that is the last chunk
+                //      k-steps ahead of the MFMAs that use them; one piece of the next-but-one chunk
+                //      is widened beside every other k-step (in the last score step that is the last chunk
                 //      once more, into a tile nobody reads: no branch inside the product loop)
                 constexpr int kPf = 8;
                 u32x4_t ka[KSTEPS][2];
-                const uint8_t *k_rd = &sh.k[tile][ln * kMlaRowBytes + lq * 16];
+                // unit 4t + lq of rows ln and 16 + ln (same row & 7), swizzled: two lane offsets by parity of t
+                const uint8_t *k_rd = &sh.k[tile][ln * kMlaRowBytes];
+                const int k_off[2] = {(lq ^ (ln & 7)) << 4, ((4 + lq) ^ (ln & 7)) << 4};
                 auto read_k = [&](int t) {
-                    ka[t][0] = *reinterpret_cast<const u32x4_t *>(k_rd + t * 64);
-                    ka[t][1] = *reinterpret_cast<const u32x4_t *>(k_rd + 16 * kMlaRowBytes + t * 64);
+                    ka[t][0] = *reinterpret_cast<const u32x4_t *>(k_rd + k_off[t & 1] + (t >> 1) * 128);
+                    ka[t][1] = *reinterpret_cast<const u32x4_t *>(k_rd + 16 * kMlaRowBytes + k_off[t & 1] + (t >> 1) * 128);
                 };
 #pragma unroll
                 for (int t = 0; t < kPf; ++t) read_k(t);
@@ -183,13 +196,13 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
                 for (int t = 0; t < KSTEPS; ++t) {
                     if (t + kPf < KSTEPS) read_k(t + kPf);
                     s[0] = mfma16<T>(ka[t][0], qreg[t], s[0]);
-                    widen_word(tile_j, set, th, t);
+                    if (t & 1) widen_piece(tile_j, set, th, t >> 1);
                     s[1] = mfma16<T>(ka[t][1], qreg[t], s[1]);
                     __builtin_amdgcn_sched_barrier(0);
                 }
             } else if (do_stash) {
 #pragma unroll
-                for (int t = 0; t < KSTEPS; ++t) widen_word(tile_j, set, th, t);
+                for (int i = 0; i < kMlaRounds; ++i) widen_piece(tile_j, set, th, i);
             }
             if (do_stash) stash_scales(tile_j, set, th);
             {
@@ -292,7 +305,9 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
                     const int row = (e >> 2) * 16 + lq * 4 + (e & 3);
-                    vr[e] = *reinterpret_cast<const u32x4_t *>(&sh.k[tile][row * kMlaRowBytes + (w4 * 128 + ln * 8) * 2]);
+                    // unit w4*16 + ln of the row, swizzled with row & 7 = 4 * (lq & 1) + (e & 3)
+                    vr[e] = *reinterpret_cast<const u32x4_t *>(
+                        &sh.k[tile][row * kMlaRowBytes + (((w4 * 16 + ln) ^ (4 * (lq & 1) + (e & 3))) << 4)]);
                 }
                 u32x4_t pkg[4];
                 const uint32_t bumps = *reinterpret_cast<const uint32_t *>(sh.bump[pb]);
