@@ -28,7 +28,7 @@ for _p in (os.path.join(ROOT, "flash-attention-npu_amd"), os.path.join(ROOT, "or
 HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E
 # HBM bytes per launch of the attention kernel from the FETCH_SIZE / WRITE_SIZE counter passes
 # (calibrated against a 1 GiB device copy); the workloads are seeded, so these are constants.
-MEASURED_TRAFFIC_BYTES = {"c2": 1237.1e6}
+MEASURED_TRAFFIC_BYTES = {"c2": 1242.0e6, "c3a": 2157.5e6}
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
 
 
@@ -197,35 +197,42 @@ def cpu_decode_baseline(w, budget_s: float = 20.0):
     h = {k: (w[k].cpu() if isinstance(w.get(k), torch.Tensor) else w.get(k)) for k in keys}
     if h["k_scale"] is not None:
         h["v_cache"] = h["k_cache"][..., :w["dv"]]
-    # bounded sample: leading batch rows until the budget is used up
+    # bounded sample: whole passes over the batch rows for at least min_s seconds, cut off inside a
+    # pass once the budget is used up
     B = w["B"]
-    rows = B
+    min_s = 10.0
     t0 = time.perf_counter()
-    done = 0
-    times = []
-    for start in range(0, B):
-        sl = slice(start, start + 1)
-        t1 = time.perf_counter()
-        O.flash_attn_with_kvcache(h["q"][sl], h["k_cache"], h["v_cache"],
-                                  None if h["k"] is None else h["k"][sl], None if h["v"] is None else h["v"][sl],
-                                  rotary_cos=h["rotary_cos"], rotary_sin=h["rotary_sin"],
-                                  cache_seqlens=h["cache_seqlens"][sl], block_table=h["block_table"][sl],
-                                  softmax_scale=w["scale"], causal=w["causal"], window_size=w["window"],
-                                  rotary_interleaved=False, k_scale_cache=h["k_scale"], mode="golden")
-        times.append(time.perf_counter() - t1)
-        done += 1
-        if time.perf_counter() - t0 > budget_s:
+    secs, bytes_done, rows_done, passes = 0.0, 0.0, 0, 0
+    while time.perf_counter() - t0 < min_s:
+        times = []
+        for start in range(0, B):
+            sl = slice(start, start + 1)
+            t1 = time.perf_counter()
+            O.flash_attn_with_kvcache(h["q"][sl], h["k_cache"], h["v_cache"],
+                                      None if h["k"] is None else h["k"][sl], None if h["v"] is None else h["v"][sl],
+                                      rotary_cos=h["rotary_cos"], rotary_sin=h["rotary_sin"],
+                                      cache_seqlens=h["cache_seqlens"][sl], block_table=h["block_table"][sl],
+                                      softmax_scale=w["scale"], causal=w["causal"], window_size=w["window"],
+                                      rotary_interleaved=False, k_scale_cache=h["k_scale"], mode="golden")
+            times.append(time.perf_counter() - t1)
+            if time.perf_counter() - t0 > budget_s:
+                break
+        done = len(times)
+        sub = dict(w)
+        sub["lens"] = w["lens"][:done]
+        sub["B"] = done
+        attn, app = decode_algorithmic_bytes(sub)
+        bytes_done += attn + app
+        secs += sum(times)
+        rows_done += done
+        passes += 1
+        if done < B:
             break
-    sub = dict(w)
-    sub["lens"] = w["lens"][:done]
-    sub["B"] = done
-    attn, app = decode_algorithmic_bytes(sub)
-    secs = sum(times)
-    return dict(value=(attn + app) / secs / 1e9, unit="GB/s", cores=torch.get_num_threads(), kind="port",
-                sample=f"oracle blocked golden (fp32 math, 512-key chunks) on the first {done} of {rows} batch rows "
-                       f"of the same workload, {secs:.2f} s on {os.cpu_count()} host cpus, "
+    return dict(value=bytes_done / secs / 1e9, unit="GB/s", cores=torch.get_num_threads(), kind="port",
+                sample=f"oracle blocked golden (fp32 math, 512-key chunks), {rows_done} batch rows of the same workload "
+                       f"({passes} passes over its {B} rows), {secs:.2f} s on {os.cpu_count()} host cpus, "
                        f"torch threads {torch.get_num_threads()}",
-                ms_per_call_extrapolated=secs / done * rows * 1e3)
+                ms_per_call_extrapolated=secs / rows_done * B * 1e3)
 
 
 # ----------------------------------------------------------------------------- main
@@ -271,7 +278,12 @@ def run_decode(args, name):
     plan = _lib.SplitPlan()
     lib.fa_rocm_plan_kvcache(C.byref(calls[0].args), lib.fa_rocm_num_cus(), C.byref(plan))
 
-    kernel_name = "decode_mla_i8_kernel" if name == "c4" else "decode_paged_kernel"
+    if name == "c4":
+        kernel_name = "decode_mla_i8_kernel"
+    elif plan.mode == 1:
+        kernel_name = "decode_wave_kernel" if plan.num_workers > plan.num_wgs else "decode_balanced_kernel"
+    else:
+        kernel_name = "decode_paged_kernel"
     out = {
         "metric": "paged_decode_hbm_bandwidth", "value": total_bytes / (ms_per_step * 1e-3) / 1e9, "unit": "GB/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
