@@ -89,7 +89,8 @@ int fa_rocm_kvcache_validate(const fa_kvcache_args *a) {
     if (a->seqlen_q <= 0 || a->nheads <= 0 || a->nheads_k <= 0) return fail(FA_ERR_SHAPE, "empty query");
     if (a->nheads % a->nheads_k != 0)
         return fail(FA_ERR_SHAPE, "Number of heads in key/value must divide number of heads in query");
-    if (a->page_size <= 0 || a->page_size % 32 != 0)
+    // 32-key chunks must not straddle pages; a table one page wide (a dense cache) cannot straddle
+    if (a->page_size <= 0 || (a->page_size % 32 != 0 && a->max_blocks_per_seq != 1))
         return fail(FA_ERR_SHAPE, "page_block_size must be a positive multiple of 32");
     if (a->num_blocks <= 0 || a->max_blocks_per_seq <= 0) return fail(FA_ERR_SHAPE, "empty block_table or cache");
     if (a->softcap < 0.f) return fail(FA_ERR_SHAPE, "softcap must be non-negative (0.0 disables softcap)");

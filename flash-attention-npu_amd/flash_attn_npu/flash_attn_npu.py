@@ -65,6 +65,24 @@ def fwd_kvcache(q, kcache, vcache, k_, v_, seqlens_k_, rotary_cos_, rotary_sin_,
     return [call.out, call.lse]
 
 
+_tables = {}
+
+
+def _identity_table(batch: int, device) -> torch.Tensor:
+    """(batch, 1) int32 table 0..batch-1, built once per (device, batch)."""
+    key = ("id", batch, str(device))
+    if key not in _tables:
+        _tables[key] = torch.arange(batch, dtype=torch.int32, device=device).view(batch, 1)
+    return _tables[key]
+
+
+def _full_lengths(batch: int, seqlen: int, device) -> torch.Tensor:
+    key = ("len", batch, seqlen, str(device))
+    if key not in _tables:
+        _tables[key] = torch.full((batch,), seqlen, dtype=torch.int32, device=device)
+    return _tables[key]
+
+
 def bind_kvcache(q, kcache, vcache, k_, v_, seqlens_k_, rotary_cos_, rotary_sin_, cache_batch_idx_, leftpad_k_,
                  block_table_, alibi_slopes_, out_, softmax_scale, is_causal, window_size_left, window_size_right,
                  softcap, is_rotary_interleaved, num_splits, k_scale_cache_=None, v_scale_cache_=None) -> KvcacheCall:
@@ -81,14 +99,29 @@ def bind_kvcache(q, kcache, vcache, k_, v_, seqlens_k_, rotary_cos_, rotary_sin_
     _require(q.stride(-1) == 1, "Input tensor q must have contiguous last dimension")
     _require(kcache.stride(-1) == 1, "Input tensor kcache must have contiguous last dimension")
     _require(vcache.stride(-1) == 1, "Input tensor vcache must have contiguous last dimension")
-    _require(block_table_ is not None, "MI355X FlashAttention supports the paged KV cache only: pass block_table")
+    # A dense cache (batch_cache, seqlen_cache, nheads_k, headdim) is a paged one with a single page
+    # per row: the table is the identity, or cache_batch_idx (flash_attn_npu_interface.py:1516-1519).
+    dense = block_table_ is None
+    if dense:
+        _require(q.dim() == 4 and kcache.dim() == 4, "q, kcache and vcache must be 4-D")
+        if cache_batch_idx_ is not None:
+            _require(cache_batch_idx_.dtype == torch.int32 and cache_batch_idx_.dim() == 1
+                     and cache_batch_idx_.shape[0] == q.shape[0], "cache_batch_idx must be (batch_size,) int32")
+            block_table_ = cache_batch_idx_.contiguous().view(-1, 1)
+        else:
+            _require(kcache.shape[0] >= q.shape[0], "batch size of the cache must be at least that of q")
+            block_table_ = _identity_table(q.shape[0], q.device)
+        if seqlens_k_ is None:
+            _require(k_ is None, "cache_seqlens must be given to append k / v")
+            seqlens_k_ = _full_lengths(q.shape[0], kcache.shape[1], q.device)
+    else:
+        _require(cache_batch_idx_ is None, "Paged KVcache does not support cache_batch_idx")
     _require(block_table_.dtype == torch.int32, "block_table must have dtype int32")
     _require(block_table_.stride(-1) == 1, "block_table must have contiguous last dimension")
     _require(seqlens_k_ is not None, "cache_seqlens must be given with a paged KV cache")
     _require(seqlens_k_.dtype == torch.int32, "seqlens_k must have dtype int32")
     _require(alibi_slopes_ is None, "NPU FlashAttention does not support alibi_slopes")
     _require(leftpad_k_ is None, "NPU FlashAttention does not support leftpad_k")
-    _require(cache_batch_idx_ is None, "MI355X FlashAttention does not support cache_batch_idx")
     _require(softcap >= 0.0, "softcap must be non-negative (0.0 disables softcap)")
     _require(q.dim() == 4 and kcache.dim() == 4 and vcache.dim() == 4, "q, kcache and vcache must be 4-D")
     _require_device(q, kcache, vcache, k_, v_, seqlens_k_, block_table_, rotary_cos_, rotary_sin_)

@@ -257,11 +257,13 @@ def flash_attn_with_kvcache(
     k_scale_cache: Optional[torch.Tensor] = None,
     v_scale_cache: Optional[torch.Tensor] = None,
 ):
-    """Attention of q over a paged KV cache, with optional in-place append of k / v.
+    """Attention of q over a KV cache, with optional in-place append of k / v.
 
     q: (batch, seqlen, nheads, headdim).  k_cache / v_cache: (num_blocks, page_block_size, nheads_k,
-    headdim) addressed through block_table (batch, max_num_blocks_per_seq) int32; cache_seqlens: int or
-    (batch,) int32 keys already cached per row.  If k, v (batch, seqlen_new, nheads_k, headdim) are
+    headdim) addressed through block_table (batch, max_num_blocks_per_seq) int32, or, without a
+    block_table, (batch_cache, seqlen_cache, nheads_k, headdim) with row b of q using cache row b (or
+    cache_batch_idx[b], (batch,) int32); cache_seqlens: int or (batch,) int32 keys already cached per
+    row (a dense cache without it counts as full).  If k, v (batch, seqlen_new, nheads_k, headdim) are
     given they are written into the cache at positions cache_seqlens .. cache_seqlens+seqlen_new-1
     (the caller guarantees the pages exist) and attention sees cache_seqlens + seqlen_new keys;
     cache_seqlens itself is not changed.  With rotary_cos / rotary_sin (seqlen_ro, rotary_dim/2, dtype
@@ -269,7 +271,8 @@ def flash_attn_with_kvcache(
     cache_seqlens (otherwise); rotary_interleaved pairs dims (2c, 2c+1), else (c, c + rotary_dim/2).
     GQA/MQA, bottom-right causal mask, window_size, softcap and softmax_scale (default
     headdim**-0.5) as in flash_attn_varlen_func.  num_splits: 0 = heuristic, 1 = no KV split,
-    n > 1 = at most n splits.  cache_batch_idx, cache_leftpad and alibi_slopes are not supported.
+    n > 1 = at most n splits.  cache_leftpad, alibi_slopes and cache_batch_idx with a block_table are
+    not supported.
     An int8 k_cache (one latent kv head, 576 dims, v_cache = k_cache[..., :512]) needs
     k_scale_cache (num_blocks, page_block_size, 1) fp32 per-token scales.
 

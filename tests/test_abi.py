@@ -126,8 +126,10 @@ def test_operator_layer_fails_loudly_without_gpu_tensors():
         flash_attn_with_kvcache(q, kc, kc, cache_seqlens=5, block_table=bt)
     with pytest.raises(RuntimeError, match="FP16 and BF16"):
         flash_attn_with_kvcache(q.float(), kc.float(), kc.float(), cache_seqlens=5, block_table=bt)
-    with pytest.raises(RuntimeError, match="block_table"):
-        flash_attn_with_kvcache(q, kc, kc, cache_seqlens=5)
+    with pytest.raises(RuntimeError, match="ROCm device"):
+        flash_attn_with_kvcache(q, kc, kc, cache_seqlens=5)   # dense cache: valid call, still no CPU path
+    with pytest.raises(RuntimeError, match="Paged KVcache does not support cache_batch_idx"):
+        flash_attn_with_kvcache(q, kc, kc, cache_seqlens=5, block_table=bt, cache_batch_idx=torch.zeros(1, dtype=torch.int32))
     with pytest.raises(RuntimeError, match="alibi"):
         flash_attn_with_kvcache(q, kc, kc, cache_seqlens=5, block_table=bt, alibi_slopes=torch.zeros(8))
     with pytest.raises(RuntimeError, match="leftpad"):
