@@ -58,11 +58,70 @@ def fwd_kvcache(q, kcache, vcache, k_, v_, seqlens_k_, rotary_cos_, rotary_sin_,
                 softcap, is_rotary_interleaved, num_splits, k_scale_cache_=None, v_scale_cache_=None
                 ) -> List[torch.Tensor]:
     """mha_fwd_kvcache (flash_api.cpp:356-637) on a paged cache.  Returns [out, softmax_lse]."""
+    if (isinstance(q, torch.Tensor) and q.dim() == 4 and kcache.dtype != torch.int8
+            and q.shape[-1] not in (64, 128, 256) and q.shape[-1] <= 256 and q.shape[-1] == kcache.shape[-1]
+            and q.dtype in (torch.bfloat16, torch.float16) and q.is_cuda and kcache.is_cuda):
+        return _fwd_kvcache_padded(q, kcache, vcache, k_, v_, seqlens_k_, rotary_cos_, rotary_sin_, cache_batch_idx_,
+                                   leftpad_k_, block_table_, alibi_slopes_, out_, softmax_scale, is_causal,
+                                   window_size_left, window_size_right, softcap, is_rotary_interleaved, num_splits)
     call = bind_kvcache(q, kcache, vcache, k_, v_, seqlens_k_, rotary_cos_, rotary_sin_, cache_batch_idx_, leftpad_k_,
                         block_table_, alibi_slopes_, out_, softmax_scale, is_causal, window_size_left,
                         window_size_right, softcap, is_rotary_interleaved, num_splits, k_scale_cache_, v_scale_cache_)
     call.run()
     return [call.out, call.lse]
+
+
+def _fwd_kvcache_padded(q, kcache, vcache, k_, v_, seqlens_k_, rotary_cos_, rotary_sin_, cache_batch_idx_, leftpad_k_,
+                        block_table_, alibi_slopes_, out_, softmax_scale, is_causal, window_size_left,
+                        window_size_right, softcap, is_rotary_interleaved, num_splits) -> List[torch.Tensor]:
+    """Head dimensions the kernels are not built for (the reference's tests go down to 1 and 4,
+    tests/test_flash_attn_npu_v2.py:178-183): zero-padded COPIES of q and of the caches go through the
+    kernels (zero columns change neither the scores nor the kept output columns), then the rows the
+    call appended are copied back into the caller's caches.  A slow path: it copies the whole cache."""
+    import torch.nn.functional as F
+    d, dv = q.shape[-1], vcache.shape[-1]
+    dp = 64 if max(d, dv) <= 64 else (128 if max(d, dv) <= 128 else 256)
+    _require(kcache.dim() == 4 and vcache.dim() == 4, "q, kcache and vcache must be 4-D")
+    _require(dv == d, "k and v head dimensions must match")
+
+    def pad(x):
+        return None if x is None else F.pad(x, (0, dp - x.shape[-1]))
+
+    kc_p, vc_p = pad(kcache), pad(vcache)
+    out_p, lse = fwd_kvcache(pad(q), kc_p, vc_p, pad(k_), pad(v_), seqlens_k_, rotary_cos_, rotary_sin_,
+                             cache_batch_idx_, leftpad_k_, block_table_, alibi_slopes_, None, softmax_scale, is_causal,
+                             window_size_left, window_size_right, softcap, is_rotary_interleaved, num_splits)
+    if k_ is not None:
+        # positions the call wrote, computed on the device (no host sync); rows without capacity are
+        # redirected to the first written row with that row's values, so duplicates agree
+        B, snew = k_.shape[0], k_.shape[1]
+        page, nblk = kcache.shape[1], kcache.shape[0]
+        if block_table_ is None:
+            table = (cache_batch_idx_.view(-1, 1) if cache_batch_idx_ is not None else _identity_table(B, q.device))
+        else:
+            table = block_table_
+        pos = seqlens_k_.to(torch.int64).view(B, 1) + torch.arange(snew, device=q.device, dtype=torch.int64).view(1, snew)
+        pg = pos // page
+        blk = table.to(torch.int64).gather(1, pg.clamp(max=table.shape[1] - 1))
+        ok = ((pg < table.shape[1]) & (blk >= 0) & (blk < nblk)).view(-1)
+        n = ok.numel()
+        first = torch.argmax(ok.to(torch.int32))
+        sel = torch.where(ok, torch.arange(n, device=q.device), first)
+        blk_s = blk.view(-1)[sel].clamp(0, nblk - 1)
+        row_s = (pos % page).view(-1)[sel]
+        any_ok = ok.any()
+        for cache, cache_p, width in ((kcache, kc_p, d), (vcache, vc_p, dv)):
+            new = cache_p[blk_s, row_s][..., :width]
+            cache[blk_s, row_s] = torch.where(any_ok, new, cache[blk_s, row_s])
+    out = out_p[..., :dv]
+    if out_ is not None:
+        _require(out_.dtype == q.dtype and tuple(out_.shape) == tuple(out.shape),
+                 "out must have shape (batch_size, seqlen_q, num_heads, head_size_v) and the dtype of q")
+        out_.copy_(out)
+        out = out_
+    else:
+        out = out.contiguous()
+    return [out, lse]
 
 
 _tables = {}

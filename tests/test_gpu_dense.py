@@ -121,3 +121,35 @@ def test_dense_rejections():
     with pytest.raises(RuntimeError, match="Paged KVcache does not support cache_batch_idx"):
         flash_attn_with_kvcache(dev["q"], dev["k_cache"], dev["v_cache"], cache_seqlens=dev["cache_seqlens"],
                                 block_table=bt, cache_batch_idx=torch.zeros(2, dtype=torch.int32, device="cuda"))
+
+
+@pytest.mark.parametrize("d,hq,hk,sq,s_cache,window", [(4, 512, 1, 1, 1024, (542, 647)), (4, 512, 1, 1, 1024, (-1, -1)),
+                                                      (1, 4, 2, 4, 4096, (826, 973)), (96, 8, 2, 1, 640, (-1, -1)),
+                                                      (192, 8, 4, 3, 300, (-1, -1))])
+def test_dense_odd_head_dims(d, hq, hk, sq, s_cache, window):
+    # head dimensions outside 64/128/256 (the reference's tests use 4 and 1,
+    # tests/test_flash_attn_npu_v2.py:178-183) run on zero-padded copies
+    case = make_dense_case(2, hq, hk, d, s_cache, [s_cache, s_cache // 3], seqlen_q=sq, dtype=torch.float16, seed=26)
+    got, ref, gold, _ = run_dense(case, causal=True, window_size=window)
+    assert got[0].shape[-1] == d
+    check_out(got[0], ref[0], got[1], ref[1], f"d={d}")
+
+
+def test_paged_odd_head_dim_append_written_back():
+    from flash_attn_npu import flash_attn_with_kvcache
+    from helpers import make_paged_case, to_dev
+    case = make_paged_case(3, 6, 2, 80, 128, [100, 255, 128], seqlen_new=2, seed=27)
+    case["cache_seqlens"][2] = 128   # second page of row 2 starts with the appended rows
+    dev = to_dev(case)
+    before_k = dev["k_cache"].clone()
+    out, lse = flash_attn_with_kvcache(dev["q"], dev["k_cache"], dev["v_cache"], dev["k"], dev["v"],
+                                       cache_seqlens=dev["cache_seqlens"], block_table=dev["block_table"], causal=True,
+                                       return_softmax_lse=True)
+    torch.cuda.synchronize()
+    kc, vc = case["k_cache"].clone(), case["v_cache"].clone()
+    ref, ref_lse = O.flash_attn_with_kvcache(case["q"], kc, vc, case["k"], case["v"], cache_seqlens=case["cache_seqlens"],
+                                             block_table=case["block_table"], causal=True, mode="fp32")
+    assert torch.equal(dev["k_cache"].cpu().view(torch.int16), kc.view(torch.int16))
+    assert torch.equal(dev["v_cache"].cpu().view(torch.int16), vc.view(torch.int16))
+    assert not torch.equal(dev["k_cache"], before_k)
+    check_out(out, ref, lse, ref_lse, "d=80 append")
