@@ -66,6 +66,55 @@ __global__ void __launch_bounds__(64) append_kv_kernel(const AppendParams p) {
     for (int d = threadIdx.x; d < p.headdim_v; d += 64) vdst[d] = vsrc[d];
 }
 
+// Quantising append into the int8 latent cache: one wave per new token.
+//   scale = absmax / 127 (fp32, correctly rounded division); code = clamp(rne(x / scale), -127, 127);
+//   an all-zero token gets scale 0 and codes 0.
+// The codes go to k_cache (v_cache is a view of it), the scale to k_scale (and to v_scale when that
+// is a separate tensor).  Every operation is a single correctly rounded fp32 operation, so codes
+// and scales can be compared bit-for-bit with a host computation.
+template <typename T>
+__global__ void __launch_bounds__(64) append_quant_i8_kernel(const AppendParams p) {
+    const int t = blockIdx.x;
+    const int b = blockIdx.y;
+    const int lane = threadIdx.x;
+    const int pos = p.cache_seqlens[b] + t;
+    if (pos < 0) return;
+    const int page = pos / p.page_size;
+    if (page >= p.max_blocks) return;   // no capacity: nothing is written
+    const int blk = p.block_table[(int64_t)b * p.bt_stride_b + page];
+    if (blk < 0 || blk >= p.num_blocks) return;
+    const int inpage = pos - page * p.page_size;
+    const int d = p.headdim_qk;
+
+    const uint16_t *src = reinterpret_cast<const uint16_t *>(p.k_new) + (int64_t)b * p.kn_stride_b + (int64_t)t * p.kn_stride_s;
+    int8_t *dst = reinterpret_cast<int8_t *>(p.k_cache) + (int64_t)blk * p.k_stride_block + (int64_t)inpage * p.k_stride_row;
+
+    float absmax = 0.f;
+    for (int e = lane; e < d; e += 64) absmax = fmaxf(absmax, fabsf(to_float<T>(src[e])));
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) absmax = fmaxf(absmax, __shfl_xor(absmax, m, 64));
+    const float scale = __fdiv_rn(absmax, 127.0f);
+    for (int e = lane; e < d; e += 64) {
+        float c = 0.f;
+        if (scale > 0.f) c = fminf(fmaxf(rintf(__fdiv_rn(to_float<T>(src[e]), scale)), -127.f), 127.f);
+        dst[e] = (int8_t)(int)c;
+    }
+    if (lane == 0) {
+        const int64_t so = (int64_t)blk * p.ks_stride_block + (int64_t)inpage * p.ks_stride_row;
+        p.k_scale[so] = scale;
+        if (p.v_scale && p.v_scale != p.k_scale) p.v_scale[so] = scale;
+    }
+}
+
+hipError_t launch_append_quant_i8(const AppendParams &p, int dtype, hipStream_t stream) {
+    dim3 grid(p.seqlen_new, p.batch);
+    if (dtype == 0)
+        hipLaunchKernelGGL(append_quant_i8_kernel<BF16>, grid, dim3(64), 0, stream, p);
+    else
+        hipLaunchKernelGGL(append_quant_i8_kernel<FP16>, grid, dim3(64), 0, stream, p);
+    return hipGetLastError();
+}
+
 hipError_t launch_append_kv(const AppendParams &p, int dtype, hipStream_t stream) {
     dim3 grid(p.nheads_k, p.seqlen_new, p.batch);
     if (dtype == 0)

@@ -54,6 +54,8 @@ struct AppendParams {
     const void *v_new;
     const void *rotary_cos;
     const void *rotary_sin;
+    float *k_scale;      // int8 latent cache: per-token scales written by the quantising append
+    float *v_scale;
     const int32_t *cache_seqlens;
     const int32_t *block_table;
     int32_t batch, seqlen_new, nheads_k, headdim_qk, headdim_v;
@@ -63,6 +65,7 @@ struct AppendParams {
     int64_t v_stride_block, v_stride_row, v_stride_h;
     int64_t kn_stride_b, kn_stride_s, kn_stride_h;
     int64_t vn_stride_b, vn_stride_s, vn_stride_h;
+    int64_t ks_stride_block, ks_stride_row;
     int64_t bt_stride_b;
 };
 
@@ -95,6 +98,7 @@ struct PrefillParams {
 
 // dtype: 0 = bf16, 1 = fp16 (enum fa_dtype).  All return hipError_t of the launch.
 hipError_t launch_append_kv(const AppendParams &p, int dtype, hipStream_t stream);
+hipError_t launch_append_quant_i8(const AppendParams &p, int dtype, hipStream_t stream);
 hipError_t launch_decode_paged(const DecodeParams &p, int dtype, int headdim, hipStream_t stream);
 hipError_t launch_decode_wave(const DecodeParams &p, int dtype, int headdim, hipStream_t stream);
 hipError_t launch_splitkv_combine(const DecodeParams &p, int dtype, int headdim_v, hipStream_t stream);

@@ -99,7 +99,12 @@ int fa_rocm_kvcache_validate(const fa_kvcache_args *a) {
         if (!a->k_scale_cache) return fail(FA_ERR_NULL, "int8 KV cache needs k_scale_cache");
         if (a->headdim_qk != 576 || a->headdim_v != 512 || a->nheads_k != 1)
             return fail(FA_ERR_SHAPE, "int8 KV cache supports the latent layout only (1 kv head, 576/512 dims)");
-        if (a->k_new) return fail(FA_ERR_UNSUPPORTED, "append into an int8 KV cache is not supported");
+        if (a->k_new) {
+            // quantising append: new latent rows in the I/O dtype; v is the view k[..., :512] like the cache
+            if (a->v_new != a->k_new || a->vn_stride_b != a->kn_stride_b || a->vn_stride_s != a->kn_stride_s)
+                return fail(FA_ERR_UNSUPPORTED, "int8 KV cache: v must be the view k[..., :512] of the new latent rows");
+            if (a->rotary_cos) return fail(FA_ERR_UNSUPPORTED, "rotary embedding is not supported with an int8 KV cache");
+        }
         if (a->seqlen_q != 1 || a->nheads % 64 != 0)
             return fail(FA_ERR_SHAPE, "int8 KV cache needs seqlen_q == 1 and a multiple of 64 query heads");
         if (a->v_cache != a->k_cache || a->v_stride_block != a->k_stride_block || a->v_stride_row != a->k_stride_row)
@@ -224,6 +229,11 @@ static void fill_append(const fa_kvcache_args *a, fa::AppendParams &p) {
     p.vn_stride_s = a->vn_stride_s;
     p.vn_stride_h = a->vn_stride_h;
     p.bt_stride_b = a->bt_stride_b;
+    // the scale tensors are inputs of attention and outputs of the quantising append
+    p.k_scale = const_cast<float *>(static_cast<const float *>(a->k_scale_cache));
+    p.v_scale = const_cast<float *>(static_cast<const float *>(a->v_scale_cache));
+    p.ks_stride_block = a->ks_stride_block;
+    p.ks_stride_row = a->ks_stride_row;
 }
 
 int fa_rocm_append_kv(const fa_kvcache_args *a, void *stream) {
@@ -232,7 +242,8 @@ int fa_rocm_append_kv(const fa_kvcache_args *a, void *stream) {
     if (!a->k_new) return FA_OK;
     fa::AppendParams p;
     fill_append(a, p);
-    const hipError_t e = fa::launch_append_kv(p, a->io_dtype, static_cast<hipStream_t>(stream));
+    const hipError_t e = is_mla_i8(a) ? fa::launch_append_quant_i8(p, a->io_dtype, static_cast<hipStream_t>(stream))
+                                      : fa::launch_append_kv(p, a->io_dtype, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return fail(FA_ERR_LAUNCH, "append_kv launch failed: %s", hipGetErrorString(e));
     return FA_OK;
 }

@@ -228,6 +228,11 @@ def bind_kvcache(q, kcache, vcache, k_, v_, seqlens_k_, rotary_cos_, rotary_sin_
         _require(k_.dtype == q.dtype and v_.dtype == q.dtype, "Key and value must have the same dtype as query")
         _require(k_.dim() == 4 and k_.shape[0] == B and k_.shape[2] == hk and k_.shape[3] == d
                  and tuple(v_.shape) == (B, k_.shape[1], hk, dv), "k / v must be (batch_size, seqlen_new, nheads_k, headdim)")
+        if is_i8:
+            # quantising append: the new latent rows come in the I/O dtype, v aliased like the cache
+            _require(k_.stride(-1) == 1 and v_.data_ptr() == k_.data_ptr() and v_.stride() == k_.stride(),
+                     "int8 KV cache: v must be the view k[..., :512] of the new latent rows")
+            _require(rotary_cos_ is None and rotary_sin_ is None, "rotary embedding is not supported with an int8 KV cache")
         k_ = k_ if k_.stride(-1) == 1 else k_.contiguous()
         v_ = v_ if v_.stride(-1) == 1 else v_.contiguous()
         keep += [k_, v_]

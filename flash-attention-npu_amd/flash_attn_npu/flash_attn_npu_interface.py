@@ -274,7 +274,8 @@ def flash_attn_with_kvcache(
     n > 1 = at most n splits.  cache_leftpad, alibi_slopes and cache_batch_idx with a block_table are
     not supported.
     An int8 k_cache (one latent kv head, 576 dims, v_cache = k_cache[..., :512]) needs
-    k_scale_cache (num_blocks, page_block_size, 1) fp32 per-token scales.
+    k_scale_cache (num_blocks, page_block_size, 1) fp32 per-token scales; k (dtype of q, with
+    v = k[..., :512]) is then quantised per token (scale = absmax / 127) and appended with its scale.
 
     Returns out (batch, seqlen, nheads, headdim_v), or (out, softmax_lse (batch, nheads, seqlen) fp32)
     when return_softmax_lse=True.  Does not support backward.

@@ -52,7 +52,8 @@ typedef struct fa_kvcache_args {
     float *softmax_lse;          /* (B, Hq, Sq) fp32, natural log; +inf for rows with no key     */
     void *k_cache;               /* (num_blocks, page, Hk, Dqk) kv dtype; written when k_new set */
     void *v_cache;               /* (num_blocks, page, Hk, Dv)  kv dtype; may alias k_cache      */
-    const float *k_scale_cache;  /* (num_blocks, page, Hk) fp32 per-token scale; int8 cache only */
+    const float *k_scale_cache;  /* (num_blocks, page, Hk) fp32 per-token scale; int8 cache only;
+                                    written for the appended tokens when k_new is given         */
     const float *v_scale_cache;  /* same for V; NULL = use k_scale_cache                         */
     const void *k_new;           /* (B, Snew, Hk, Dqk) io dtype or NULL                          */
     const void *v_new;           /* (B, Snew, Hk, Dv)  io dtype or NULL                          */

@@ -29,7 +29,9 @@ Pin status (what independent check holds each function; see tests/test_oracle_*.
   ref_flash_attention   torch.softmax / torch.logsumexp in fp64 on the same inputs
   attention_fp32        same library routines
   combine_splits        logsumexp identity; split == unsplit
-  append_kv             brute-force scalar loop, bit-exact; untouched bytes unchanged
+  append_kv             brute-force scalar loop, bit-exact; untouched bytes unchanged; the
+                        quantising form: scalar-loop codes and scales per appended token,
+                        attention equal to a cache quantised with the rows in place
   apply_rotary          complex-multiplication form, identity cases, norm preservation
   quantize_per_token    brute-force scalar loop, bit-exact codes
   The reference has no implementation or test of append, rotary or int8 KV: for
@@ -136,20 +138,30 @@ def apply_rotary(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, position
 def append_kv(k_cache: torch.Tensor, v_cache: torch.Tensor, k_new: torch.Tensor, v_new: torch.Tensor,
               cache_seqlens: torch.Tensor, block_table: torch.Tensor,
               rotary_cos: Optional[torch.Tensor] = None, rotary_sin: Optional[torch.Tensor] = None,
-              rotary_interleaved: bool = True) -> None:
+              rotary_interleaved: bool = True, k_scale_cache: Optional[torch.Tensor] = None,
+              v_scale_cache: Optional[torch.Tensor] = None) -> None:
     """In-place paged append (flash_attn_npu_interface.py:1460-1467,1508-1510).
 
     For t < Snew: p = cache_seqlens[b] + t;
-        k_cache[bt[b, p // page], p % page] = rope(k_new[b, t], pos=p);  v likewise without rope."""
+        k_cache[bt[b, p // page], p % page] = rope(k_new[b, t], pos=p);  v likewise without rope.
+    int8 latent cache (k_scale_cache given; v_cache is a view of k_cache): the new rows are
+    quantised per token (quantize_per_token) and codes and scale are written at the same place."""
     B, snew = k_new.shape[0], k_new.shape[1]
     page = k_cache.shape[1]
     for b in range(B):
         base = int(cache_seqlens[b])
         pos = base + torch.arange(snew)
+        blk = block_table[b].to(torch.long)[pos // page]
+        if k_scale_cache is not None:
+            code, scale = quantize_per_token(k_new[b])          # (snew, Hk, d), (snew, Hk)
+            k_cache[blk, pos % page] = code
+            k_scale_cache[blk, pos % page] = scale
+            if v_scale_cache is not None and v_scale_cache.data_ptr() != k_scale_cache.data_ptr():
+                v_scale_cache[blk, pos % page] = scale
+            continue
         kb = k_new[b]
         if rotary_cos is not None:
             kb = apply_rotary(kb, rotary_cos, rotary_sin, pos, rotary_interleaved)
-        blk = block_table[b].to(torch.long)[pos // page]
         k_cache[blk, pos % page] = kb
         v_cache[blk, pos % page] = v_new[b]
 
@@ -314,7 +326,8 @@ def flash_attn_with_kvcache(q, k_cache, v_cache, k=None, v=None, rotary_cos=None
     snew = 0
     if k is not None:
         snew = k.shape[1]
-        append_kv(k_cache, v_cache, k, v, cache_seqlens, block_table, rotary_cos, rotary_sin, rotary_interleaved)
+        append_kv(k_cache, v_cache, k, v, cache_seqlens, block_table, rotary_cos, rotary_sin, rotary_interleaved,
+                  k_scale_cache, v_scale_cache)
     if softmax_scale is None:
         softmax_scale = d ** (-0.5)
     lens = [int(x) + snew for x in cache_seqlens]

@@ -65,3 +65,44 @@ def test_mla_codes_and_scales_untouched():
     flash_attn_with_kvcache(case["q"].cuda(), kc, kc[..., :512], cache_seqlens=case["cache_seqlens"].cuda(),
                             block_table=case["block_table"].cuda(), softmax_scale=192 ** -0.5, causal=True, k_scale_cache=ks)
     assert torch.equal(kc.cpu(), case["k_cache"]) and torch.equal(ks.cpu(), case["k_scale"])
+
+
+@pytest.mark.parametrize("snew", [1, 3])
+def test_mla_quantising_append_bit_exact(snew):
+    # new latent rows are quantised per token on the device: codes, scales and every untouched byte
+    # must equal the oracle's; attention then sees cache_seqlens + snew keys
+    from flash_attn_npu import flash_attn_with_kvcache
+    lens = [700, 255, 0, 2047]
+    case = mla_case(4, 128, [l + snew for l in lens], seed=5)      # pages sized for the appended rows
+    case["cache_seqlens"] = torch.tensor(lens, dtype=torch.int32)
+    g = torch.Generator().manual_seed(55)
+    k_new = torch.randn(4, snew, 1, 576, generator=g).to(torch.bfloat16)
+    k_new[1, 0] = 0                                                 # an all-zero new token
+    kc, ks = case["k_cache"].cuda(), case["k_scale"].cuda()
+    kn = k_new.cuda()
+    out, lse = flash_attn_with_kvcache(case["q"].cuda(), kc, kc[..., :512], kn, kn[..., :512],
+                                       cache_seqlens=case["cache_seqlens"].cuda(), block_table=case["block_table"].cuda(),
+                                       softmax_scale=192 ** -0.5, causal=True, return_softmax_lse=True, k_scale_cache=ks)
+    torch.cuda.synchronize()
+    kc_o, ks_o = case["k_cache"].clone(), case["k_scale"].clone()
+    ref, ref_lse = O.flash_attn_with_kvcache(case["q"], kc_o, kc_o[..., :512], k_new, k_new[..., :512],
+                                             cache_seqlens=case["cache_seqlens"], block_table=case["block_table"],
+                                             softmax_scale=192 ** -0.5, causal=True, k_scale_cache=ks_o, mode="fp32")
+    assert torch.equal(kc.cpu(), kc_o), "codes differ"
+    assert torch.equal(ks.cpu().view(torch.int32), ks_o.view(torch.int32)), "scales differ"
+    assert not torch.equal(kc_o, case["k_cache"])
+    check_out(out, ref, lse, ref_lse, "mla append")
+
+
+def test_mla_append_rejections():
+    from flash_attn_npu import flash_attn_with_kvcache
+    case = mla_case(1, 64, [40], seed=6)
+    kc, ks = case["k_cache"].cuda(), case["k_scale"].cuda()
+    kn = torch.zeros(1, 1, 1, 576, dtype=torch.bfloat16, device="cuda")
+    vn = torch.zeros(1, 1, 1, 512, dtype=torch.bfloat16, device="cuda")
+    kw = dict(cache_seqlens=case["cache_seqlens"].cuda(), block_table=case["block_table"].cuda(), k_scale_cache=ks)
+    with pytest.raises(RuntimeError, match="v must be the view"):
+        flash_attn_with_kvcache(case["q"].cuda(), kc, kc[..., :512], kn, vn, **kw)
+    cos = torch.ones(64, 32, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(RuntimeError, match="rotary embedding is not supported with an int8"):
+        flash_attn_with_kvcache(case["q"].cuda(), kc, kc[..., :512], kn, kn[..., :512], rotary_cos=cos, rotary_sin=cos, **kw)

@@ -146,3 +146,47 @@ def test_combine_splits_identity():
         assert (out - full).abs().max() < 1e-5 and (lse.T - full_lse).abs().max() < 1e-5
     out, lse = O.combine_splits(torch.zeros(3, 1, 4, 16), torch.full((3, 1, 4), float("inf")))
     assert (out == 0).all() and torch.isinf(lse).all() and (lse > 0).all()
+
+
+def test_quantising_append_brute_force():
+    """int8 latent cache: appended rows hold the scalar-loop codes and scale of their token at
+    p = cache_seqlens[b] + t, nothing else changes, and attention over the appended cache equals
+    attention over a cache that was quantised with the rows already in place."""
+    g = torch.Generator().manual_seed(7)
+    B, page, d, snew = 2, 32, 576, 2
+    lens = [30, 5]
+    latent = torch.randn(4, page, 1, d, generator=g).to(torch.bfloat16)
+    bt = torch.tensor([[2, 0], [3, 1]], dtype=torch.int32)
+    k_new = torch.randn(B, snew, 1, d, generator=g).to(torch.bfloat16)
+    k_new[1, 1] = 0
+    code, scale = O.quantize_per_token(latent)
+    kc, ks = code.clone(), scale.clone()
+    O.append_kv(kc, kc[..., :512], k_new, k_new[..., :512], torch.tensor(lens, dtype=torch.int32), bt, k_scale_cache=ks)
+    touched = torch.zeros(4, page, dtype=torch.bool)
+    for b in range(B):
+        for t in range(snew):
+            p = lens[b] + t
+            blk, row = int(bt[b][p // page]), p % page
+            x = k_new[b, t, 0].to(torch.float32)
+            absmax = float(x.abs().max())
+            sc = torch.tensor(absmax, dtype=torch.float32) / 127.0
+            assert ks[blk, row, 0].item() == sc.item()
+            for e in range(0, d, 37):       # sampled scalar loop
+                want = 0 if sc == 0 else max(-127, min(127, int(torch.round(x[e] / sc))))
+                assert int(kc[blk, row, 0, e]) == want
+            touched[blk, row] = True
+    assert torch.equal(kc[~touched], code[~touched]) and torch.equal(ks[~touched], scale[~touched])
+    # same attention as a cache built with the new rows in place before quantisation
+    full = latent.clone()
+    for b in range(B):
+        for t in range(snew):
+            p = lens[b] + t
+            full[int(bt[b][p // page]), p % page] = k_new[b, t]
+    code2, scale2 = O.quantize_per_token(full)
+    q = torch.randn(B, 1, 8, d, generator=g).to(torch.bfloat16)
+    kc3, ks3 = code.clone(), scale.clone()
+    a, la = O.flash_attn_with_kvcache(q, kc3, kc3[..., :512], k_new, k_new[..., :512], cache_seqlens=torch.tensor(lens, dtype=torch.int32),
+                                      block_table=bt, causal=True, k_scale_cache=ks3, mode="fp32")
+    b2, lb = O.flash_attn_with_kvcache(q, code2, code2[..., :512], cache_seqlens=torch.tensor([l + snew for l in lens], dtype=torch.int32),
+                                       block_table=bt, causal=True, k_scale_cache=scale2, mode="fp32")
+    assert torch.equal(a, b2) and torch.equal(la, lb)
