@@ -233,6 +233,81 @@ def flash_attn_varlen_func(
     )
 
 
+_cu_cache = {}
+
+
+def _even_cu_seqlens(batch: int, seqlen: int, device) -> torch.Tensor:
+    """cu_seqlens of `batch` sequences of `seqlen` tokens each, built once per (batch, seqlen, device)."""
+    key = (batch, seqlen, str(device))
+    if key not in _cu_cache:
+        _cu_cache[key] = torch.arange(0, (batch + 1) * seqlen, max(seqlen, 1), dtype=torch.int32, device=device)[: batch + 1]
+    return _cu_cache[key]
+
+
+def flash_attn_func(
+    q,
+    k,
+    v,
+    dropout_p=0.0,
+    softmax_scale=None,
+    causal=False,
+    window_size=(-1, -1),  # -1 means infinite context window
+    softcap=0.0,  # 0.0 means deactivated
+    alibi_slopes=None,
+    deterministic=False,
+    return_attn_probs=False,
+):
+    """Attention forward over dense batches (reference flash_attn_npu_interface.py:1109-1183; forward only).
+
+    q: (batch, seqlen_q, nheads, headdim); k, v: (batch, seqlen_k, nheads_k, headdim).  Runs on the
+    varlen kernel as `batch` sequences of equal length; masks, GQA, softcap and softmax_scale as in
+    flash_attn_varlen_func.  Returns out (batch, seqlen_q, nheads, headdim), or (out, softmax_lse
+    (batch, nheads, seqlen_q) fp32, S_dmask (empty)) when return_attn_probs=True.
+    """
+    assert q.dim() == 4 and k.dim() == 4 and v.dim() == 4, "q, k, v must be (batch, seqlen, nheads, headdim)"
+    B, sq, hq, d = q.shape
+    sk = k.shape[1]
+    res = flash_attn_varlen_func(
+        q.reshape(B * sq, hq, d), k.reshape(B * sk, k.shape[2], d), v.reshape(B * sk, v.shape[2], v.shape[3]),
+        _even_cu_seqlens(B, sq, q.device), _even_cu_seqlens(B, sk, q.device), sq, sk, dropout_p, softmax_scale, causal,
+        window_size, softcap, alibi_slopes, deterministic, return_attn_probs,
+    )
+    if not return_attn_probs:
+        return res.reshape(B, sq, hq, -1)
+    out, lse, s_dmask = res
+    return out.reshape(B, sq, hq, -1), lse.reshape(hq, B, sq).permute(1, 0, 2).contiguous(), s_dmask
+
+
+def flash_attn_kvpacked_func(q, kv, dropout_p=0.0, softmax_scale=None, causal=False, window_size=(-1, -1), softcap=0.0,
+                             alibi_slopes=None, deterministic=False, return_attn_probs=False):
+    """flash_attn_func with kv: (batch, seqlen_k, 2, nheads_k, headdim) (reference :1031-1106; forward only)."""
+    return flash_attn_func(q, kv[:, :, 0], kv[:, :, 1], dropout_p, softmax_scale, causal, window_size, softcap,
+                           alibi_slopes, deterministic, return_attn_probs)
+
+
+def flash_attn_qkvpacked_func(qkv, dropout_p=0.0, softmax_scale=None, causal=False, window_size=(-1, -1), softcap=0.0,
+                              alibi_slopes=None, deterministic=False, return_attn_probs=False):
+    """flash_attn_func with qkv: (batch, seqlen, 3, nheads, headdim) (reference :972-1028; forward only)."""
+    return flash_attn_func(qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2], dropout_p, softmax_scale, causal, window_size,
+                           softcap, alibi_slopes, deterministic, return_attn_probs)
+
+
+def flash_attn_varlen_kvpacked_func(q, kv, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dropout_p=0.0,
+                                    softmax_scale=None, causal=False, window_size=(-1, -1), softcap=0.0,
+                                    alibi_slopes=None, deterministic=False, return_attn_probs=False):
+    """flash_attn_varlen_func with kv: (total_k, 2, nheads_k, headdim) (reference :1252-1341; forward only)."""
+    return flash_attn_varlen_func(q, kv[:, 0], kv[:, 1], cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dropout_p,
+                                  softmax_scale, causal, window_size, softcap, alibi_slopes, deterministic, return_attn_probs)
+
+
+def flash_attn_varlen_qkvpacked_func(qkv, cu_seqlens, max_seqlen, dropout_p=0.0, softmax_scale=None, causal=False,
+                                     window_size=(-1, -1), softcap=0.0, alibi_slopes=None, deterministic=False,
+                                     return_attn_probs=False):
+    """flash_attn_varlen_func with qkv: (total, 3, nheads, headdim) (reference :1186-1249; forward only)."""
+    return flash_attn_varlen_func(qkv[:, 0], qkv[:, 1], qkv[:, 2], cu_seqlens, cu_seqlens, max_seqlen, max_seqlen, dropout_p,
+                                  softmax_scale, causal, window_size, softcap, alibi_slopes, deterministic, return_attn_probs)
+
+
 def flash_attn_with_kvcache(
     q,
     k_cache,

@@ -149,3 +149,11 @@ def test_missing_library_is_an_error(monkeypatch):
     monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libfa_rocm.so")
     with pytest.raises(RuntimeError, match="no CPU or PyTorch fallback"):
         _lib.load()
+
+
+def test_package_exports_reference_names():
+    # reference flash_attn_npu/__init__.py:12-21
+    import flash_attn_npu
+    for name in ("flash_attn_func", "flash_attn_kvpacked_func", "flash_attn_qkvpacked_func", "flash_attn_varlen_func",
+                 "flash_attn_varlen_kvpacked_func", "flash_attn_varlen_qkvpacked_func", "flash_attn_with_kvcache"):
+        assert callable(getattr(flash_attn_npu, name)), name

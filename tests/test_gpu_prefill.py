@@ -139,3 +139,34 @@ def test_varlen_window_more_queries_than_keys(window):
     c = varlen_case([200, 40], [30, 90], 4, 2, 128, seed=12)
     got, ref, gold = run_varlen(c, causal=False, window_size=window)
     check_out(got[0], ref[0], got[1], ref[1], f"sq>sk window={window}")
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_dense_batch_functions(causal):
+    # flash_attn_func and the packed wrappers (reference flash_attn_npu_interface.py:972-1341) are the
+    # varlen kernel on equal-length sequences
+    from flash_attn_npu import (flash_attn_func, flash_attn_kvpacked_func, flash_attn_qkvpacked_func,
+                                flash_attn_varlen_kvpacked_func, flash_attn_varlen_qkvpacked_func)
+    B, sq, sk, hq, hk, d = 3, 200, 333, 8, 2, 128
+    c = varlen_case([sq] * B, [sk] * B, hq, hk, d, seed=40)
+    ref, ref_lse = O.flash_attn_varlen(c["q"], c["k"], c["v"], c["cu_q"], c["cu_k"], sq, sk, mode="fp32", causal=causal)
+    q4, k4, v4 = c["q"].view(B, sq, hq, d).cuda(), c["k"].view(B, sk, hk, d).cuda(), c["v"].view(B, sk, hk, d).cuda()
+    out, lse, _ = flash_attn_func(q4, k4, v4, causal=causal, return_attn_probs=True)
+    torch.cuda.synchronize()
+    assert out.shape == (B, sq, hq, d) and lse.shape == (B, hq, sq)
+    check_out(out.reshape(B * sq, hq, d), ref, lse.permute(1, 0, 2).reshape(hq, B * sq), ref_lse, "flash_attn_func")
+    kv = torch.stack([k4, v4], dim=2)
+    out2 = flash_attn_kvpacked_func(q4, kv, causal=causal)
+    assert torch.equal(out2, out)
+    out3 = flash_attn_varlen_kvpacked_func(q4.reshape(B * sq, hq, d), kv.reshape(B * sk, 2, hk, d), c["cu_q"].cuda(),
+                                           c["cu_k"].cuda(), sq, sk, causal=causal)
+    assert torch.equal(out3.reshape(B, sq, hq, d), out)
+    # qkv packed needs equal head counts and lengths
+    c2 = varlen_case([sq] * B, [sq] * B, 4, 4, d, seed=41)
+    ref2, _ = O.flash_attn_varlen(c2["q"], c2["k"], c2["v"], c2["cu_q"], c2["cu_k"], sq, sq, mode="fp32", causal=causal)
+    qkv = torch.stack([c2["q"], c2["k"], c2["v"]], dim=1).cuda()          # (total, 3, H, D)
+    o4 = flash_attn_varlen_qkvpacked_func(qkv, c2["cu_q"].cuda(), sq, causal=causal)
+    o5 = flash_attn_qkvpacked_func(qkv.view(B, sq, 3, 4, d), causal=causal)
+    torch.cuda.synchronize()
+    check_out(o4, ref2, None, None, "varlen_qkvpacked")
+    assert torch.equal(o5.reshape(B * sq, 4, d), o4)
