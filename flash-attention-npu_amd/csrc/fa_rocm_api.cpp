@@ -272,6 +272,8 @@ static int fwd_kvcache_impl(const fa_kvcache_args *a, void *stream_, void *const
 
     if (!is_mla_i8(a) && rows > fa::kDecodeMaxRows) {
         // query block too tall for the decode kernel: tiled forward over the paged cache
+        if (a->rotary_cos)   // before anything is written
+            return fail(FA_ERR_UNSUPPORTED, "rotary embedding needs seqlen_q * (nheads / nheads_k) <= %d", fa::kDecodeMaxRows);
         if (a->k_new) {
             rc = fa_rocm_append_kv(a, stream_);
             if (rc != FA_OK) return rc;
@@ -321,8 +323,6 @@ static int fwd_kvcache_impl(const fa_kvcache_args *a, void *stream_, void *const
         pp.window_left = a->window_left;
         pp.window_right = a->window_right;
         pp.window_norm_m = 0;
-        if (a->rotary_cos)
-            return fail(FA_ERR_UNSUPPORTED, "rotary embedding needs seqlen_q * (nheads / nheads_k) <= %d", fa::kDecodeMaxRows);
         const hipError_t e = fa::launch_prefill(pp, a->io_dtype, a->headdim_qk, stream);
         if (e != hipSuccess) return fail(FA_ERR_LAUNCH, "prefill launch failed: %s", hipGetErrorString(e));
         mark(2);
