@@ -163,7 +163,11 @@ int fa_rocm_plan_kvcache(const fa_kvcache_args *a, int num_cus, fa_split_plan *p
         // workgroup is the worker.
         const bool wave_workers = !is_mla_i8(a) && rows <= 16 && !std::getenv("FA_ROCM_DECODE_BLOCK_WORKERS");
         plan->num_workers = wave_workers ? plan->num_wgs * 4 : plan->num_wgs;
-        if (wave_workers) plan->min_share = 8;
+        if (wave_workers) plan->min_share = 2;   // short shares: the pipeline fill dominates tiny contexts otherwise
+        if (const char *env = std::getenv("FA_ROCM_MIN_SHARE")) {
+            const int v = std::atoi(env);
+            if (v > 0) plan->min_share = v;
+        }
         // every worker writes at most two partials (the units cut at the two ends of its share)
         plan->workspace_bytes = (size_t)plan->num_workers * 2 * slot_bytes;
         return FA_OK;

@@ -95,7 +95,7 @@ def test_split_plan_invariants():
     a = good_args()
     assert lib.fa_rocm_plan_kvcache(C.byref(a), 256, C.byref(plan)) == 0
     assert plan.mode == 1 and plan.num_wgs == 512                      # balanced: two workgroups per CU
-    assert plan.num_workers == 2048 and plan.min_share == 8            # one 16-row tile: every wave is a worker
+    assert plan.num_workers == 2048 and plan.min_share == 2            # one 16-row tile: every wave is a worker
     rows = 4
     assert plan.workspace_bytes == 2048 * 2 * rows * (128 + 1) * 4 == lib.fa_rocm_kvcache_workspace_bytes(C.byref(a), 256)
     a.seqlen_q = 5                                                      # 20 rows: two tiles, the workgroup is the worker
