@@ -255,7 +255,16 @@ __device__ __forceinline__ void wave_piece(const DecodeParams &p, const int b, c
 #pragma unroll
     for (int t = 0; t < Cfg::kColTiles; ++t) o_acc[t] = float4_t{0.f, 0.f, 0.f, 0.f};
 
+    // The two waves of a SIMD belong to different workgroups and stream independent shares; with
+    // equal priority the older one wins every arbitration and finishes ~10 % earlier, and the
+    // launch lasts as long as the slower.  Alternating the priority chunk by chunk, in opposite
+    // phase for the two wave slots, evens them out.
+    const int hw_slot = __builtin_amdgcn_s_getreg((1 << 11) | 4) & 1;   // HW_ID.WAVE_ID bit 0
     while (c < c_end) {
+        if ((c ^ hw_slot) & 1)
+            __builtin_amdgcn_s_setprio(1);
+        else
+            __builtin_amdgcn_s_setprio(0);
         // staged chunk: K -> swizzled LDS tile, V -> transposed operand registers
 #pragma unroll
         for (int j = 0; j < Cfg::kKLoads; ++j) {
