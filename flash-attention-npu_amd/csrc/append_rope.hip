@@ -115,6 +115,53 @@ hipError_t launch_append_quant_i8(const AppendParams &p, int dtype, hipStream_t 
     return hipGetLastError();
 }
 
+// q rotated at position cache_seqlens[b] + i (per-token) or cache_seqlens[b] (all tokens alike),
+// same arithmetic as the append (flash_attn_npu_interface.py:1469-1474).  grid: (Hq, Sq, B)
+template <typename T>
+__global__ void __launch_bounds__(64) rotate_q_kernel(const RotateQParams p) {
+    const int h = blockIdx.x;
+    const int i = blockIdx.y;
+    const int b = blockIdx.z;
+    const int pos = p.cache_seqlens[b] + (p.rotary_per_token ? i : 0);
+    const int rpos = min(max(pos, 0), p.seqlen_ro - 1);
+    const uint16_t *src = reinterpret_cast<const uint16_t *>(p.q) + (int64_t)b * p.q_stride_b + (int64_t)i * p.q_stride_s +
+                          (int64_t)h * p.q_stride_h;
+    uint16_t *dst = reinterpret_cast<uint16_t *>(p.out) + (((int64_t)b * p.seqlen_q + i) * p.nheads + h) * p.headdim;
+    const uint16_t *cosT = reinterpret_cast<const uint16_t *>(p.rotary_cos);
+    const uint16_t *sinT = reinterpret_cast<const uint16_t *>(p.rotary_sin);
+    const int rot = p.rotary_dim;
+    const int half = rot >> 1;
+    for (int c = threadIdx.x; c < p.headdim / 2; c += 64) {
+        int d1, d2;
+        if (c < half) {
+            d1 = p.rotary_interleaved ? 2 * c : c;
+            d2 = p.rotary_interleaved ? 2 * c + 1 : c + half;
+        } else {
+            d1 = rot + 2 * (c - half);
+            d2 = d1 + 1;
+        }
+        uint16_t o1 = src[d1], o2 = src[d2];
+        if (c < half) {
+            const float cs = to_float<T>(cosT[(int64_t)rpos * half + c]);
+            const float sn = to_float<T>(sinT[(int64_t)rpos * half + c]);
+            const float x1 = to_float<T>(o1), x2 = to_float<T>(o2);
+            o1 = from_float<T>(__fsub_rn(__fmul_rn(x1, cs), __fmul_rn(x2, sn)));
+            o2 = from_float<T>(__fadd_rn(__fmul_rn(x1, sn), __fmul_rn(x2, cs)));
+        }
+        dst[d1] = o1;
+        dst[d2] = o2;
+    }
+}
+
+hipError_t launch_rotate_q(const RotateQParams &p, int dtype, hipStream_t stream) {
+    dim3 grid(p.nheads, p.seqlen_q, p.batch);
+    if (dtype == 0)
+        hipLaunchKernelGGL(rotate_q_kernel<BF16>, grid, dim3(64), 0, stream, p);
+    else
+        hipLaunchKernelGGL(rotate_q_kernel<FP16>, grid, dim3(64), 0, stream, p);
+    return hipGetLastError();
+}
+
 hipError_t launch_append_kv(const AppendParams &p, int dtype, hipStream_t stream) {
     dim3 grid(p.nheads_k, p.seqlen_new, p.batch);
     if (dtype == 0)

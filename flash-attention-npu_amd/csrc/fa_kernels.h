@@ -69,6 +69,19 @@ struct AppendParams {
     int64_t bt_stride_b;
 };
 
+// Rotation of the query block of a kvcache call into a contiguous (B, Sq, Hq, D) copy, for the
+// query blocks that go to the tiled forward (the decode kernels rotate q while they stage it).
+struct RotateQParams {
+    const void *q;
+    void *out;
+    const void *rotary_cos;
+    const void *rotary_sin;
+    const int32_t *cache_seqlens;
+    int32_t batch, seqlen_q, nheads, headdim;
+    int32_t rotary_dim, seqlen_ro, rotary_interleaved, rotary_per_token;
+    int64_t q_stride_b, q_stride_s, q_stride_h;
+};
+
 // Parameters of the tiled (MFMA) forward used for varlen prefill and for kvcache calls whose
 // query block does not fit the decode kernel.
 struct PrefillParams {
@@ -99,6 +112,7 @@ struct PrefillParams {
 // dtype: 0 = bf16, 1 = fp16 (enum fa_dtype).  All return hipError_t of the launch.
 hipError_t launch_append_kv(const AppendParams &p, int dtype, hipStream_t stream);
 hipError_t launch_append_quant_i8(const AppendParams &p, int dtype, hipStream_t stream);
+hipError_t launch_rotate_q(const RotateQParams &p, int dtype, hipStream_t stream);
 hipError_t launch_decode_paged(const DecodeParams &p, int dtype, int headdim, hipStream_t stream);
 hipError_t launch_decode_wave(const DecodeParams &p, int dtype, int headdim, hipStream_t stream);
 hipError_t launch_splitkv_combine(const DecodeParams &p, int dtype, int headdim_v, hipStream_t stream);

@@ -147,6 +147,15 @@ int fa_rocm_plan_kvcache(const fa_kvcache_args *a, int num_cus, fa_split_plan *p
     // the int8 latent kernel works on units of 64 query heads and always uses the balanced partition
     const size_t rows = is_mla_i8(a) ? 64 : (size_t)a->seqlen_q * group;
     const size_t slot_bytes = rows * ((size_t)a->headdim_v + 1) * sizeof(float);
+    if (!is_mla_i8(a) && rows > (size_t)fa::kDecodeMaxRows) {
+        // query block too tall for the decode kernels: one pass of the tiled forward, nothing is
+        // split; with rotary embedding the workspace holds the rotated copy of q
+        plan->mode = FA_SPLIT_GRID;
+        plan->nsplits = 1;
+        plan->workspace_bytes =
+            a->rotary_cos ? (size_t)a->batch * a->seqlen_q * a->nheads * a->headdim_qk * sizeof(uint16_t) : 0;
+        return FA_OK;
+    }
     if (a->num_splits == 0 || is_mla_i8(a)) {
         plan->mode = FA_SPLIT_BALANCED;
         plan->nsplits = 1;
@@ -276,8 +285,9 @@ static int fwd_kvcache_impl(const fa_kvcache_args *a, void *stream_, void *const
 
     if (!is_mla_i8(a) && rows > fa::kDecodeMaxRows) {
         // query block too tall for the decode kernel: tiled forward over the paged cache
-        if (a->rotary_cos)   // before anything is written
-            return fail(FA_ERR_UNSUPPORTED, "rotary embedding needs seqlen_q * (nheads / nheads_k) <= %d", fa::kDecodeMaxRows);
+        const size_t q_bytes = (size_t)a->batch * a->seqlen_q * a->nheads * a->headdim_qk * sizeof(uint16_t);
+        if (a->rotary_cos && (!a->workspace || a->workspace_bytes < q_bytes))   // before anything is written
+            return fail(FA_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", q_bytes, a->workspace ? a->workspace_bytes : (size_t)0);
         if (a->k_new) {
             rc = fa_rocm_append_kv(a, stream_);
             if (rc != FA_OK) return rc;
@@ -327,6 +337,32 @@ static int fwd_kvcache_impl(const fa_kvcache_args *a, void *stream_, void *const
         pp.window_left = a->window_left;
         pp.window_right = a->window_right;
         pp.window_norm_m = 0;
+        if (a->rotary_cos) {
+            fa::RotateQParams rq;
+            std::memset(&rq, 0, sizeof(rq));
+            rq.q = a->q;
+            rq.out = a->workspace;
+            rq.rotary_cos = a->rotary_cos;
+            rq.rotary_sin = a->rotary_sin;
+            rq.cache_seqlens = a->cache_seqlens;
+            rq.batch = a->batch;
+            rq.seqlen_q = a->seqlen_q;
+            rq.nheads = a->nheads;
+            rq.headdim = a->headdim_qk;
+            rq.rotary_dim = a->rotary_dim;
+            rq.seqlen_ro = a->seqlen_ro;
+            rq.rotary_interleaved = a->rotary_interleaved;
+            rq.rotary_per_token = (a->causal || local) ? 1 : 0;
+            rq.q_stride_b = a->q_stride_b;
+            rq.q_stride_s = a->q_stride_s;
+            rq.q_stride_h = a->q_stride_h;
+            const hipError_t er = fa::launch_rotate_q(rq, a->io_dtype, stream);
+            if (er != hipSuccess) return fail(FA_ERR_LAUNCH, "rotate_q launch failed: %s", hipGetErrorString(er));
+            pp.q = a->workspace;
+            pp.q_stride_h = a->headdim_qk;
+            pp.q_stride_t = (int64_t)a->nheads * a->headdim_qk;
+            pp.q_stride_b = (int64_t)a->seqlen_q * pp.q_stride_t;
+        }
         const hipError_t e = fa::launch_prefill(pp, a->io_dtype, a->headdim_qk, stream);
         if (e != hipSuccess) return fail(FA_ERR_LAUNCH, "prefill launch failed: %s", hipGetErrorString(e));
         mark(2);

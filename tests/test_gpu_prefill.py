@@ -170,3 +170,25 @@ def test_dense_batch_functions(causal):
     torch.cuda.synchronize()
     check_out(o4, ref2, None, None, "varlen_qkvpacked")
     assert torch.equal(o5.reshape(B * sq, 4, d), o4)
+
+
+@pytest.mark.parametrize("interleaved,causal", [(False, True), (True, True), (False, False)])
+def test_tall_query_block_with_append_and_rotary(interleaved, causal):
+    # chunked prefill through the kvcache call: 40 new tokens x group 4 = 160 query rows go to the
+    # tiled kernel; K is rotated by the append, q by a pre-pass into the workspace
+    from flash_attn_npu import flash_attn_with_kvcache
+    from helpers import rotary_tables
+    case = make_paged_case(2, 8, 2, 128, 128, [300, 77], seqlen_q=40, seqlen_new=40, seed=50)
+    cos, sin = rotary_tables(512, 64)
+    dev = to_dev(case)
+    out, lse = flash_attn_with_kvcache(dev["q"], dev["k_cache"], dev["v_cache"], dev["k"], dev["v"], rotary_cos=cos.cuda(),
+                                       rotary_sin=sin.cuda(), cache_seqlens=dev["cache_seqlens"], block_table=dev["block_table"],
+                                       causal=causal, rotary_interleaved=interleaved, return_softmax_lse=True)
+    torch.cuda.synchronize()
+    kc, vc = case["k_cache"].clone(), case["v_cache"].clone()
+    ref, ref_lse = O.flash_attn_with_kvcache(case["q"], kc, vc, case["k"], case["v"], rotary_cos=cos, rotary_sin=sin,
+                                             cache_seqlens=case["cache_seqlens"], block_table=case["block_table"], causal=causal,
+                                             rotary_interleaved=interleaved, mode="fp32")
+    assert torch.equal(dev["k_cache"].cpu().view(torch.int16), kc.view(torch.int16))
+    assert torch.equal(dev["v_cache"].cpu().view(torch.int16), vc.view(torch.int16))
+    check_out(out, ref, lse, ref_lse, "tall rotary")
