@@ -84,6 +84,22 @@ __device__ __forceinline__ bool batch_chunk_prefix(const DecodeParams &p, int *s
     return any_empty;
 }
 
+// Query token and query head of row `row` of unit `kvh` of a batch row.  Ordinary caches: the unit
+// is a kv head, its rows are (query token, head of the group).  Latent int8 cache
+// (p.units_per_token > 0): the unit is (query token, 64-head group) and its rows are heads.
+struct RowId { int qi, head; };
+__device__ __forceinline__ RowId row_id(const DecodeParams &p, int kvh, int row) {
+    RowId r;
+    if (p.units_per_token > 0) {
+        r.qi = kvh / p.units_per_token;
+        r.head = (kvh - r.qi * p.units_per_token) * p.group + row;
+    } else {
+        r.qi = row / p.group;
+        r.head = kvh * p.group + (row - r.qi * p.group);
+    }
+    return r;
+}
+
 struct UnitPos {
     int b;          // batch row
     int pref;       // chunks of rows before b (one kv head's worth)
@@ -149,8 +165,8 @@ __device__ __forceinline__ void combine_row_wave(const DecodeParams &p, int b, i
         for (int c = 0; c < CPL; ++c) acc[c] += w * src[c];
     }
     const float inv = (tot > 0.f) ? 1.f / tot : 0.f;
-    const int qi = row / p.group;
-    const int head = kvh * p.group + (row - qi * p.group);
+    const RowId rid = row_id(p, kvh, row);
+    const int qi = rid.qi, head = rid.head;
     uint16_t *dst = reinterpret_cast<uint16_t *>(p.out) + (int64_t)b * p.o_stride_b + (int64_t)qi * p.o_stride_s +
                     (int64_t)head * p.o_stride_h + lane * CPL;
     if constexpr (CPL == 1) {
@@ -168,8 +184,8 @@ template <int DV> __device__ __forceinline__ void init_empty_unit(const DecodePa
     for (int idx = threadIdx.x; idx < p.rows * (DV / 8); idx += blockDim.x) {
         const int row = idx / (DV / 8);
         const int piece = idx - row * (DV / 8);
-        const int qi = row / p.group;
-        const int head = kvh * p.group + (row - qi * p.group);
+        const RowId rid = row_id(p, kvh, row);
+        const int qi = rid.qi, head = rid.head;
         uint16_t *dst = reinterpret_cast<uint16_t *>(p.out) + (int64_t)b * p.o_stride_b + (int64_t)qi * p.o_stride_s +
                         (int64_t)head * p.o_stride_h + piece * 8;
         store16(dst, u32x4_t{0, 0, 0, 0});

@@ -1,7 +1,7 @@
 // Latent-attention (MLA) decode over an int8 paged cache with per-token fp32 scales, gfx950.
 //
 // Layout: one latent kv head, 576 key dims, V = the first 512 of them (v_cache aliases k_cache);
-// 128 q heads (any multiple of 64), seqlen_q = 1.  The reference has no quantised path
+// 128 q heads (any multiple of 64), any seqlen_q (each query token is its own set of units).  The reference has no quantised path
 // (dtypes are limited to fp16/bf16 at csrc/ascend910/flash_attn_npu/flash_api.cpp:386-388 and
 // descales are rejected at flash_attn_npu_3/flash_api.cpp:153-155); the attention arithmetic is
 // the same as the bf16 decode kernel's (mha_fwd_kvcache.cpp:632-969 in the reference) applied to
@@ -66,9 +66,16 @@ struct MlaShared {
 };
 
 template <typename T>
-__device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, const int half, const UnitRange &ur,
+__device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, const int unit, const UnitRange &ur,
                                           const int range_lo, const int range_hi, const bool write_final,
                                           const int64_t slot, MlaShared &sh) {
+    // unit = (query token qi, 64-head group `half`); the chunks walked are those of the whole query
+    // block, the keys this token may not see (causal / window bounds of its own row) are masked
+    const int qi = unit / p.units_per_token;
+    const int half = unit - qi * p.units_per_token;
+    const int row_off = ur.Lk - p.seqlen_q + qi;                       // key aligned with this query token
+    const int mask_lo = max(range_lo, ur.wl >= 0 ? row_off - ur.wl : 0);
+    const int mask_hi = min(range_hi, ur.wr >= 0 ? row_off + ur.wr + 1 : ur.Lk);
     constexpr int KSTEPS = kMlaDqk / 32;   // 18
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -88,11 +95,11 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
         // =========================== score waves ===========================================
         const int lane0 = tid & 63;
         const int head = half * kMlaHeadsPerUnit + w4 * 16 + (lane0 & 15);   // head of this lane column
-        // Q^T operand (seqlen_q == 1): lane (lq, ln) holds head `head`, elements t*32 + lq*8 .. +7
+        // Q^T operand: lane (lq, ln) holds head `head` of query token qi, elements t*32 + lq*8 .. +7
         u32x4_t qreg[KSTEPS];
         {
             const uint16_t *src = reinterpret_cast<const uint16_t *>(p.q) + (int64_t)b * p.q_stride_b +
-                                  (int64_t)head * p.q_stride_h + (lane0 >> 4) * 8;
+                                  (int64_t)qi * p.q_stride_s + (int64_t)head * p.q_stride_h + (lane0 >> 4) * 8;
 #pragma unroll
             for (int t = 0; t < KSTEPS; ++t) qreg[t] = load16(src + t * 32);
         }
@@ -226,7 +233,7 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
                     for (int i = 0; i < 4; ++i) {
                         const int key = key_base + tt * 16 + i;
                         float v = s[tt][i] * ksv[i] * p.scale_log2;
-                        v = (key >= range_lo && key < range_hi) ? v : -INFINITY;
+                        v = (key >= mask_lo && key < mask_hi) ? v : -INFINITY;
                         x[tt * 4 + i] = v;
                         vsc[tt * 4 + i] = vsv[i];
                         mloc = fmaxf(mloc, v);
@@ -276,7 +283,7 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
             sh.l[w4][ln] = l_run;
             const int row = w4 * 16 + ln;
             if (write_final)
-                p.lse[(int64_t)b * p.nheads + head] = (l_run > 0.f) ? (m_run + fast_log2(l_run)) * kLn2 : INFINITY;
+                p.lse[((int64_t)b * p.nheads + head) * p.seqlen_q + qi] = (l_run > 0.f) ? (m_run + fast_log2(l_run)) * kLn2 : INFINITY;
             else
                 p.lse_partial[slot * p.rows + row] = (l_run > 0.f) ? m_run + fast_log2(l_run) : -INFINITY;
         }
@@ -365,8 +372,8 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
             const float lg = sh.l[hg][ln];
             const float inv = (lg > 0.f) ? 1.f / lg : 0.f;
             if (write_final) {
-                uint16_t *dst = reinterpret_cast<uint16_t *>(p.out) + (int64_t)b * p.o_stride_b + (int64_t)hd * p.o_stride_h +
-                                w4 * 128;
+                uint16_t *dst = reinterpret_cast<uint16_t *>(p.out) + (int64_t)b * p.o_stride_b + (int64_t)qi * p.o_stride_s +
+                                (int64_t)hd * p.o_stride_h + w4 * 128;
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     u32x4_t o4;
@@ -393,14 +400,14 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
 
 template <typename T> __global__ void __launch_bounds__(kMlaThreads) decode_mla_i8_kernel(const DecodeParams p) {
     __shared__ MlaShared sh;
-    balanced_driver<kMlaDv>(p, [&](int b, int half, const UnitRange &ur, int range_lo, int range_hi, bool whole, int64_t slot) {
-        mla_piece<T>(p, b, half, ur, range_lo, range_hi, whole, slot, sh);
+    balanced_driver<kMlaDv>(p, [&](int b, int unit, const UnitRange &ur, int range_lo, int range_hi, bool whole, int64_t slot) {
+        mla_piece<T>(p, b, unit, ur, range_lo, range_hi, whole, slot, sh);
     });
 }
 
-// p.nheads_k counts 64-head halves here (units per batch row), p.group = p.rows = 64.
+// p.nheads_k counts units per batch row here (seqlen_q * 64-head groups), p.group = p.rows = 64.
 hipError_t launch_decode_mla_i8(const DecodeParams &p, int dtype, hipStream_t stream) {
-    if (p.seqlen_q != 1 || p.rows != kMlaHeadsPerUnit || p.group != kMlaHeadsPerUnit || !p.balanced)
+    if (p.units_per_token <= 0 || p.rows != kMlaHeadsPerUnit || p.group != kMlaHeadsPerUnit || !p.balanced)
         return hipErrorInvalidValue;
     dim3 grid(p.num_wgs), block(kMlaThreads);
     if (dtype == 0)

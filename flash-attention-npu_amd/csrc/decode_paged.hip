@@ -535,8 +535,8 @@ __device__ __forceinline__ void combine_row_block(const DecodeParams &p, int b, 
             acc[3] += o.w;
         }
         const float inv = (tot > 0.f) ? 1.f / tot : 0.f;
-        const int qi = row / p.group;
-        const int head = kvh * p.group + (row - qi * p.group);
+        const RowId rid = row_id(p, kvh, row);
+        const int qi = rid.qi, head = rid.head;
         uint16_t *out_row = reinterpret_cast<uint16_t *>(p.out) + (int64_t)b * p.o_stride_b + (int64_t)qi * p.o_stride_s +
                             (int64_t)head * p.o_stride_h;
         uint2 o2;

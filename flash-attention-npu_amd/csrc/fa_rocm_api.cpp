@@ -105,8 +105,7 @@ int fa_rocm_kvcache_validate(const fa_kvcache_args *a) {
                 return fail(FA_ERR_UNSUPPORTED, "int8 KV cache: v must be the view k[..., :512] of the new latent rows");
             if (a->rotary_cos) return fail(FA_ERR_UNSUPPORTED, "rotary embedding is not supported with an int8 KV cache");
         }
-        if (a->seqlen_q != 1 || a->nheads % 64 != 0)
-            return fail(FA_ERR_SHAPE, "int8 KV cache needs seqlen_q == 1 and a multiple of 64 query heads");
+        if (a->nheads % 64 != 0) return fail(FA_ERR_SHAPE, "int8 KV cache needs a multiple of 64 query heads");
         if (a->v_cache != a->k_cache || a->v_stride_block != a->k_stride_block || a->v_stride_row != a->k_stride_row)
             return fail(FA_ERR_UNSUPPORTED, "int8 KV cache: v_cache must be the view k_cache[..., :512] of the latent cache");
         if (a->softcap > 0.f) return fail(FA_ERR_UNSUPPORTED, "softcap is not supported with an int8 KV cache");
@@ -469,7 +468,8 @@ static int fwd_kvcache_impl(const fa_kvcache_args *a, void *stream_, void *const
 
     hipError_t e;
     if (is_mla_i8(a)) {
-        p.nheads_k = a->nheads / 64;   // units per batch row: 64-head halves
+        p.units_per_token = a->nheads / 64;               // 64-head groups
+        p.nheads_k = a->seqlen_q * p.units_per_token;     // units per batch row
         p.group = 64;
         p.rows = 64;
         e = fa::launch_decode_mla_i8(p, a->io_dtype, stream);

@@ -106,3 +106,47 @@ def test_mla_append_rejections():
     cos = torch.ones(64, 32, dtype=torch.bfloat16, device="cuda")
     with pytest.raises(RuntimeError, match="rotary embedding is not supported with an int8"):
         flash_attn_with_kvcache(case["q"].cuda(), kc, kc[..., :512], kn, kn[..., :512], rotary_cos=cos, rotary_sin=cos, **kw)
+
+
+@pytest.mark.parametrize("sq,causal,window", [(2, True, (-1, -1)), (3, True, (-1, -1)), (2, False, (-1, -1)), (4, True, (300, 0))])
+def test_mla_several_query_tokens(sq, causal, window):
+    # multi-token decode (speculative / multi-token prediction): every query token is its own set
+    # of units with its own causal / window bound
+    from flash_attn_npu import flash_attn_with_kvcache
+    lens = [700, 2, 1025, 64]
+    case = mla_case(4, 128, lens, seed=7)
+    g = torch.Generator().manual_seed(77)
+    q = torch.randn(4, sq, 128, 576, generator=g).to(torch.bfloat16)
+    kc = case["k_cache"].cuda()
+    print("mla multi", sq, causal, window, lens, flush=True)
+    out, lse = flash_attn_with_kvcache(q.cuda(), kc, kc[..., :512], cache_seqlens=case["cache_seqlens"].cuda(),
+                                       block_table=case["block_table"].cuda(), softmax_scale=192 ** -0.5, causal=causal,
+                                       window_size=window, return_softmax_lse=True, k_scale_cache=case["k_scale"].cuda())
+    torch.cuda.synchronize()
+    ref, ref_lse = O.flash_attn_with_kvcache(q, case["k_cache"], case["k_cache"][..., :512], cache_seqlens=case["cache_seqlens"],
+                                             block_table=case["block_table"], softmax_scale=192 ** -0.5, causal=causal,
+                                             window_size=window, k_scale_cache=case["k_scale"], mode="fp32")
+    assert out.shape == (4, sq, 128, 512) and lse.shape == (4, 128, sq)
+    check_out(out, ref, lse, ref_lse, f"mla sq={sq}")
+
+
+def test_mla_multi_token_with_append():
+    from flash_attn_npu import flash_attn_with_kvcache
+    sq = 2
+    lens = [300, 0, 511]
+    case = mla_case(3, 64, [l + sq for l in lens], seed=8)
+    case["cache_seqlens"] = torch.tensor(lens, dtype=torch.int32)
+    g = torch.Generator().manual_seed(88)
+    q = torch.randn(3, sq, 64, 576, generator=g).to(torch.bfloat16)
+    k_new = torch.randn(3, sq, 1, 576, generator=g).to(torch.bfloat16)
+    kc, ks, kn = case["k_cache"].cuda(), case["k_scale"].cuda(), k_new.cuda()
+    out, lse = flash_attn_with_kvcache(q.cuda(), kc, kc[..., :512], kn, kn[..., :512], cache_seqlens=case["cache_seqlens"].cuda(),
+                                       block_table=case["block_table"].cuda(), softmax_scale=192 ** -0.5, causal=True,
+                                       return_softmax_lse=True, k_scale_cache=ks)
+    torch.cuda.synchronize()
+    kc_o, ks_o = case["k_cache"].clone(), case["k_scale"].clone()
+    ref, ref_lse = O.flash_attn_with_kvcache(q, kc_o, kc_o[..., :512], k_new, k_new[..., :512], cache_seqlens=case["cache_seqlens"],
+                                             block_table=case["block_table"], softmax_scale=192 ** -0.5, causal=True,
+                                             k_scale_cache=ks_o, mode="fp32")
+    assert torch.equal(kc.cpu(), kc_o) and torch.equal(ks.cpu().view(torch.int32), ks_o.view(torch.int32))
+    check_out(out, ref, lse, ref_lse, "mla multi append")
