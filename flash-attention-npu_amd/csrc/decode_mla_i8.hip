@@ -65,7 +65,7 @@ struct MlaShared {
     float l[4][16];                                              // final sum per head
 };
 
-template <typename T>
+template <typename T, bool SOFTCAP>
 __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, const int unit, const UnitRange &ur,
                                           const int range_lo, const int range_hi, const bool write_final,
                                           const int64_t slot, MlaShared &sh) {
@@ -232,7 +232,13 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
                         const int key = key_base + tt * 16 + i;
-                        float v = s[tt][i] * ksv[i] * p.scale_log2;
+                        float v = s[tt][i] * ksv[i];
+                        if constexpr (SOFTCAP) {
+                            const float e2 = __expf(2.f * v * p.softcap_pre);
+                            v = p.softcap_post * (1.f - 2.f / (e2 + 1.f));
+                        } else {
+                            v *= p.scale_log2;
+                        }
                         v = (key >= mask_lo && key < mask_hi) ? v : -INFINITY;
                         x[tt * 4 + i] = v;
                         vsc[tt * 4 + i] = vsv[i];
@@ -398,10 +404,11 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
     __syncthreads();   // the LDS tiles and sums are reused by the next piece
 }
 
-template <typename T> __global__ void __launch_bounds__(kMlaThreads) decode_mla_i8_kernel(const DecodeParams p) {
+template <typename T, bool SOFTCAP>
+__global__ void __launch_bounds__(kMlaThreads) decode_mla_i8_kernel(const DecodeParams p) {
     __shared__ MlaShared sh;
     balanced_driver<kMlaDv>(p, [&](int b, int unit, const UnitRange &ur, int range_lo, int range_hi, bool whole, int64_t slot) {
-        mla_piece<T>(p, b, unit, ur, range_lo, range_hi, whole, slot, sh);
+        mla_piece<T, SOFTCAP>(p, b, unit, ur, range_lo, range_hi, whole, slot, sh);
     });
 }
 
@@ -410,10 +417,18 @@ hipError_t launch_decode_mla_i8(const DecodeParams &p, int dtype, hipStream_t st
     if (p.units_per_token <= 0 || p.rows != kMlaHeadsPerUnit || p.group != kMlaHeadsPerUnit || !p.balanced)
         return hipErrorInvalidValue;
     dim3 grid(p.num_wgs), block(kMlaThreads);
-    if (dtype == 0)
-        hipLaunchKernelGGL(decode_mla_i8_kernel<BF16>, grid, block, 0, stream, p);
-    else
-        hipLaunchKernelGGL(decode_mla_i8_kernel<FP16>, grid, block, 0, stream, p);
+    const bool softcap = p.softcap_post != 0.f;
+    if (dtype == 0) {
+        if (softcap)
+            hipLaunchKernelGGL((decode_mla_i8_kernel<BF16, true>), grid, block, 0, stream, p);
+        else
+            hipLaunchKernelGGL((decode_mla_i8_kernel<BF16, false>), grid, block, 0, stream, p);
+    } else {
+        if (softcap)
+            hipLaunchKernelGGL((decode_mla_i8_kernel<FP16, true>), grid, block, 0, stream, p);
+        else
+            hipLaunchKernelGGL((decode_mla_i8_kernel<FP16, false>), grid, block, 0, stream, p);
+    }
     return hipGetLastError();
 }
 

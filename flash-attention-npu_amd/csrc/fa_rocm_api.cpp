@@ -108,7 +108,6 @@ int fa_rocm_kvcache_validate(const fa_kvcache_args *a) {
         if (a->nheads % 64 != 0) return fail(FA_ERR_SHAPE, "int8 KV cache needs a multiple of 64 query heads");
         if (a->v_cache != a->k_cache || a->v_stride_block != a->k_stride_block || a->v_stride_row != a->k_stride_row)
             return fail(FA_ERR_UNSUPPORTED, "int8 KV cache: v_cache must be the view k_cache[..., :512] of the latent cache");
-        if (a->softcap > 0.f) return fail(FA_ERR_UNSUPPORTED, "softcap is not supported with an int8 KV cache");
         if (a->k_stride_row % 16 || a->k_stride_block % 16)
             return fail(FA_ERR_SHAPE, "int8 cache strides must be multiples of 16 bytes");
     } else {

@@ -150,3 +150,17 @@ def test_mla_multi_token_with_append():
                                              k_scale_cache=ks_o, mode="fp32")
     assert torch.equal(kc.cpu(), kc_o) and torch.equal(ks.cpu().view(torch.int32), ks_o.view(torch.int32))
     check_out(out, ref, lse, ref_lse, "mla multi append")
+
+
+def test_mla_softcap():
+    from flash_attn_npu import flash_attn_with_kvcache
+    case = mla_case(2, 128, [900, 130], seed=9)
+    kc = case["k_cache"].cuda()
+    out, lse = flash_attn_with_kvcache(case["q"].cuda(), kc, kc[..., :512], cache_seqlens=case["cache_seqlens"].cuda(),
+                                       block_table=case["block_table"].cuda(), softmax_scale=192 ** -0.5, causal=True, softcap=20.0,
+                                       return_softmax_lse=True, k_scale_cache=case["k_scale"].cuda())
+    torch.cuda.synchronize()
+    ref, ref_lse = O.flash_attn_with_kvcache(case["q"], case["k_cache"], case["k_cache"][..., :512], cache_seqlens=case["cache_seqlens"],
+                                             block_table=case["block_table"], softmax_scale=192 ** -0.5, causal=True, softcap=20.0,
+                                             k_scale_cache=case["k_scale"], mode="fp32")
+    check_out(out, ref, lse, ref_lse, "mla softcap")
