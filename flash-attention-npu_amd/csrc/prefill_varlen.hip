@@ -245,6 +245,34 @@ __global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) prefill_kernel(const 
 #pragma unroll
                 for (int r = 0; r < 16; ++r) mloc = fmaxf(mloc, s[tt][r]);
             mloc *= p.scale_log2;
+        } else if (!SOFTCAP && need_mask) {
+            // masked tile (the diagonal of a causal block, window edges, the ragged end): element r
+            // of half tt is key tile0 + 4*lh + e(tt, r) with e a compile-time constant, so the
+            // row's bounds are compared in tile coordinates; a side that cannot bite is skipped
+            const int lo_rel = klo_r - tile0 - 4 * lh;
+            const int hi_rel = khi_r - tile0 - 4 * lh;
+            const bool need_lo = __builtin_amdgcn_readfirstlane(tile0 < wave_klo_max);
+            if (!need_lo) {
+#pragma unroll
+                for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const int e = tt * 32 + 8 * (r >> 2) + (r & 3);
+                        const float v = (e <= hi_rel) ? s[tt][r] * p.scale_log2 : -INFINITY;
+                        s[tt][r] = v;
+                        mloc = fmaxf(mloc, v);
+                    }
+            } else {
+#pragma unroll
+                for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const int e = tt * 32 + 8 * (r >> 2) + (r & 3);
+                        const float v = (e >= lo_rel && e <= hi_rel) ? s[tt][r] * p.scale_log2 : -INFINITY;
+                        s[tt][r] = v;
+                        mloc = fmaxf(mloc, v);
+                    }
+            }
         } else {
 #pragma unroll
             for (int tt = 0; tt < 2; ++tt)
@@ -258,10 +286,8 @@ __global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) prefill_kernel(const 
                     } else {
                         v *= p.scale_log2;
                     }
-                    if (need_mask) {
-                        const int key = tile0 + tt * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
-                        v = (key >= klo_r && key <= khi_r) ? v : -INFINITY;
-                    }
+                    const int e = tt * 32 + 8 * (r >> 2) + (r & 3);
+                    v = (!need_mask || (e >= klo_r - tile0 - 4 * lh && e <= khi_r - tile0 - 4 * lh)) ? v : -INFINITY;
                     s[tt][r] = v;
                     mloc = fmaxf(mloc, v);
                 }
