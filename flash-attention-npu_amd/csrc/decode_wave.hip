@@ -183,7 +183,7 @@ __device__ __forceinline__ void wave_piece(const DecodeParams &p, const int b, c
     };
     auto load_v = [&](const uint8_t *s2, int e, int hh) {
         if constexpr (Cfg::kVW == 8) {
-            const u32x4_t t4 = load16(s2);
+            const u32x4_t t4 = load16_stream(s2);
             vreg[e][hh][0] = t4[0];
             vreg[e][hh][1] = t4[1];
             vreg[e][hh][2] = t4[2];
@@ -205,7 +205,7 @@ __device__ __forceinline__ void wave_piece(const DecodeParams &p, const int b, c
         if (last >= kChunk - 1) {
 #pragma unroll
             for (int j = 0; j < Cfg::kKLoads; ++j)
-                kreg[j] = load16(kb + (size_t)(j * Cfg::kRowsPerLoad) * k_row_bytes + k_lane_off);
+                kreg[j] = load16_stream(kb + (size_t)(j * Cfg::kRowsPerLoad) * k_row_bytes + k_lane_off);
 #pragma unroll
             for (int e = 0; e < 8; ++e)
 #pragma unroll

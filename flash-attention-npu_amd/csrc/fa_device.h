@@ -155,6 +155,10 @@ __device__ __forceinline__ int block_max_keys(const int32_t *seqlens, int batch,
 
 // 16-byte global load / store through plain vector types
 __device__ __forceinline__ u32x4_t load16(const void *p) { return *reinterpret_cast<const u32x4_t *>(p); }
+// the same load marked non-temporal: data that is read once (the KV stream) need not stay in the caches
+__device__ __forceinline__ u32x4_t load16_stream(const void *p) {
+    return __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(p));
+}
 __device__ __forceinline__ void store16(void *p, const u32x4_t &v) { *reinterpret_cast<u32x4_t *>(p) = v; }
 
 }  // namespace fa
