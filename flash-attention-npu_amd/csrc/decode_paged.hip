@@ -126,11 +126,12 @@ __device__ __forceinline__ void process_piece(const DecodeParams &p, const int b
             vreg[e][hh][2] = t4[2];
             vreg[e][hh][3] = t4[3];
         } else if constexpr (Cfg::kVW == 4) {
-            const uint2 t2 = *reinterpret_cast<const uint2 *>(s2);
-            vreg[e][hh][0] = t2.x;
-            vreg[e][hh][1] = t2.y;
+            typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+            const u32x2_t t2 = __builtin_nontemporal_load(reinterpret_cast<const u32x2_t *>(s2));
+            vreg[e][hh][0] = t2[0];
+            vreg[e][hh][1] = t2[1];
         } else {
-            vreg[e][hh][0] = *reinterpret_cast<const uint32_t *>(s2);
+            vreg[e][hh][0] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(s2));
         }
     };
 
