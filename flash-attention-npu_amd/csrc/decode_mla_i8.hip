@@ -314,14 +314,17 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
                 const int pb = set;                                  // (j - 2) & 1
                 // ---- O^T += V^T P^T on this wave's 128-column slice, all four head groups.
                 //      k slot 8*lq + e of the MFMA is key (e >> 2) * 16 + lq * 4 + (e & 3) of the chunk.
-                u32x4_t vr[8];
+                //      The V^T operands come from the transposing LDS read (ds_read_b64_tr_b16): in a
+                //      16-lane group, lane s points at 4 columns (4*(s%4)..) of key row s/4 and receives
+                //      column s of the group's 16 for its 4 key rows.  Column tile ct = columns ct*16..+15
+                //      of the slice; the 16-byte unit of a row is swizzled with row & 7 = 4*(lq&1) + ln/4.
+                typedef short v4s_t __attribute__((ext_vector_type(4)));
+                const int tr_row = lq * 4 + (ln >> 2);
+                const int tr_k = 4 * (lq & 1) + (ln >> 2);
+                const uint8_t *tr_base = &sh.k[tile][tr_row * kMlaRowBytes + w4 * 256 + 8 * (ln & 1)];
+                int tr_off[4];   // unit (2*(ct&3) + (ln&3)/2) ^ tr_k inside its aligned group of eight
 #pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const int row = (e >> 2) * 16 + lq * 4 + (e & 3);
-                    // unit w4*16 + ln of the row, swizzled with row & 7 = 4 * (lq & 1) + (e & 3)
-                    vr[e] = *reinterpret_cast<const u32x4_t *>(
-                        &sh.k[tile][row * kMlaRowBytes + (((w4 * 16 + ln) ^ (4 * (lq & 1) + (e & 3))) << 4)]);
-                }
+                for (int c4 = 0; c4 < 4; ++c4) tr_off[c4] = ((2 * c4 + ((ln & 3) >> 1)) ^ tr_k) << 4;
                 u32x4_t pkg[4];
                 const uint32_t bumps = *reinterpret_cast<const uint32_t *>(sh.bump[pb]);
 #pragma unroll
@@ -339,18 +342,18 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
                     }
                 }
 #pragma unroll
-                for (int w2 = 0; w2 < 4; ++w2) {
-                    u32x4_t a_lo, a_hi;
+                for (int ct = 0; ct < 8; ++ct) {
+                    u32x4_t va;
 #pragma unroll
-                    for (int u = 0; u < 4; ++u) {
-                        a_lo[u] = __builtin_amdgcn_perm(vr[2 * u + 1][w2], vr[2 * u][w2], 0x05040100u);
-                        a_hi[u] = __builtin_amdgcn_perm(vr[2 * u + 1][w2], vr[2 * u][w2], 0x07060302u);
+                    for (int hv = 0; hv < 2; ++hv) {
+                        const v4s_t r4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                            (__attribute__((address_space(3))) v4s_t *)(tr_base + hv * 16 * kMlaRowBytes + (ct >> 2) * 128 + tr_off[ct & 3]));
+                        const uint2 r2 = __builtin_bit_cast(uint2, r4);
+                        va[2 * hv] = r2.x;
+                        va[2 * hv + 1] = r2.y;
                     }
 #pragma unroll
-                    for (int hg = 0; hg < 4; ++hg) {
-                        o_acc[hg][2 * w2] = mfma16<T>(a_lo, pkg[hg], o_acc[hg][2 * w2]);
-                        o_acc[hg][2 * w2 + 1] = mfma16<T>(a_hi, pkg[hg], o_acc[hg][2 * w2 + 1]);
-                    }
+                    for (int hg = 0; hg < 4; ++hg) o_acc[hg][ct] = mfma16<T>(va, pkg[hg], o_acc[hg][ct]);
                 }
             }
             __syncthreads();
@@ -366,7 +369,7 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
         }
 
         // ---- write the column slice: register i of tile t of group hg is column
-        //      w4*128 + (lq*4 + i)*8 + t of head hg*16 + ln
+        //      w4*128 + t*16 + lq*4 + i of head hg*16 + ln
         __syncthreads();   // sums of all heads are in LDS
         const int lane = tid & 63;
         const int lq = lane >> 4;
@@ -381,23 +384,18 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
                 uint16_t *dst = reinterpret_cast<uint16_t *>(p.out) + (int64_t)b * p.o_stride_b + (int64_t)qi * p.o_stride_s +
                                 (int64_t)hd * p.o_stride_h + w4 * 128;
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    u32x4_t o4;
-#pragma unroll
-                    for (int u = 0; u < 4; ++u) o4[u] = pack2<T>(o_acc[hg][2 * u][i] * inv, o_acc[hg][2 * u + 1][i] * inv);
-                    store16(dst + (lq * 4 + i) * 8, o4);
+                for (int t = 0; t < 8; ++t) {
+                    const uint2 o2 = make_uint2(pack2<T>(o_acc[hg][t][0] * inv, o_acc[hg][t][1] * inv),
+                                                pack2<T>(o_acc[hg][t][2] * inv, o_acc[hg][t][3] * inv));
+                    *reinterpret_cast<uint2 *>(dst + t * 16 + lq * 4) = o2;
                 }
             } else {
                 const int64_t srow = slot * p.rows + row;
                 float *dst = p.o_partial + srow * kMlaDv + w4 * 128;
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    float *d2 = dst + (lq * 4 + i) * 8;
-                    *reinterpret_cast<float4 *>(d2) = make_float4(o_acc[hg][0][i] * inv, o_acc[hg][1][i] * inv,
-                                                                  o_acc[hg][2][i] * inv, o_acc[hg][3][i] * inv);
-                    *reinterpret_cast<float4 *>(d2 + 4) = make_float4(o_acc[hg][4][i] * inv, o_acc[hg][5][i] * inv,
-                                                                      o_acc[hg][6][i] * inv, o_acc[hg][7][i] * inv);
-                }
+                for (int t = 0; t < 8; ++t)
+                    *reinterpret_cast<float4 *>(dst + t * 16 + lq * 4) =
+                        make_float4(o_acc[hg][t][0] * inv, o_acc[hg][t][1] * inv, o_acc[hg][t][2] * inv, o_acc[hg][t][3] * inv);
             }
         }
     }
