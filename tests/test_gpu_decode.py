@@ -138,3 +138,15 @@ def test_decode_window_more_queries_than_keys(window):
     case = make_paged_case(2, 4, 2, 128, 256, [2, 1], seqlen_q=5, seed=13)
     got, ref, gold, _ = run_both(case, causal=False, window_size=window)
     check_out(got[0], ref[0], got[1], ref[1], f"sq>sk window={window}")
+
+
+@pytest.mark.parametrize("B,num_splits", [(300, 0), (700, 0), (300, 2)])
+def test_decode_batch_larger_than_prefix_segments(B, num_splits):
+    # the balanced partition scans the batch in 256 segments: more than 256 rows puts several rows
+    # into one segment (rows with no key, short and long rows mixed)
+    import random
+    r = random.Random(B)
+    lens = [r.choice([0, 1, 5, 33, 64, 100, 257, 600]) for _ in range(B)]
+    case = make_paged_case(B, 8, 2, 128, 64, lens, seed=B)
+    got, ref, gold, _ = run_both(case, causal=True, num_splits=num_splits)
+    check_out(got[0], ref[0], got[1], ref[1], f"B={B}")

@@ -164,3 +164,12 @@ def test_mla_softcap():
                                              block_table=case["block_table"], softmax_scale=192 ** -0.5, causal=True, softcap=20.0,
                                              k_scale_cache=case["k_scale"], mode="fp32")
     check_out(out, ref, lse, ref_lse, "mla softcap")
+
+
+def test_mla_batch_larger_than_prefix_segments():
+    import random
+    r = random.Random(9)
+    lens = [r.choice([0, 1, 40, 300]) for _ in range(270)]
+    case = mla_case(270, 64, lens, page=64, seed=10)
+    got, ref, gold = run(case)
+    check_out(got[0], ref[0], got[1], ref[1], "mla B=270")
