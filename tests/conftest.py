@@ -1,11 +1,12 @@
-"""pytest setup: puts the oracle and the package on sys.path, registers the `gpu` marker."""
+"""pytest setup: puts the oracle, the package and the repository root (bench.py's workload builders)
+on sys.path, registers the `gpu` marker."""
 import os
 import sys
 
 import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-for p in (os.path.join(ROOT, "flash-attention-npu_amd"), os.path.join(ROOT, "oracle"), os.path.join(ROOT, "tests")):
+for p in (ROOT, os.path.join(ROOT, "flash-attention-npu_amd"), os.path.join(ROOT, "oracle"), os.path.join(ROOT, "tests")):
     if p not in sys.path:
         sys.path.insert(0, p)
 

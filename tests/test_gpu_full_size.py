@@ -1,0 +1,204 @@
+"""The benchmark workloads at their full sizes (bench.py builds them: 64 rows of 1-8K keys, 4 rows of
+131072 keys, the int8 latent batch, the 32768-token packed prefill), checked through properties that
+do not need the oracle on the whole input: batch rows picked from the launch against the oracle on
+their own pages, appended rows bit-exact and every other cache byte untouched, the same result under
+a relabelling of the physical pages (bit-identical) and under another split of the keys, a long
+context against the log-sum-exp merge of its two halves, a window against the sliced cache, packed
+sequences against the same sequence run alone (bit-identical)."""
+import pytest
+import torch
+
+import fa_oracle as O
+from helpers import check_out
+
+pytestmark = pytest.mark.gpu
+
+# two launches that cut the keys differently round the 16-bit output differently: one bf16 ulp of a
+# value below 2 (2^-7), LSE in fp32
+SPLIT_OUT_ABS = 8e-3
+SPLIT_LSE_REL = 2e-5
+
+
+def run_call(w, num_splits=0, **over):
+    from bench import bind_decode
+    ww = dict(w)
+    ww.update(over)
+    call = bind_decode(ww, num_splits=num_splits)
+    call.run()
+    torch.cuda.synchronize()
+    return call.out, call.lse
+
+
+def close_splits(a, b, what):
+    (oa, la), (ob, lb) = a, b
+    d = (oa.float() - ob.float()).abs().max().item()
+    assert d <= SPLIT_OUT_ABS, f"{what}: outputs differ by {d:.3e}"
+    fin = ~torch.isinf(la)
+    assert torch.equal(torch.isinf(la), torch.isinf(lb))
+    rel = ((la[fin] - lb[fin]).abs() / la[fin].abs().clamp_min(1.0)).max().item()
+    assert rel <= SPLIT_LSE_REL, f"{what}: LSE differs by {rel:.3e}"
+
+
+def row_case(w, b, k_cache, v_cache, k_scale=None):
+    """Batch row b on its own pages, on the host: the inputs of a one-row oracle call."""
+    lens, page, snew = w["lens"], w["page"], w["snew"]
+    n = -(-(int(lens[b]) + snew) // page)
+    blocks = w["block_table"][b, :n].long()
+    c = dict(q=w["q"][b:b + 1].cpu(), k_cache=k_cache[blocks].cpu(), v_cache=v_cache[blocks].cpu(),
+             cache_seqlens=torch.tensor([int(lens[b])], dtype=torch.int32),
+             block_table=torch.arange(n, dtype=torch.int32).view(1, n),
+             k=None if w["k"] is None else w["k"][b:b + 1].cpu(), v=None if w["v"] is None else w["v"][b:b + 1].cpu(),
+             rotary_cos=None if w["rotary_cos"] is None else w["rotary_cos"].cpu(),
+             rotary_sin=None if w["rotary_sin"] is None else w["rotary_sin"].cpu())
+    if k_scale is not None:
+        c["k_scale_cache"] = k_scale[blocks].cpu()
+    return c
+
+
+def oracle_row(w, c):
+    kw = {}
+    if "k_scale_cache" in c:
+        kw["k_scale_cache"] = c["k_scale_cache"]
+    return O.flash_attn_with_kvcache(c["q"], c["k_cache"], c["v_cache"], c["k"], c["v"], rotary_cos=c["rotary_cos"],
+                                     rotary_sin=c["rotary_sin"], cache_seqlens=c["cache_seqlens"],
+                                     block_table=c["block_table"], softmax_scale=w["scale"], causal=w["causal"],
+                                     window_size=w["window"], rotary_interleaved=False, mode="fp32", **kw)
+
+
+def sample_rows(lens):
+    g = torch.Generator().manual_seed(5)
+    rows = {int(lens.argmin()), int(lens.argmax())}
+    rows.update(int(x) for x in torch.randperm(len(lens), generator=g)[:2])
+    return sorted(rows)
+
+
+def test_c2_headline_decode_full_size():
+    from bench import decode_workload
+    w = decode_workload("c2", "cuda")
+    B, page = w["B"], w["page"]
+    lens = w["lens"]
+    k_before, v_before = w["k_cache"].clone(), w["v_cache"].clone()
+    print("full size c2: balanced call", flush=True)
+    out, lse = run_call(w)
+
+    # appended rows: bit-exact against the oracle's rotation, every other row of the pool untouched
+    pos = lens.long()
+    blk = w["block_table"].cpu()[torch.arange(B), pos // page].long()
+    row = pos % page
+    one = dict(k=[], v=[])
+    for b in range(B):
+        c = row_case(w, b, k_before, v_before)
+        O.append_kv(c["k_cache"], c["v_cache"], c["k"], c["v"], c["cache_seqlens"], c["block_table"], c["rotary_cos"],
+                    c["rotary_sin"], False)
+        one["k"].append(c["k_cache"][int(pos[b]) // page, int(row[b])])
+        one["v"].append(c["v_cache"][int(pos[b]) // page, int(row[b])])
+    got_k = w["k_cache"][blk.cuda(), row.cuda()].cpu()
+    got_v = w["v_cache"][blk.cuda(), row.cuda()].cpu()
+    assert torch.equal(got_k.view(torch.int16), torch.stack(one["k"]).view(torch.int16)), "appended K rows"
+    assert torch.equal(got_v.view(torch.int16), torch.stack(one["v"]).view(torch.int16)), "appended V rows"
+    appended = torch.zeros(w["k_cache"].shape[0] * page, dtype=torch.bool, device="cuda")
+    appended[(blk * page + row).cuda()] = True
+    for name, now, before in (("K", w["k_cache"], k_before), ("V", w["v_cache"], v_before)):
+        changed = (now.view(torch.int16) != before.view(torch.int16)).flatten(2).any(-1).flatten()
+        assert not (changed & ~appended).any(), f"{name} cache bytes outside the appended rows changed"
+
+    # rows of the launch against the oracle on their own pages (the oracle appends and rotates itself)
+    for b in sample_rows(lens):
+        print("full size c2: oracle row", b, int(lens[b]), flush=True)
+        ref, ref_lse = oracle_row(w, row_case(w, b, k_before, v_before))
+        check_out(out[b:b + 1], ref, lse[b:b + 1], ref_lse, f"c2 row {b}")
+
+    # another cut of the keys (no split at all; the append rewrites the same bytes)
+    print("full size c2: unsplit call", flush=True)
+    close_splits((out, lse), run_call(w, num_splits=1), "c2 balanced vs unsplit")
+    close_splits((out, lse), run_call(w, num_splits=4), "c2 balanced vs 4 splits")
+
+    # the same cache under other physical page numbers: bit-identical results
+    print("full size c2: relabelled pages", flush=True)
+    pool = w["k_cache"].shape[0]
+    relabel = torch.randperm(pool, generator=torch.Generator().manual_seed(9)).cuda()   # old page -> new page
+    k2, v2 = torch.empty_like(k_before), torch.empty_like(v_before)
+    k2[relabel], v2[relabel] = k_before, v_before
+    out2, lse2 = run_call(w, k_cache=k2, v_cache=v2, block_table=relabel[w["block_table"].long()].to(torch.int32))
+    assert torch.equal(out2, out) and torch.equal(lse2, lse), "page relabelling changed the result"
+
+
+def test_c3_long_context_full_size():
+    from bench import decode_workload
+    w = decode_workload("c3a", "cuda")
+    page, L = w["page"], 131072
+    print("full size c3a: whole context", flush=True)
+    out, lse = run_call(w)
+    # a row against the oracle
+    ref, ref_lse = oracle_row(w, row_case(w, 2, w["k_cache"], w["v_cache"]))
+    check_out(out[2:3], ref, lse[2:3], ref_lse, "c3a row 2")
+    # the two halves of the context, merged on the host by their log-sum-exps.  Causal with one query
+    # row hides nothing, so each half is an ordinary call on half of the table.
+    half = torch.full_like(w["cache_seqlens"], L // 2)
+    cols = L // 2 // page
+    print("full size c3a: halves", flush=True)
+    o1, l1 = run_call(w, cache_seqlens=half, lens=half.cpu())
+    o2, l2 = run_call(w, cache_seqlens=half, lens=half.cpu(), block_table=w["block_table"][:, cols:].contiguous())
+    l12 = torch.logaddexp(l1, l2)
+    w1, w2 = torch.exp(l1 - l12).permute(0, 2, 1)[..., None], torch.exp(l2 - l12).permute(0, 2, 1)[..., None]
+    merged = w1 * o1.float() + w2 * o2.float()
+    close_splits((out, lse), (merged, l12), "c3a whole vs merged halves")
+
+    # window (4095, 0) with one query row is plain attention over the last 4096 keys
+    wb = decode_workload("c3b", "cuda")
+    print("full size c3b: window", flush=True)
+    out_b, lse_b = run_call(wb)
+    last = torch.full_like(wb["cache_seqlens"], 4096)
+    tail = wb["block_table"][:, (L - 4096) // page:].contiguous()
+    sliced = run_call(wb, cache_seqlens=last, lens=last.cpu(), block_table=tail, window=(-1, -1))
+    close_splits((out_b, lse_b), sliced, "c3b window vs sliced cache")
+    ws = dict(wb, lens=last.cpu(), block_table=tail, window=(-1, -1))
+    for b in range(wb["B"]):
+        ref, ref_lse = oracle_row(ws, row_case(ws, b, wb["k_cache"], wb["v_cache"]))
+        check_out(out_b[b:b + 1], ref, lse_b[b:b + 1], ref_lse, f"c3b row {b}")
+
+
+def test_c4_latent_decode_full_size():
+    from bench import mla_workload
+    w = mla_workload("cuda")
+    codes, scales = w["k_cache"].clone(), w["k_scale"].clone()
+    print("full size c4", flush=True)
+    out, lse = run_call(w)
+    assert torch.equal(w["k_cache"], codes) and torch.equal(w["k_scale"], scales), "the call changed the cache"
+    for b in sample_rows(w["lens"])[:3]:
+        print("full size c4: oracle row", b, int(w["lens"][b]), flush=True)
+        c = row_case(w, b, w["k_cache"], w["v_cache"], w["k_scale"])
+        c["v_cache"] = c["k_cache"][..., :512]
+        ref, ref_lse = oracle_row(w, c)
+        check_out(out[b:b + 1], ref, lse[b:b + 1], ref_lse, f"c4 row {b}")
+    pool = codes.shape[0]
+    relabel = torch.randperm(pool, generator=torch.Generator().manual_seed(10)).cuda()
+    k2, s2 = torch.empty_like(codes), torch.empty_like(scales)
+    k2[relabel], s2[relabel] = codes, scales
+    out2, lse2 = run_call(w, k_cache=k2, v_cache=k2[..., :512], k_scale=s2,
+                          block_table=relabel[w["block_table"].long()].to(torch.int32))
+    assert torch.equal(out2, out) and torch.equal(lse2, lse), "page relabelling changed the result"
+
+
+def test_c5_packed_prefill_full_size():
+    from bench import prefill_workload
+    from flash_attn_npu import flash_attn_varlen_func
+    w = prefill_workload("cuda")
+    cu, lens = w["cu"], w["lens"]
+    print("full size c5", lens.tolist(), flush=True)
+    out, lse, _ = flash_attn_varlen_func(w["q"], w["k"], w["v"], cu, cu, w["max_len"], w["max_len"], causal=True,
+                                         return_attn_probs=True)
+    torch.cuda.synchronize()
+    order = torch.argsort(lens)
+    for b in (int(order[0]), int(order[len(order) // 2]), int(order[-1])):
+        a, e = int(cu[b]), int(cu[b + 1])
+        one_cu = torch.tensor([0, e - a], dtype=torch.int32, device="cuda")
+        one, one_lse, _ = flash_attn_varlen_func(w["q"][a:e], w["k"][a:e], w["v"][a:e], one_cu, one_cu, e - a, e - a,
+                                                 causal=True, return_attn_probs=True)
+        assert torch.equal(one, out[a:e]) and torch.equal(one_lse, lse[:, a:e]), f"sequence {b} depends on its batch"
+        if e - a <= 2600:
+            print("full size c5: oracle sequence", b, e - a, flush=True)
+            hcu = torch.tensor([0, e - a], dtype=torch.int32)
+            ref, ref_lse = O.flash_attn_varlen(w["q"][a:e].cpu(), w["k"][a:e].cpu(), w["v"][a:e].cpu(), hcu, hcu, e - a,
+                                               e - a, causal=True, mode="fp32")
+            check_out(out[a:e], ref, lse[:, a:e], ref_lse, f"c5 sequence {b}")
