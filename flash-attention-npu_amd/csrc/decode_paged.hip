@@ -478,9 +478,13 @@ __global__ void __launch_bounds__(64) splitkv_combine_kernel(const DecodeParams 
     const int kvh = blockIdx.y;
     const int b = blockIdx.z;
     const UnitRange ur = unit_range(p, b, window_norm_m(p));
+    int split_keys = p.split_keys;
+    if (p.split_adaptive)
+        split_keys = adaptive_split_keys(min(block_max_keys(p.cache_seqlens, p.batch, p.seqlen_new), p.max_blocks * p.page_size),
+                                         p.nsplits);
     const int lo_al = ur.c0 * kChunk;
-    const int ns = (ur.nchunks == 0) ? 1 : min(p.nsplits, (ur.hi - lo_al + p.split_keys - 1) / p.split_keys);
-    if (ns == 1) return;  // the decode kernel already wrote this unit
+    const int ns = (ur.nchunks == 0) ? 1 : min(p.nsplits, (ur.hi - lo_al + split_keys - 1) / split_keys);
+    if (ns == 1) return;  // the kernel that computed this unit already wrote it
     combine_row_wave<T, D>(p, b, kvh, row, ns,
                            [&](int s) -> int64_t { return ((int64_t)b * p.nheads_k + kvh) * p.nsplits + s; });
 }

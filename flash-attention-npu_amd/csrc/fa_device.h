@@ -153,6 +153,14 @@ __device__ __forceinline__ int block_max_keys(const int32_t *seqlens, int batch,
     return m;
 }
 
+// Keys per split when a launch cuts every unit into at most `nsplits` ranges and the cut is sized on
+// the device from the longest sequence of the batch (a multiple of 256 keys).  The kernel that
+// writes the partial results and the one that merges them must agree on it.
+__device__ __forceinline__ int adaptive_split_keys(int max_keys, int nsplits) {
+    const int per = (max(max_keys, 1) + nsplits - 1) / nsplits;
+    return (per + 255) / 256 * 256;
+}
+
 // 16-byte global load / store through plain vector types
 __device__ __forceinline__ u32x4_t load16(const void *p) { return *reinterpret_cast<const u32x4_t *>(p); }
 // the same load marked non-temporal: data that is read once (the KV stream) need not stay in the caches

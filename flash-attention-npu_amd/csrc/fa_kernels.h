@@ -45,6 +45,7 @@ struct DecodeParams {
     int32_t num_workers, min_share;  // workers sharing the chunk list (workgroups, or waves), least chunks per share
     int32_t wave_workers;          // 1: every wave is a worker (num_workers = 4 * num_wgs)
     int32_t head_interleave;       // 1: worker w streams share w / Hk of the per-head list for kv head w % Hk
+    int32_t split_adaptive;        // grid mode: keys per split = adaptive_split_keys(longest sequence, nsplits), not split_keys
     int32_t units_per_token;       // latent int8 cache: 64-head groups per query token (nheads_k = seqlen_q * this); else 0
 };
 
@@ -96,6 +97,7 @@ struct PrefillParams {
     const int32_t *seqused_k;      // paged: keys per row (cache_seqlens)
     const int32_t *block_table;    // NULL: dense K/V
     int32_t batch, nheads, nheads_k, group;
+    int32_t pack;                  // set by the launcher: 1, or group when tile rows are (query, head) pairs
     int32_t seqlen_q_fixed, seqlen_k_add;   // kvcache layout: Sq per row, keys appended this call
     int32_t max_seqlen_q, total_q;
     int32_t page_size, max_blocks, num_blocks;
@@ -108,7 +110,19 @@ struct PrefillParams {
     float scale_log2, softcap_pre, softcap_post;
     int32_t causal, window_left, window_right;
     int32_t window_norm_m;                  // key count the window is normalised with; 0 = each row's own
+    // split of the keys (kvcache layout only): blockIdx.z = batch row * nsplits + split, ranges of
+    // adaptive_split_keys() keys; a unit cut into several ranges leaves fp32 partials and base-2 LSEs
+    // in slot (batch row * nheads_k + kv head) * nsplits + split for the split-KV combine kernel
+    int32_t nsplits, rows;                  // rows = seqlen_q_fixed * group
+    float *o_partial;
+    float *lse_partial;
 };
+
+// GQA group packed into the tile rows of the tiled forward for query blocks of max_seqlen_q rows
+// (1 = one q head per tile).
+int prefill_pack(int group, int max_seqlen_q);
+// Tiles (workgroups) of the tiled forward per batch row.
+int prefill_tiles(int nheads, int nheads_k, int max_seqlen_q);
 
 // dtype: 0 = bf16, 1 = fp16 (enum fa_dtype).  All return hipError_t of the launch.
 hipError_t launch_append_kv(const AppendParams &p, int dtype, hipStream_t stream);

@@ -48,6 +48,14 @@ int device_cus() {
 bool is_mla_i8(const fa_kvcache_args *a) { return a->kv_dtype == FA_INT8; }
 
 // Upper bound of the live key range any row can have, from shapes alone.
+// bytes of the rotated copy of q that a tall query block with rotary embedding keeps at the start of
+// the workspace (a multiple of 256 so that the partials behind it stay aligned)
+size_t tall_q_bytes(const fa_kvcache_args *a) {
+    if (!a->rotary_cos) return 0;
+    const size_t n = (size_t)a->batch * a->seqlen_q * a->nheads * a->headdim_qk * sizeof(uint16_t);
+    return (n + 255) / 256 * 256;
+}
+
 int64_t live_keys_bound(const fa_kvcache_args *a) {
     int64_t cap = (int64_t)a->max_blocks_per_seq * a->page_size;
     const int wr = a->causal ? 0 : a->window_right;
@@ -146,12 +154,28 @@ int fa_rocm_plan_kvcache(const fa_kvcache_args *a, int num_cus, fa_split_plan *p
     const size_t rows = is_mla_i8(a) ? 64 : (size_t)a->seqlen_q * group;
     const size_t slot_bytes = rows * ((size_t)a->headdim_v + 1) * sizeof(float);
     if (!is_mla_i8(a) && rows > (size_t)fa::kDecodeMaxRows) {
-        // query block too tall for the decode kernels: one pass of the tiled forward, nothing is
-        // split; with rotary embedding the workspace holds the rotated copy of q
+        // Query block too tall for the decode kernels: the tiled forward.  When its tiles alone
+        // cannot fill the device (few sequences, short blocks) the keys of every unit are cut into
+        // ranges as well; the range length is sized on the device from the longest sequence, so only
+        // the number of ranges is planned here.  With rotary embedding the workspace starts with the
+        // rotated copy of q.
         plan->mode = FA_SPLIT_GRID;
-        plan->nsplits = 1;
-        plan->workspace_bytes =
-            a->rotary_cos ? (size_t)a->batch * a->seqlen_q * a->nheads * a->headdim_qk * sizeof(uint16_t) : 0;
+        const int64_t bound = live_keys_bound(a);
+        int64_t n = 1;
+        if (a->num_splits > 1) {
+            n = a->num_splits;
+        } else if (a->num_splits == 0) {
+            const int64_t tiles = (int64_t)a->batch * fa::prefill_tiles(a->nheads, a->nheads_k, a->seqlen_q);
+            const int64_t slots = (int64_t)num_cus * (a->headdim_qk <= 128 ? 2 : 1);
+            if (tiles * 2 <= slots) n = (slots + tiles - 1) / tiles;
+        }
+        const int64_t most = (bound + 1023) / 1024;   // at least 1024 keys per range
+        if (n > most) n = most;
+        if (n > 64) n = 64;
+        if (n < 1) n = 1;
+        plan->nsplits = (int32_t)n;
+        plan->split_keys = 0;
+        plan->workspace_bytes = tall_q_bytes(a) + (n > 1 ? (size_t)a->batch * a->nheads_k * n * slot_bytes : 0);
         return FA_OK;
     }
     if (a->num_splits == 0 || is_mla_i8(a)) {
@@ -283,9 +307,14 @@ static int fwd_kvcache_impl(const fa_kvcache_args *a, void *stream_, void *const
 
     if (!is_mla_i8(a) && rows > fa::kDecodeMaxRows) {
         // query block too tall for the decode kernel: tiled forward over the paged cache
-        const size_t q_bytes = (size_t)a->batch * a->seqlen_q * a->nheads * a->headdim_qk * sizeof(uint16_t);
-        if (a->rotary_cos && (!a->workspace || a->workspace_bytes < q_bytes))   // before anything is written
-            return fail(FA_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", q_bytes, a->workspace ? a->workspace_bytes : (size_t)0);
+        int cus_t = device_cus();
+        if (cus_t <= 0) cus_t = 256;
+        fa_split_plan tplan;
+        rc = fa_rocm_plan_kvcache(a, cus_t, &tplan);
+        if (rc != FA_OK) return rc;
+        if (tplan.workspace_bytes > 0 && (!a->workspace || a->workspace_bytes < tplan.workspace_bytes))   // before anything is written
+            return fail(FA_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", tplan.workspace_bytes,
+                        a->workspace ? a->workspace_bytes : (size_t)0);
         if (a->k_new) {
             rc = fa_rocm_append_kv(a, stream_);
             if (rc != FA_OK) return rc;
@@ -361,9 +390,47 @@ static int fwd_kvcache_impl(const fa_kvcache_args *a, void *stream_, void *const
             pp.q_stride_t = (int64_t)a->nheads * a->headdim_qk;
             pp.q_stride_b = (int64_t)a->seqlen_q * pp.q_stride_t;
         }
+        float *partials = reinterpret_cast<float *>(static_cast<char *>(a->workspace) + tall_q_bytes(a));
+        const size_t slot_rows = (size_t)a->batch * a->nheads_k * tplan.nsplits * rows;
+        if (tplan.nsplits > 1) {
+            pp.nsplits = tplan.nsplits;
+            pp.rows = rows;
+            pp.o_partial = partials;
+            pp.lse_partial = partials + slot_rows * a->headdim_v;
+        }
         const hipError_t e = fa::launch_prefill(pp, a->io_dtype, a->headdim_qk, stream);
         if (e != hipSuccess) return fail(FA_ERR_LAUNCH, "prefill launch failed: %s", hipGetErrorString(e));
         mark(2);
+        if (tplan.nsplits > 1) {
+            // the decode kernels' grid-mode combine merges the ranges: same slots, same row order
+            fa::DecodeParams cp;
+            std::memset(&cp, 0, sizeof(cp));
+            cp.out = a->out;
+            cp.lse = a->softmax_lse;
+            cp.cache_seqlens = a->cache_seqlens;
+            cp.batch = a->batch;
+            cp.seqlen_q = a->seqlen_q;
+            cp.nheads = a->nheads;
+            cp.nheads_k = a->nheads_k;
+            cp.group = group;
+            cp.rows = rows;
+            cp.seqlen_new = a->seqlen_new;
+            cp.page_size = a->page_size;
+            cp.max_blocks = a->max_blocks_per_seq;
+            cp.o_stride_b = a->o_stride_b;
+            cp.o_stride_s = a->o_stride_s;
+            cp.o_stride_h = a->o_stride_h;
+            cp.causal = a->causal;
+            cp.window_left = a->window_left;
+            cp.window_right = a->window_right;
+            cp.nsplits = tplan.nsplits;
+            cp.split_keys = 256;
+            cp.split_adaptive = 1;
+            cp.o_partial = pp.o_partial;
+            cp.lse_partial = pp.lse_partial;
+            const hipError_t ec = fa::launch_splitkv_combine(cp, a->io_dtype, a->headdim_v, stream);
+            if (ec != hipSuccess) return fail(FA_ERR_LAUNCH, "combine launch failed: %s", hipGetErrorString(ec));
+        }
         mark(3);
         return FA_OK;
     }

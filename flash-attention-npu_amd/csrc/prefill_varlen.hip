@@ -6,7 +6,10 @@
 // flash_api.cpp:848-1089).  Where the reference ping-pongs S, P and O_tmp between its matrix and
 // vector cores through global memory, everything between the K/V tile loads and the final store
 // stays in registers here:
-//   * one workgroup = 128 query rows of one (sequence, q head); 4 waves x 32 rows;
+//   * one workgroup = 128 query rows of one (sequence, q head); 4 waves x 32 rows.  Short query
+//     blocks under GQA are packed instead (p.pack = group): the 128 rows are (query, head of the
+//     group) pairs of one kv head, query-major, so a 16-token block of an 8-head group fills a tile
+//     and K/V are read once per kv head (the reference packs heads the same way, flash_api.cpp:33-95);
 //   * K/V tiles of 64 keys are fetched once per workgroup with 16-byte coalesced loads and
 //     double-buffered in LDS (K rows XOR-swizzled so MFMA operand reads are conflict free);
 //   * S^T = K Q^T and O^T = V^T P^T on the 32x32x16 MFMA: a query row is one lane column in both
@@ -48,9 +51,12 @@ __global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) prefill_kernel(const 
     const int ln = lane & 31;   // MFMA row / column
 
     const int mb = gridDim.x - 1 - blockIdx.x;  // tall causal blocks first
-    const int h = blockIdx.y;
-    const int b = blockIdx.z;
-    const int hk = h / p.group;
+    const int b = (p.nsplits > 1) ? blockIdx.z / p.nsplits : blockIdx.z;
+    const int split = blockIdx.z - b * max(p.nsplits, 1);
+    // tile row R of the block is query R / pg of head h_base + R % pg (pg = 1: one q head per block)
+    const int pg = p.pack;
+    const int hk = (pg > 1) ? blockIdx.y : blockIdx.y / p.group;
+    const int h_base = (pg > 1) ? blockIdx.y * p.group : blockIdx.y;
 
     int q0, Sq, k0 = 0, Sk;
     if (p.cu_seqlens_q) {
@@ -77,30 +83,71 @@ __global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) prefill_kernel(const 
     }
     if (norm_m <= 0) norm_m = max(Sk, 1);
     normalize_window(wl, wr_eff, p.causal, norm_m);
-    if (mb * kBM >= Sq) return;
+    int batch_max = 0;
+    if constexpr (PAGED) {
+        if (p.nsplits > 1) batch_max = min(block_max_keys(p.seqused_k, p.batch, p.seqlen_k_add), p.max_blocks * p.page_size);
+    }
+    const int n_rows = Sq * pg;
+    const int R0 = mb * kBM;
+    if (R0 >= n_rows) return;
     const int off = Sk - Sq;
 
-    const uint16_t *qb = reinterpret_cast<const uint16_t *>(p.q) + (int64_t)b * p.q_stride_b + (int64_t)h * p.q_stride_h;
-    uint16_t *ob = reinterpret_cast<uint16_t *>(p.out) + (int64_t)b * p.o_stride_b + (int64_t)h * p.o_stride_h;
-    float *lse_b = p.lse + (int64_t)b * p.lse_stride_b + (int64_t)h * p.lse_stride_h;
+    // split of the unit's visible keys: the same cut as the decode kernels' grid mode, so that the
+    // same combine kernel merges the partials
+    int range_lo = 0, range_hi = Sk;
+    bool whole = true;
+    int64_t slot = 0;
+    if (p.nsplits > 1) {
+        int u_lo = 0, u_hi = Sk;
+        if (wr_eff >= 0) u_hi = min(Sk, Sq - 1 + off + wr_eff + 1);
+        if (wl >= 0) u_lo = max(0, off - wl);
+        const bool empty = Sk <= 0 || u_hi <= u_lo;
+        const int lo_al = u_lo / 32 * 32;
+        const int sk = adaptive_split_keys(batch_max, p.nsplits);
+        const int ns_row = empty ? 1 : min(p.nsplits, (u_hi - lo_al + sk - 1) / sk);
+        if (split >= ns_row) return;
+        if (!empty) {
+            range_lo = max(u_lo, lo_al + split * sk);
+            range_hi = (split == ns_row - 1) ? u_hi : min(u_hi, lo_al + (split + 1) * sk);
+        }
+        whole = ns_row == 1;
+        slot = ((int64_t)b * p.nheads_k + hk) * p.nsplits + split;
+    }
 
-    // key range the whole 128-row block can see
-    const int r_lo = mb * kBM;
-    const int r_hi = min(Sq, r_lo + kBM) - 1;
+    const int my_R = min(R0 + wave * 32 + ln, n_rows - 1);   // rows past the end repeat the last one and are dropped
+    const bool row_ok = R0 + wave * 32 + ln < n_rows;
+    const int my_row = my_R / pg;                            // query position of this lane column
+    const int my_head = h_base + (my_R - my_row * pg);
+    const uint16_t *q_row = reinterpret_cast<const uint16_t *>(p.q) + (int64_t)b * p.q_stride_b +
+                            (int64_t)my_head * p.q_stride_h + (int64_t)(q0 + my_row) * p.q_stride_t;
+    uint16_t *o_row = reinterpret_cast<uint16_t *>(p.out) + (int64_t)b * p.o_stride_b + (int64_t)my_head * p.o_stride_h +
+                      (int64_t)(q0 + my_row) * p.o_stride_t;
+    float *lse_row = p.lse + (int64_t)b * p.lse_stride_b + (int64_t)my_head * p.lse_stride_h + q0 + my_row;
+
+    // key range the whole block (query positions r_lo .. r_hi) can see
+    const int r_lo = R0 / pg;
+    const int r_hi = (min(n_rows, R0 + kBM) - 1) / pg;
     int k_lo = 0, k_hi = Sk;
     if (wl >= 0) k_lo = max(0, r_lo + off - wl);
     if (wr_eff >= 0) k_hi = min(Sk, r_hi + off + wr_eff + 1);
-    k_hi = max(k_hi, 0);
-
-    const int my_row = r_lo + wave * 32 + ln;   // query row of this lane column
-    const bool row_ok = my_row < Sq;
+    k_lo = max(k_lo, range_lo);
+    k_hi = max(min(k_hi, range_hi), 0);
+    // where this lane's row goes when the unit is cut: row (query, head of the group) of the slot
+    float *part_row = nullptr, *part_lse = nullptr;
+    if (!whole) {
+        const int64_t prow = slot * p.rows + (int64_t)my_row * p.group + (my_head - hk * p.group);
+        part_row = p.o_partial + prow * D;
+        part_lse = p.lse_partial + prow;
+    }
 
     if (k_hi <= k_lo) {
         // nothing visible for the whole block: out = 0, lse = +inf
-        if (row_ok) {
-            uint16_t *dst = ob + (int64_t)(q0 + my_row) * p.o_stride_t;
-            for (int c = lh * (D / 2); c < (lh + 1) * (D / 2); c += 8) store16(dst + c, u32x4_t{0, 0, 0, 0});
-            if (lh == 0) lse_b[q0 + my_row] = INFINITY;
+        if (row_ok && whole) {
+            for (int c = lh * (D / 2); c < (lh + 1) * (D / 2); c += 8) store16(o_row + c, u32x4_t{0, 0, 0, 0});
+            if (lh == 0) *lse_row = INFINITY;
+        } else if (row_ok) {
+            for (int c = lh * (D / 2); c < (lh + 1) * (D / 2); c += 4) *reinterpret_cast<float4 *>(part_row + c) = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (lh == 0) *part_lse = -INFINITY;
         }
         return;
     }
@@ -109,16 +156,18 @@ __global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) prefill_kernel(const 
     int klo_r = 0, khi_r = Sk - 1;
     if (wl >= 0) klo_r = max(0, my_row + off - wl);
     if (wr_eff >= 0) khi_r = min(Sk - 1, my_row + off + wr_eff);
+    klo_r = max(klo_r, range_lo);
+    khi_r = min(khi_r, range_hi - 1);
     // bounds that decide, per wave, whether a tile needs element masks
-    const int rw0 = r_lo + wave * 32;
-    const int rw1 = min(Sq - 1, rw0 + 31);
-    const int wave_klo_max = (wl >= 0) ? max(0, rw1 + off - wl) : 0;
-    const int wave_khi_min = (wr_eff >= 0) ? min(Sk - 1, rw0 + off + wr_eff) : Sk - 1;
+    const int rw0 = min(R0 + wave * 32, n_rows - 1) / pg;        // first and last query position of the wave
+    const int rw1 = (min(n_rows, R0 + wave * 32 + 32) - 1) / pg;
+    const int wave_klo_max = max(range_lo, (wl >= 0) ? max(0, rw1 + off - wl) : 0);
+    const int wave_khi_min = min(range_hi - 1, (wr_eff >= 0) ? min(Sk - 1, rw0 + off + wr_eff) : Sk - 1);
 
     // Q^T operand: lane (lh, ln) holds row ln, elements t*16 + lh*8 .. +7
     u32x4_t qreg[Cfg::kKSteps];
     {
-        const uint16_t *src = qb + (int64_t)(q0 + min(my_row, Sq - 1)) * p.q_stride_t + lh * 8;
+        const uint16_t *src = q_row + lh * 8;
 #pragma unroll
         for (int t = 0; t < Cfg::kKSteps; ++t) {
             qreg[t] = load16(src + t * 16);
@@ -369,8 +418,22 @@ __global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) prefill_kernel(const 
     //      t*32 + 8*(r/4) + 4*lh + r%4 of query row ln: four consecutive columns per (t, r/4).
     l_run = halves_sum(l_run);
     const float inv = (l_run > 0.f) ? 1.f / l_run : 0.f;
+    if (!whole) {
+        // one of several ranges of the unit: normalised fp32 partial and base-2 LSE for the combine
+        if (row_ok) {
+#pragma unroll
+            for (int t = 0; t < Cfg::kMT; ++t)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    *reinterpret_cast<float4 *>(part_row + t * 32 + 8 * j + 4 * lh) =
+                        make_float4(o_acc[t][4 * j] * inv, o_acc[t][4 * j + 1] * inv, o_acc[t][4 * j + 2] * inv,
+                                    o_acc[t][4 * j + 3] * inv);
+            if (lh == 0) *part_lse = (l_run > 0.f) ? m_run + fast_log2(l_run) : -INFINITY;
+        }
+        return;
+    }
     if (row_ok) {
-        uint16_t *dst = ob + (int64_t)(q0 + my_row) * p.o_stride_t;
+        uint16_t *dst = o_row;
 #pragma unroll
         for (int t = 0; t < Cfg::kMT; ++t)
 #pragma unroll
@@ -380,13 +443,28 @@ __global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) prefill_kernel(const 
                 o2.y = pack2<T>(o_acc[t][4 * j + 2] * inv, o_acc[t][4 * j + 3] * inv);
                 *reinterpret_cast<uint2 *>(dst + t * 32 + 8 * j + 4 * lh) = o2;
             }
-        if (lh == 0) lse_b[q0 + my_row] = (l_run > 0.f) ? (m_run + fast_log2(l_run)) * kLn2 : INFINITY;
+        if (lh == 0) *lse_row = (l_run > 0.f) ? (m_run + fast_log2(l_run)) * kLn2 : INFINITY;
     }
 }
 
-template <typename T, int D> static hipError_t launch_prefill_d(const PrefillParams &p, hipStream_t stream) {
-    const int num_mb = (p.max_seqlen_q + kBM - 1) / kBM;
-    dim3 grid(num_mb, p.nheads, p.batch);
+// pack the heads of a GQA group into the tile rows when that saves at least a quarter of the tiles
+int prefill_pack(int group, int max_seqlen_q) {
+    const int tiles_plain = group * ((max_seqlen_q + kBM - 1) / kBM);
+    const int tiles_packed = (max_seqlen_q * group + kBM - 1) / kBM;
+    return (group > 1 && tiles_packed * 4 <= tiles_plain * 3) ? group : 1;
+}
+
+int prefill_tiles(int nheads, int nheads_k, int max_seqlen_q) {
+    const int pack = prefill_pack(nheads / nheads_k, max_seqlen_q);
+    return (pack > 1 ? nheads_k : nheads) * ((max_seqlen_q * pack + kBM - 1) / kBM);
+}
+
+template <typename T, int D> static hipError_t launch_prefill_d(const PrefillParams &p_in, hipStream_t stream) {
+    PrefillParams p = p_in;
+    p.pack = prefill_pack(p.group, p.max_seqlen_q);
+    const int num_mb = (p.max_seqlen_q * p.pack + kBM - 1) / kBM;
+    if (p.nsplits > 1 && (!p.block_table || p.cu_seqlens_q || !p.o_partial)) return hipErrorInvalidValue;
+    dim3 grid(num_mb, p.pack > 1 ? p.nheads_k : p.nheads, p.batch * max(p.nsplits, 1));
     dim3 block(256);
     const bool softcap = p.softcap_post != 0.f;
     const bool paged = p.block_table != nullptr;

@@ -192,3 +192,72 @@ def test_tall_query_block_with_append_and_rotary(interleaved, causal):
     assert torch.equal(dev["k_cache"].cpu().view(torch.int16), kc.view(torch.int16))
     assert torch.equal(dev["v_cache"].cpu().view(torch.int16), vc.view(torch.int16))
     check_out(out, ref, lse, ref_lse, "tall rotary")
+
+
+@pytest.mark.parametrize("sq,hq,hk,d", [(16, 64, 8, 128), (20, 12, 2, 128), (9, 24, 3, 64), (40, 10, 2, 256), (100, 6, 2, 128)])
+@pytest.mark.parametrize("causal,window", [(True, (-1, -1)), (False, (-1, -1)), (False, (30, 3)), (True, (100, 0))])
+def test_kvcache_short_blocks_packed_heads(sq, hq, hk, d, causal, window):
+    # seqlen_q * group > 64 with fewer than 128 query rows per head: the tile rows are (query, head)
+    # pairs of one kv head; groups that do not divide 128 (6, 8 of 3, 5) put a query's heads in two tiles
+    from flash_attn_npu import flash_attn_with_kvcache
+    case = make_paged_case(3, hq, hk, d, 64, [700, 64, sq], seqlen_q=sq, seed=31, dtype=torch.float16)
+    dev = to_dev(case)
+    print("packed heads", sq, hq, hk, d, causal, window, flush=True)
+    out, lse = flash_attn_with_kvcache(dev["q"], dev["k_cache"], dev["v_cache"], cache_seqlens=dev["cache_seqlens"],
+                                       block_table=dev["block_table"], causal=causal, window_size=window,
+                                       return_softmax_lse=True)
+    torch.cuda.synchronize()
+    ref, ref_lse = O.flash_attn_with_kvcache(case["q"], case["k_cache"], case["v_cache"], cache_seqlens=case["cache_seqlens"],
+                                             block_table=case["block_table"], causal=causal, window_size=window, mode="fp32")
+    check_out(out, ref, lse, ref_lse, f"packed sq={sq} g={hq // hk}")
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_varlen_short_sequences_packed_heads(causal):
+    # packed sequences all shorter than a tile, GQA group 5: ragged (query, head) rows, some
+    # sequences with more queries than keys, one of a single token
+    c = varlen_case([5, 40, 17, 1, 90], [300, 40, 9, 64, 1000], 10, 2, 128, seed=32)
+    got, ref, gold = run_varlen(c, causal=causal)
+    check_out(got[0], ref[0], got[1], ref[1], "varlen packed heads")
+    check_vs_golden(got[0], gold[0], got[1], gold[1], "varlen packed heads")
+
+
+@pytest.mark.parametrize("num_splits", [0, 2, 5])
+@pytest.mark.parametrize("sq,hq,hk,d", [(16, 64, 8, 128), (128, 8, 2, 128), (300, 4, 4, 64), (70, 6, 2, 256)])
+@pytest.mark.parametrize("causal,window", [(True, (-1, -1)), (False, (-1, -1)), (True, (700, 0))])
+def test_kvcache_tall_blocks_split_keys(sq, hq, hk, d, causal, window, num_splits):
+    # few sequences with tall query blocks over long contexts: the tiled kernel cuts every unit's
+    # keys into ranges (num_splits 0: as many as fill the device, 2 / 5: at most that many) and the
+    # combine kernel merges them; rows of very different lengths, one shorter than the query block
+    from flash_attn_npu import flash_attn_with_kvcache
+    lens = [5000, 40] if sq <= 128 else [3000, 301]
+    case = make_paged_case(2, hq, hk, d, 128, lens, seqlen_q=sq, seed=41)
+    dev = to_dev(case)
+    print("tall split", sq, hq, hk, d, causal, window, num_splits, flush=True)
+    out, lse = flash_attn_with_kvcache(dev["q"], dev["k_cache"], dev["v_cache"], cache_seqlens=dev["cache_seqlens"],
+                                       block_table=dev["block_table"], causal=causal, window_size=window,
+                                       num_splits=num_splits, return_softmax_lse=True)
+    torch.cuda.synchronize()
+    ref, ref_lse = O.flash_attn_with_kvcache(case["q"], case["k_cache"], case["v_cache"], cache_seqlens=case["cache_seqlens"],
+                                             block_table=case["block_table"], causal=causal, window_size=window, mode="fp32")
+    check_out(out, ref, lse, ref_lse, f"tall split sq={sq} n={num_splits}")
+
+
+def test_kvcache_tall_split_with_append_and_rotary():
+    # the workspace holds the rotated q in front of the partials
+    from flash_attn_npu import flash_attn_with_kvcache
+    from helpers import rotary_tables
+    case = make_paged_case(1, 16, 2, 128, 256, [6000], seqlen_q=24, seqlen_new=24, seed=42)
+    cos, sin = rotary_tables(8192, 128)
+    dev = to_dev(case)
+    out, lse = flash_attn_with_kvcache(dev["q"], dev["k_cache"], dev["v_cache"], dev["k"], dev["v"], rotary_cos=cos.cuda(),
+                                       rotary_sin=sin.cuda(), cache_seqlens=dev["cache_seqlens"],
+                                       block_table=dev["block_table"], causal=True, rotary_interleaved=False,
+                                       return_softmax_lse=True)
+    torch.cuda.synchronize()
+    kc, vc = case["k_cache"].clone(), case["v_cache"].clone()
+    ref, ref_lse = O.flash_attn_with_kvcache(case["q"], kc, vc, case["k"], case["v"], rotary_cos=cos, rotary_sin=sin,
+                                             cache_seqlens=case["cache_seqlens"], block_table=case["block_table"],
+                                             causal=True, rotary_interleaved=False, mode="fp32")
+    assert torch.equal(dev["k_cache"].cpu().view(torch.int16), kc.view(torch.int16))
+    check_out(out, ref, lse, ref_lse, "tall split append rotary")
