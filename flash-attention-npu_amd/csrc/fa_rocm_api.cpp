@@ -149,7 +149,10 @@ int fa_rocm_plan_kvcache(const fa_kvcache_args *a, int num_cus, fa_split_plan *p
     if (!a || !plan) return fail(FA_ERR_NULL, "args or plan is NULL");
     if (num_cus <= 0) num_cus = 256;
     std::memset(plan, 0, sizeof(*plan));
-    const int group = a->nheads / (a->nheads_k > 0 ? a->nheads_k : 1);
+    if (a->batch <= 0 || a->seqlen_q <= 0) return fail(FA_ERR_SHAPE, "batch size and seqlen_q must be positive");
+    if (a->nheads <= 0 || a->nheads_k <= 0 || a->nheads % a->nheads_k != 0)
+        return fail(FA_ERR_SHAPE, "Number of heads in key/value must divide number of heads in query");
+    const int group = a->nheads / a->nheads_k;
     // the int8 latent kernel works on units of 64 query heads and always uses the balanced partition
     const size_t rows = is_mla_i8(a) ? 64 : (size_t)a->seqlen_q * group;
     const size_t slot_bytes = rows * ((size_t)a->headdim_v + 1) * sizeof(float);
