@@ -16,6 +16,8 @@
 //     products, so the running max / sum / rescale never leave the lane (one xor-32 exchange);
 //   * V^T operands come straight from the transposing LDS read (ds_read_b64_tr_b16);
 //   * key tiles outside the causal / window range of the 128-row block are never loaded.
+#include <type_traits>
+
 #include "fa_device.h"
 #include "fa_kernels.h"
 
@@ -38,7 +40,8 @@ template <int D> struct PrefillCfg {
     static constexpr int kPieces = kBN * kChunks / 256;  // 16-byte pieces per thread per tile
 };
 
-template <typename T, int D, bool PAGED, bool SOFTCAP>
+// EXT: packed heads and / or a split of the keys (p.pack, p.nsplits); without it both are compiled out
+template <typename T, int D, bool PAGED, bool SOFTCAP, bool EXT>
 __global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) prefill_kernel(const PrefillParams p) {
     using Cfg = PrefillCfg<D>;
     __shared__ __attribute__((aligned(16))) uint8_t s_k[2][Cfg::kTileBytes];
@@ -51,10 +54,11 @@ __global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) prefill_kernel(const 
     const int ln = lane & 31;   // MFMA row / column
 
     const int mb = gridDim.x - 1 - blockIdx.x;  // tall causal blocks first
-    const int b = (p.nsplits > 1) ? blockIdx.z / p.nsplits : blockIdx.z;
-    const int split = blockIdx.z - b * max(p.nsplits, 1);
+    const int nsplits = EXT ? max(p.nsplits, 1) : 1;
+    const int b = blockIdx.z / nsplits;
+    const int split = blockIdx.z - b * nsplits;
     // tile row R of the block is query R / pg of head h_base + R % pg (pg = 1: one q head per block)
-    const int pg = p.pack;
+    const int pg = EXT ? p.pack : 1;
     const int hk = (pg > 1) ? blockIdx.y : blockIdx.y / p.group;
     const int h_base = (pg > 1) ? blockIdx.y * p.group : blockIdx.y;
 
@@ -85,7 +89,7 @@ __global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) prefill_kernel(const 
     normalize_window(wl, wr_eff, p.causal, norm_m);
     int batch_max = 0;
     if constexpr (PAGED) {
-        if (p.nsplits > 1) batch_max = min(block_max_keys(p.seqused_k, p.batch, p.seqlen_k_add), p.max_blocks * p.page_size);
+        if (nsplits > 1) batch_max = min(block_max_keys(p.seqused_k, p.batch, p.seqlen_k_add), p.max_blocks * p.page_size);
     }
     const int n_rows = Sq * pg;
     const int R0 = mb * kBM;
@@ -97,21 +101,21 @@ __global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) prefill_kernel(const 
     int range_lo = 0, range_hi = Sk;
     bool whole = true;
     int64_t slot = 0;
-    if (p.nsplits > 1) {
+    if (nsplits > 1) {
         int u_lo = 0, u_hi = Sk;
         if (wr_eff >= 0) u_hi = min(Sk, Sq - 1 + off + wr_eff + 1);
         if (wl >= 0) u_lo = max(0, off - wl);
         const bool empty = Sk <= 0 || u_hi <= u_lo;
         const int lo_al = u_lo / 32 * 32;
-        const int sk = adaptive_split_keys(batch_max, p.nsplits);
-        const int ns_row = empty ? 1 : min(p.nsplits, (u_hi - lo_al + sk - 1) / sk);
+        const int sk = adaptive_split_keys(batch_max, nsplits);
+        const int ns_row = empty ? 1 : min(nsplits, (u_hi - lo_al + sk - 1) / sk);
         if (split >= ns_row) return;
         if (!empty) {
             range_lo = max(u_lo, lo_al + split * sk);
             range_hi = (split == ns_row - 1) ? u_hi : min(u_hi, lo_al + (split + 1) * sk);
         }
         whole = ns_row == 1;
-        slot = ((int64_t)b * p.nheads_k + hk) * p.nsplits + split;
+        slot = ((int64_t)b * p.nheads_k + hk) * nsplits + split;
     }
 
     const int my_R = min(R0 + wave * 32 + ln, n_rows - 1);   // rows past the end repeat the last one and are dropped
@@ -468,17 +472,18 @@ template <typename T, int D> static hipError_t launch_prefill_d(const PrefillPar
     dim3 block(256);
     const bool softcap = p.softcap_post != 0.f;
     const bool paged = p.block_table != nullptr;
-    if (paged) {
-        if (softcap)
-            hipLaunchKernelGGL((prefill_kernel<T, D, true, true>), grid, block, 0, stream, p);
-        else
-            hipLaunchKernelGGL((prefill_kernel<T, D, true, false>), grid, block, 0, stream, p);
-    } else {
-        if (softcap)
-            hipLaunchKernelGGL((prefill_kernel<T, D, false, true>), grid, block, 0, stream, p);
-        else
-            hipLaunchKernelGGL((prefill_kernel<T, D, false, false>), grid, block, 0, stream, p);
-    }
+    const bool ext = p.pack > 1 || p.nsplits > 1;
+    auto launch = [&](auto paged_c, auto softcap_c, auto ext_c) {
+        hipLaunchKernelGGL((prefill_kernel<T, D, decltype(paged_c)::value, decltype(softcap_c)::value, decltype(ext_c)::value>),
+                           grid, block, 0, stream, p);
+    };
+    auto pick_ext = [&](auto paged_c, auto softcap_c) {
+        if (ext) launch(paged_c, softcap_c, std::true_type{}); else launch(paged_c, softcap_c, std::false_type{});
+    };
+    auto pick_softcap = [&](auto paged_c) {
+        if (softcap) pick_ext(paged_c, std::true_type{}); else pick_ext(paged_c, std::false_type{});
+    };
+    if (paged) pick_softcap(std::true_type{}); else pick_softcap(std::false_type{});
     return hipGetLastError();
 }
 
