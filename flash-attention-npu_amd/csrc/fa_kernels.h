@@ -98,6 +98,7 @@ struct PrefillParams {
     const int32_t *block_table;    // NULL: dense K/V
     int32_t batch, nheads, nheads_k, group;
     int32_t pack;                  // set by the launcher: 1, or group when tile rows are (query, head) pairs
+    int32_t num_mb, units8;        // set by the launcher: 128-row blocks per unit, units rounded up to 8
     int32_t seqlen_q_fixed, seqlen_k_add;   // kvcache layout: Sq per row, keys appended this call
     int32_t max_seqlen_q, total_q;
     int32_t page_size, max_blocks, num_blocks;

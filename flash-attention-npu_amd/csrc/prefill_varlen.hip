@@ -53,14 +53,36 @@ __global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) prefill_kernel(const 
     const int lh = lane >> 5;   // half: MFMA k-slot
     const int ln = lane & 31;   // MFMA row / column
 
-    const int mb = gridDim.x - 1 - blockIdx.x;  // tall causal blocks first
+    // Workgroup i of the 1-D grid runs on XCD i % 8.  The grid is ordered by 128-row block, tallest
+    // first, and inside a block by position e: XCD lane e % 8 walks the units (sequence, key range,
+    // kv head) congruent to it, the q heads of a unit one after the other.  Every XCD so gets the same
+    // mix of tall and short causal blocks whatever the number of blocks is, and the heads that share
+    // a unit's K/V meet in one L2.
     const int nsplits = EXT ? max(p.nsplits, 1) : 1;
-    const int b = blockIdx.z / nsplits;
-    const int split = blockIdx.z - b * nsplits;
-    // tile row R of the block is query R / pg of head h_base + R % pg (pg = 1: one q head per block)
-    const int pg = EXT ? p.pack : 1;
-    const int hk = (pg > 1) ? blockIdx.y : blockIdx.y / p.group;
-    const int h_base = (pg > 1) ? blockIdx.y * p.group : blockIdx.y;
+    const int pg = EXT ? p.pack : 1;               // tile row R is query R / pg of head h_base + R % pg
+    const int heads_per_unit = (pg > 1) ? 1 : p.group;
+    int mb, unit, head_in_unit;
+    if (p.num_mb > 2) {
+        const int per_block = p.units8 * heads_per_unit;
+        mb = p.num_mb - 1 - (int)(blockIdx.x / per_block);
+        const int e = blockIdx.x % per_block;
+        unit = ((e >> 3) / heads_per_unit) * 8 + (e & 7);
+        head_in_unit = (e >> 3) % heads_per_unit;
+    } else {
+        // one or two blocks per unit (short sequences, all equally light): a unit's blocks stay
+        // neighbours in their XCD's queue, so its K/V are fetched into that L2 once
+        const int per_unit = p.num_mb * heads_per_unit;
+        const int r = blockIdx.x >> 3;
+        unit = (r / per_unit) * 8 + (blockIdx.x & 7);
+        head_in_unit = (r % per_unit) / p.num_mb;
+        mb = p.num_mb - 1 - r % p.num_mb;
+    }
+    if (unit >= p.batch * nsplits * p.nheads_k) return;
+    const int z = unit / p.nheads_k;
+    const int hk = unit - z * p.nheads_k;
+    const int b = z / nsplits;
+    const int split = z - b * nsplits;
+    const int h_base = hk * p.group + ((pg > 1) ? 0 : head_in_unit);
 
     int q0, Sq, k0 = 0, Sk;
     if (p.cu_seqlens_q) {
@@ -466,9 +488,13 @@ int prefill_tiles(int nheads, int nheads_k, int max_seqlen_q) {
 template <typename T, int D> static hipError_t launch_prefill_d(const PrefillParams &p_in, hipStream_t stream) {
     PrefillParams p = p_in;
     p.pack = prefill_pack(p.group, p.max_seqlen_q);
-    const int num_mb = (p.max_seqlen_q * p.pack + kBM - 1) / kBM;
+    p.num_mb = (p.max_seqlen_q * p.pack + kBM - 1) / kBM;
     if (p.nsplits > 1 && (!p.block_table || p.cu_seqlens_q || !p.o_partial)) return hipErrorInvalidValue;
-    dim3 grid(num_mb, p.pack > 1 ? p.nheads_k : p.nheads, p.batch * max(p.nsplits, 1));
+    const int64_t units = (int64_t)p.batch * max(p.nsplits, 1) * p.nheads_k;
+    p.units8 = (int32_t)((units + 7) / 8 * 8);
+    const int64_t wgs = (int64_t)p.num_mb * p.units8 * (p.pack > 1 ? 1 : p.group);
+    if (wgs <= 0 || wgs >= (1ll << 31)) return hipErrorInvalidValue;
+    dim3 grid((unsigned)wgs);
     dim3 block(256);
     const bool softcap = p.softcap_post != 0.f;
     const bool paged = p.block_table != nullptr;
