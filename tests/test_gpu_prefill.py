@@ -261,3 +261,18 @@ def test_kvcache_tall_split_with_append_and_rotary():
                                              causal=True, rotary_interleaved=False, mode="fp32")
     assert torch.equal(dev["k_cache"].cpu().view(torch.int16), kc.view(torch.int16))
     check_out(out, ref, lse, ref_lse, "tall split append rotary")
+
+
+def test_varlen_empty_sequences():
+    # a sequence without query tokens, one without keys (its rows: 0 and +inf), one with neither
+    from flash_attn_npu import flash_attn_varlen_func
+    c = varlen_case([40, 0, 25, 0, 130], [40, 70, 0, 0, 300], 8, 2, 128, seed=51)
+    for causal in (False, True):
+        got, ref, gold = run_varlen(c, causal=causal)
+        check_out(got[0], ref[0], got[1], ref[1], "empty sequences")
+        a, e = int(c["cu_q"][2]), int(c["cu_q"][3])
+        assert torch.count_nonzero(got[0][a:e]) == 0 and torch.isinf(got[1][:, a:e]).all()
+    total0 = torch.zeros(0, 8, 128, dtype=torch.bfloat16, device="cuda")
+    cu0 = torch.zeros(3, dtype=torch.int32, device="cuda")
+    out = flash_attn_varlen_func(total0, c["k"].cuda(), c["v"].cuda(), cu0, c["cu_k"].cuda()[:3], 1, 70)
+    assert out.shape == (0, 8, 128)
