@@ -104,8 +104,8 @@ def _varlen_forward_eager(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max
 
 
 # ------------------------------------------------------------------ kvcache forward custom op
-@torch.library.custom_op("flash_attn_npu::_flash_attn_kvcache_forward", mutates_args=("k_cache", "v_cache"),
-                         device_types="cuda")
+@torch.library.custom_op("flash_attn_npu::_flash_attn_kvcache_forward",
+                         mutates_args=("k_cache", "v_cache", "k_scale_cache", "v_scale_cache"), device_types="cuda")
 def _flash_attn_kvcache_forward(
     q: torch.Tensor,
     k_cache: torch.Tensor,
@@ -126,8 +126,8 @@ def _flash_attn_kvcache_forward(
     softcap: float,
     rotary_interleaved: bool,
     num_splits: int,
-    k_scale_cache: Optional[torch.Tensor] = None,
-    v_scale_cache: Optional[torch.Tensor] = None,
+    k_scale_cache: Optional[torch.Tensor],   # no defaults: the dispatcher drops trailing default arguments,
+    v_scale_cache: Optional[torch.Tensor],   # and a mutated argument must be there to be version-bumped
 ) -> Tuple[torch.Tensor, torch.Tensor]:
     out, softmax_lse = flash_attn_npu.fwd_kvcache(
         q, k_cache, v_cache, k, v, cache_seqlens, rotary_cos, rotary_sin, cache_batch_idx, cache_leftpad,
@@ -141,7 +141,7 @@ def _flash_attn_kvcache_forward(
 def _flash_attn_kvcache_forward_fake(
     q, k_cache, v_cache, k, v, cache_seqlens, rotary_cos, rotary_sin, cache_batch_idx, cache_leftpad, block_table,
     alibi_slopes, softmax_scale, causal, window_size_left, window_size_right, softcap, rotary_interleaved, num_splits,
-    k_scale_cache=None, v_scale_cache=None,
+    k_scale_cache, v_scale_cache,
 ):
     B, sq, hq, _ = q.shape
     out = torch.empty((B, sq, hq, v_cache.shape[-1]), dtype=q.dtype, device=q.device)
