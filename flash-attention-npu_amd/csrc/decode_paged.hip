@@ -555,7 +555,7 @@ __device__ __forceinline__ void combine_row_block(const DecodeParams &p, int b, 
 }
 
 // Balanced mode: blockIdx = (row group, kv head, batch row).  The workgroup recomputes the partition,
-// finds the unit's pieces and merges query rows 4*blockIdx.x .. +3, then 4*gridDim.x further on, ...
+// finds the unit's pieces and merges its share of the query rows
 template <typename T, int D>
 __global__ void __launch_bounds__(256) splitkv_combine_balanced_kernel(const DecodeParams p) {
     __shared__ int s_pref[257];
@@ -576,9 +576,8 @@ __global__ void __launch_bounds__(256) splitkv_combine_balanced_kernel(const Dec
             combine_row_wave<T, D>(p, b, kvh, row, pcs.ns, [&](int s) { return pcs.slot(s); });
         return;
     }
-    // many pieces: the whole workgroup on one row at a time, four consecutive rows per workgroup
-    for (int row0 = blockIdx.x * 4; row0 < p.rows; row0 += gridDim.x * 4)
-        for (int row = row0; row < min(row0 + 4, p.rows); ++row) combine_row_block<T, D>(p, b, kvh, row, pcs);
+    // many pieces: the whole workgroup on one row at a time
+    for (int row = blockIdx.x; row < p.rows; row += gridDim.x) combine_row_block<T, D>(p, b, kvh, row, pcs);
 }
 
 template <typename T, int D, int RT>
@@ -627,9 +626,10 @@ int decode_wgs_per_cu(int headdim, int rows) { return (headdim <= 128 && rows <=
 
 template <typename T, int D> static void launch_combine_d(const DecodeParams &p, hipStream_t stream) {
     if (p.balanced) {
-        // one workgroup per unit when there are many units, one per four query rows when there are few
+        // one workgroup per unit when there are many units, up to one per query row when there are few (units
+        // of few pieces use the first quarter of them, four rows each)
         const int units = p.nheads_k * p.batch;
-        const int row_groups = max(1, min((p.rows + 3) / 4, 1024 / max(units, 1)));
+        const int row_groups = max(1, min(p.rows, 1024 / max(units, 1)));
         hipLaunchKernelGGL((splitkv_combine_balanced_kernel<T, D>), dim3(row_groups, p.nheads_k, p.batch), dim3(256), 0,
                            stream, p);
     } else {
