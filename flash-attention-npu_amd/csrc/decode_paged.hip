@@ -605,7 +605,7 @@ template <typename T, int D> static hipError_t launch_decode_d(const DecodeParam
     const int rt = (p.rows + 15) / 16;
     if (rt <= 1) return launch_decode_rt<T, D, 1>(p, stream);
     if (rt <= 2) return launch_decode_rt<T, D, 2>(p, stream);
-    return launch_decode_rt<T, D, 4>(p, stream);
+    return hipErrorInvalidValue;   // taller blocks belong to the tiled kernel (kDecodeMaxRows)
 }
 
 template <typename T> static hipError_t launch_decode_t(const DecodeParams &p, int headdim, hipStream_t stream) {

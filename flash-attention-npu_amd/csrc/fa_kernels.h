@@ -138,7 +138,11 @@ hipError_t launch_prefill(const PrefillParams &p, int dtype, int headdim, hipStr
 // Resident decode workgroups per compute unit for a head dimension / query-block height.
 int decode_wgs_per_cu(int headdim, int rows);
 
-// Largest query block (seqlen_q * group) the decode kernel packs into one workgroup.
-constexpr int kDecodeMaxRows = 64;
+// Largest query block (seqlen_q * group) that runs on the decode kernels: one or two 16-row MFMA
+// tiles.  Taller blocks run on the tiled kernel with the GQA heads packed into its 128-row tiles, which
+// measures faster from 33 rows on for every head dimension and batch shape tried (a four-tile decode
+// variant existed: 64 rows x 8 K keys x 64 sequences 552 vs 468 us, ragged 256 x 2 K 712 vs 351 us,
+// D = 256 2131 vs 937 us).
+constexpr int kDecodeMaxRows = 32;
 
 }  // namespace fa

@@ -144,7 +144,7 @@ int fa_rocm_num_cus(void);
  *     are computed on the device from cache_seqlens.
  *   mode FA_SPLIT_GRID (num_splits >= 1): every unit is cut into at most `nsplits` ranges of
  *     `split_keys` keys (a multiple of 256); num_splits == 1 gives nsplits == 1 (no split).
- *     Query blocks of more than 64 rows (seqlen_q * nheads / nheads_k) run on the tiled kernel and
+ *     Query blocks of more than 32 rows (seqlen_q * nheads / nheads_k) run on the tiled kernel and
  *     always get this mode: num_splits == 0 then picks as many ranges as it takes to fill the device
  *     when the tiles alone cannot (at most 64, at least 1024 addressable keys each), and
  *     `split_keys` is 0: the range length is set on the device from the longest sequence.

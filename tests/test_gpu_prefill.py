@@ -107,7 +107,7 @@ def test_varlen_paged_kv():
 
 @pytest.mark.parametrize("sq,hq,hk", [(128, 8, 2), (1024, 4, 4), (33, 8, 1), (17, 16, 2)])
 def test_kvcache_tall_query_blocks(sq, hq, hk):
-    # chunked prefill through the kvcache call: seqlen_q * group > 64 runs on the tiled kernel
+    # chunked prefill through the kvcache call: seqlen_q * group > 32 runs on the tiled kernel
     from flash_attn_npu import flash_attn_with_kvcache
     case = make_paged_case(2, hq, hk, 128, 128, [2048, 1100], seqlen_q=sq, seqlen_new=0, seed=10)
     dev = to_dev(case)
@@ -197,7 +197,7 @@ def test_tall_query_block_with_append_and_rotary(interleaved, causal):
 @pytest.mark.parametrize("sq,hq,hk,d", [(16, 64, 8, 128), (20, 12, 2, 128), (9, 24, 3, 64), (40, 10, 2, 256), (100, 6, 2, 128)])
 @pytest.mark.parametrize("causal,window", [(True, (-1, -1)), (False, (-1, -1)), (False, (30, 3)), (True, (100, 0))])
 def test_kvcache_short_blocks_packed_heads(sq, hq, hk, d, causal, window):
-    # seqlen_q * group > 64 with fewer than 128 query rows per head: the tile rows are (query, head)
+    # seqlen_q * group > 32 with fewer than 128 query rows per head: the tile rows are (query, head)
     # pairs of one kv head; groups that do not divide 128 (6, 8 of 3, 5) put a query's heads in two tiles
     from flash_attn_npu import flash_attn_with_kvcache
     case = make_paged_case(3, hq, hk, d, 64, [700, 64, sq], seqlen_q=sq, seed=31, dtype=torch.float16)
