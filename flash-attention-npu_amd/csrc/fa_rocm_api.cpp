@@ -56,6 +56,17 @@ size_t tall_q_bytes(const fa_kvcache_args *a) {
     return (n + 255) / 256 * 256;
 }
 
+// Tallest query block (rows = seqlen_q * group) that runs on the decode kernels.
+int decode_max_rows(const fa_kvcache_args *a) {
+    // tuning aid: FA_ROCM_DECODE_MAX_ROWS (16 or 32) overrides the rule
+    if (const char *env = std::getenv("FA_ROCM_DECODE_MAX_ROWS")) {
+        const int v = std::atoi(env);
+        if (v == 16 || v == 32) return v;
+    }
+    (void)a;
+    return fa::kDecodeMaxRows;
+}
+
 int64_t live_keys_bound(const fa_kvcache_args *a) {
     int64_t cap = (int64_t)a->max_blocks_per_seq * a->page_size;
     const int wr = a->causal ? 0 : a->window_right;
@@ -156,7 +167,7 @@ int fa_rocm_plan_kvcache(const fa_kvcache_args *a, int num_cus, fa_split_plan *p
     // the int8 latent kernel works on units of 64 query heads and always uses the balanced partition
     const size_t rows = is_mla_i8(a) ? 64 : (size_t)a->seqlen_q * group;
     const size_t slot_bytes = rows * ((size_t)a->headdim_v + 1) * sizeof(float);
-    if (!is_mla_i8(a) && rows > (size_t)fa::kDecodeMaxRows) {
+    if (!is_mla_i8(a) && rows > (size_t)decode_max_rows(a)) {
         // Query block too tall for the decode kernels: the tiled forward.  When its tiles alone
         // cannot fill the device (few sequences, short blocks) the keys of every unit are cut into
         // ranges as well; the range length is sized on the device from the longest sequence, so only
@@ -172,7 +183,7 @@ int fa_rocm_plan_kvcache(const fa_kvcache_args *a, int num_cus, fa_split_plan *p
             const int64_t slots = (int64_t)num_cus * (a->headdim_qk <= 128 ? 2 : 1);
             if (tiles * 2 <= slots) n = (slots + tiles - 1) / tiles;
         }
-        const int64_t most = (bound + 1023) / 1024;   // at least 1024 keys per range
+        const int64_t most = (bound + 255) / 256;   // at least 256 keys (four tiles) per range
         if (n > most) n = most;
         if (n > 64) n = 64;
         if (n < 1) n = 1;
@@ -308,7 +319,7 @@ static int fwd_kvcache_impl(const fa_kvcache_args *a, void *stream_, void *const
 
     const bool local = a->window_left >= 0 || a->window_right >= 0;
 
-    if (!is_mla_i8(a) && rows > fa::kDecodeMaxRows) {
+    if (!is_mla_i8(a) && rows > decode_max_rows(a)) {
         // query block too tall for the decode kernel: tiled forward over the paged cache
         int cus_t = device_cus();
         if (cus_t <= 0) cus_t = 256;

@@ -146,7 +146,7 @@ int fa_rocm_num_cus(void);
  *     `split_keys` keys (a multiple of 256); num_splits == 1 gives nsplits == 1 (no split).
  *     Query blocks of more than 32 rows (seqlen_q * nheads / nheads_k) run on the tiled kernel and
  *     always get this mode: num_splits == 0 then picks as many ranges as it takes to fill the device
- *     when the tiles alone cannot (at most 64, at least 1024 addressable keys each), and
+ *     when the tiles alone cannot (at most 64, at least 256 addressable keys each), and
  *     `split_keys` is 0: the range length is set on the device from the longest sequence.
  * Pure host integer code: needs no GPU.  `num_cus` <= 0 means 256.
  */

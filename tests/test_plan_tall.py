@@ -1,6 +1,6 @@
 """Host plan of kvcache calls whose query block goes to the tiled kernel (no GPU needed): the keys
 are cut into ranges only when the tiles alone cannot fill the device, never into ranges shorter than
-1024 keys, and the workspace holds the rotated q (rotary) in front of the partials."""
+256 keys, and the workspace holds the rotated q (rotary) in front of the partials."""
 import ctypes as C
 
 from flash_attn_npu import _lib
@@ -27,12 +27,12 @@ def test_tall_plan():
     # 64 sequences x 8 kv heads of packed 128-row tiles fill the 512 slots: no cut
     p = plan_of(64, 16, 64, 8, 128, 32)
     assert p.mode == 0 and p.nsplits == 1 and p.workspace_bytes == 0
-    # one sequence: 8 tiles for 512 slots -> 64 ranges at most, 1024 keys each at least
+    # one sequence: 8 tiles for 512 slots -> 64 ranges at most, 256 keys each at least
     p = plan_of(1, 16, 64, 8, 128, 512)
     assert p.nsplits == 64 and p.workspace_bytes == 1 * 8 * 64 * rows * 129 * 4
-    p = plan_of(1, 16, 64, 8, 128, 16)          # 4096 addressable keys: 4 ranges
-    assert p.nsplits == 4
-    p = plan_of(1, 16, 64, 8, 128, 2)           # 512 keys: nothing to cut
+    p = plan_of(1, 16, 64, 8, 128, 16)          # 4096 addressable keys: 16 ranges
+    assert p.nsplits == 16
+    p = plan_of(1, 16, 64, 8, 128, 1)           # 256 keys: nothing to cut
     assert p.nsplits == 1 and p.workspace_bytes == 0
     # explicit counts: 1 = never, n = at most n
     assert plan_of(1, 16, 64, 8, 128, 512, num_splits=1).nsplits == 1
@@ -42,4 +42,4 @@ def test_tall_plan():
     # rotary: the rotated q (rounded up to 256 bytes) comes first
     q_bytes = 1 * 24 * 16 * 128 * 2
     p = plan_of(1, 24, 16, 2, 128, 32, rotary=True)
-    assert p.nsplits == 8 and p.workspace_bytes == q_bytes + 1 * 2 * 8 * (24 * 8) * 129 * 4
+    assert p.nsplits == 32 and p.workspace_bytes == q_bytes + 1 * 2 * 32 * (24 * 8) * 129 * 4
