@@ -197,7 +197,9 @@ int fa_rocm_plan_kvcache(const fa_kvcache_args *a, int num_cus, fa_split_plan *p
         plan->nsplits = 1;
         const int per_cu = is_mla_i8(a) ? 1 : fa::decode_wgs_per_cu(a->headdim_qk, (int)rows);
         plan->num_wgs = num_cus * per_cu;
-        plan->min_share = 1;
+        // latent kernel: a piece costs ~15 us of pipeline fill and a 131 KB partial, so tiny launches are
+        // not cut below 4 chunks per workgroup (1 sequence x 8 K tokens: 46 -> 37 us)
+        plan->min_share = is_mla_i8(a) ? 4 : 1;
         // tuning aid: FA_ROCM_DECODE_WGS overrides the workgroup count of the balanced partition
         if (const char *env = std::getenv("FA_ROCM_DECODE_WGS")) {
             const int v = std::atoi(env);
