@@ -131,8 +131,6 @@ def _identity_table(batch: int, device) -> torch.Tensor:
     """(batch, 1) int32 table 0..batch-1, built once per (device, batch)."""
     key = ("id", batch, str(device))
     if key not in _tables:
-        if len(_tables) >= 256:   # many distinct shapes: start over rather than grow without bound
-            _tables.clear()
         _tables[key] = torch.arange(batch, dtype=torch.int32, device=device).view(batch, 1)
     return _tables[key]
 
@@ -140,8 +138,6 @@ def _identity_table(batch: int, device) -> torch.Tensor:
 def _full_lengths(batch: int, seqlen: int, device) -> torch.Tensor:
     key = ("len", batch, seqlen, str(device))
     if key not in _tables:
-        if len(_tables) >= 256:
-            _tables.clear()
         _tables[key] = torch.full((batch,), seqlen, dtype=torch.int32, device=device)
     return _tables[key]
 
