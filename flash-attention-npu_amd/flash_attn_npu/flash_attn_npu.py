@@ -124,6 +124,8 @@ def _fwd_kvcache_padded(q, kcache, vcache, k_, v_, seqlens_k_, rotary_cos_, rota
     return [out, lse]
 
 
+# Small constant tensors, one per (shape, device), never evicted: a captured HIP graph may hold
+# their addresses long after the call that made them.
 _tables = {}
 
 
