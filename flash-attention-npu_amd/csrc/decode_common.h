@@ -53,33 +53,52 @@ __device__ __forceinline__ UnitRange unit_range(const DecodeParams &p, int b, in
     return u;
 }
 
-// exclusive prefix of per-row chunk counts over 256 equal segments of the batch: s_pref[t] =
-// chunks of rows [0, t*seg); s_pref[256] = total.  All threads of the block must call (256 or more
-// threads; the first 256 do the work).  Returns whether some batch row has no visible key at all.
-__device__ __forceinline__ bool batch_chunk_prefix(const DecodeParams &p, int *s_pref, int seg, int M) {
-    __shared__ int s_wave[4];
+// Length of a unit in the list that the partition cuts: its chunks plus `cost`, the fixed cost of
+// starting on a unit (lengths -> table -> keys, q staging, pipeline fill, the stores) in units of one
+// chunk's streaming time.  The cost sits at the beginning of the unit's interval, so a worker whose
+// share holds the start of a further unit gets that many fewer chunks.  Partition::cost is
+// p.piece_cost when the shares are long against it and 0 otherwise: every worker pays for its first
+// piece anyway, and with shares of a few chunks charging the unit starts would unbalance them.
+__device__ __forceinline__ int unit_cost(int nchunks, int cost) { return nchunks > 0 ? nchunks + cost : 0; }
+
+// exclusive prefixes over 256 equal segments of the batch: s_pref[t] = chunks of rows [0, t*seg),
+// s_cnt[t] = rows among them with a visible key; [256] = totals.  All threads of the block must call
+// (256 or more threads; the first 256 do the work).  Returns whether some batch row has no visible key.
+__device__ __forceinline__ bool batch_chunk_prefix(const DecodeParams &p, int *s_pref, int *s_cnt, int seg, int M) {
+    __shared__ int s_wave[4], s_wave_cnt[4];
     const int tid = threadIdx.x;
-    int sum = 0;
-    bool empty_row = false;
+    int sum = 0, cnt = 0;
     for (int b = tid * seg; b < min(p.batch, (tid + 1) * seg); ++b) {
         const int n = unit_range(p, b, M).nchunks;
         sum += n;
-        empty_row |= (n == 0);
+        cnt += (n > 0);
     }
-    int inc = sum;
+    const bool empty_row = tid * seg < p.batch && cnt < min(p.batch, (tid + 1) * seg) - tid * seg;
+    int inc = sum, inc_cnt = cnt;
 #pragma unroll
     for (int d = 1; d < 64; d <<= 1) {
         const int v = __shfl_up(inc, d, 64);
-        if ((tid & 63) >= d) inc += v;
+        const int vc = __shfl_up(inc_cnt, d, 64);
+        if ((tid & 63) >= d) {
+            inc += v;
+            inc_cnt += vc;
+        }
     }
-    if ((tid & 63) == 63 && tid < 256) s_wave[tid >> 6] = inc;
+    if ((tid & 63) == 63 && tid < 256) {
+        s_wave[tid >> 6] = inc;
+        s_wave_cnt[tid >> 6] = inc_cnt;
+    }
     const bool any_empty = __syncthreads_or(empty_row ? 1 : 0) != 0;
     if (tid < 256) {
-        int base = 0;
-        for (int w = 0; w < (tid >> 6); ++w) base += s_wave[w];
+        int base = 0, base_cnt = 0;
+        for (int w = 0; w < (tid >> 6); ++w) {
+            base += s_wave[w];
+            base_cnt += s_wave_cnt[w];
+        }
         s_pref[tid + 1] = base + inc;
+        s_cnt[tid + 1] = base_cnt + inc_cnt;
     }
-    if (tid == 0) s_pref[0] = 0;
+    if (tid == 0) s_pref[0] = s_cnt[0] = 0;
     __syncthreads();
     return any_empty;
 }
@@ -102,12 +121,12 @@ __device__ __forceinline__ RowId row_id(const DecodeParams &p, int kvh, int row)
 
 struct UnitPos {
     int b;          // batch row
-    int pref;       // chunks of rows before b (one kv head's worth)
+    int pref;       // list length of the rows before b (one kv head's worth)
 };
 
 // batch row whose units contain list position `pos` (0 <= pos < Hk * total)
 __device__ __forceinline__ UnitPos locate_row(const DecodeParams &p, const int *s_pref, int seg, int64_t pos, int M,
-                                              int list_heads) {
+                                              int list_heads, int cost) {
     const int target = (int)(pos / list_heads);  // rows with pref <= target < pref + n
     int lo = 0, hi = 256;                        // segment t with s_pref[t] <= target < s_pref[t+1]
     while (hi - lo > 1) {
@@ -118,7 +137,7 @@ __device__ __forceinline__ UnitPos locate_row(const DecodeParams &p, const int *
     u.b = lo * seg;
     u.pref = s_pref[lo];
     for (;;) {
-        const int n = unit_range(p, u.b, M).nchunks;
+        const int n = unit_cost(unit_range(p, u.b, M).nchunks, cost);
         if (target < u.pref + n || u.b + 1 >= p.batch) break;
         u.pref += n;
         ++u.b;
@@ -203,6 +222,7 @@ struct Partition {
     int M;          // window normalisation key count
     int seg;        // batch rows per prefix segment
     int list_heads; // kv heads inside the list: nheads_k (plain) or 1 (head-interleaved)
+    int cost;       // list length charged per unit on top of its chunks (unit_cost)
     int64_t W, S;
     bool any_empty; // some batch row has no visible key
     __device__ __forceinline__ int64_t worker_of(int64_t share, int kvh, int hk) const {
@@ -216,10 +236,18 @@ __device__ __forceinline__ Partition make_partition(const DecodeParams &p, int *
     Partition pt;
     pt.seg = (p.batch + 255) / 256;
     pt.M = window_norm_m(p);
-    pt.any_empty = batch_chunk_prefix(p, s_pref, pt.seg, pt.M);
+    __shared__ int s_cnt[257];
+    pt.any_empty = batch_chunk_prefix(p, s_pref, s_cnt, pt.seg, pt.M);
     pt.list_heads = p.head_interleave ? 1 : p.nheads_k;
-    pt.W = (int64_t)s_pref[256] * pt.list_heads;
     const int64_t shares = p.head_interleave ? max(p.num_workers / p.nheads_k, 1) : p.num_workers;
+    const int64_t chunks = (int64_t)s_pref[256] * pt.list_heads;
+    pt.cost = (p.piece_cost > 0 && chunks >= 4 * (int64_t)p.piece_cost * shares) ? p.piece_cost : 0;
+    if (pt.cost > 0) {   // block-uniform: the prefix becomes one of list lengths
+        __syncthreads();
+        for (int t = threadIdx.x; t < 257; t += blockDim.x) s_pref[t] += pt.cost * s_cnt[t];
+        __syncthreads();
+    }
+    pt.W = (int64_t)s_pref[256] * pt.list_heads;
     pt.S = max((pt.W + shares - 1) / shares, (int64_t)max(p.min_share, 1));
     return pt;
 }
@@ -228,15 +256,19 @@ __device__ __forceinline__ Partition make_partition(const DecodeParams &p, int *
 __device__ __forceinline__ int chunks_before(const DecodeParams &p, const Partition &pt, const int *s_pref, int b) {
     const int t = b / pt.seg;
     int pref = s_pref[t];
-    for (int bb = t * pt.seg; bb < b; ++bb) pref += unit_range(p, bb, pt.M).nchunks;
+    for (int bb = t * pt.seg; bb < b; ++bb) pref += unit_cost(unit_range(p, bb, pt.M).nchunks, pt.cost);
     return pref;
 }
 
-__device__ __forceinline__ UnitPieces unit_pieces(const Partition &pt, int64_t unit_start, int nchunks, int kvh, int hk) {
+// unit_start: list position of the unit's interval (its piece cost first, then its chunks)
+__device__ __forceinline__ UnitPieces unit_pieces(const Partition &pt, int64_t unit_start, int nchunks, int kvh, int hk,
+                                                  int piece_cost) {
     UnitPieces pcs;
-    pcs.g_first = unit_start / pt.S;
-    pcs.ns = (int)((unit_start + nchunks - 1) / pt.S - pcs.g_first + 1);
-    pcs.first_is_late = (unit_start != pcs.g_first * pt.S);
+    const int64_t first_chunk = unit_start + piece_cost;
+    pcs.g_first = first_chunk / pt.S;
+    pcs.ns = (int)((first_chunk + nchunks - 1) / pt.S - pcs.g_first + 1);
+    // the worker of piece 0 had a piece of an earlier unit before it iff its share begins before this unit
+    pcs.first_is_late = (pcs.g_first * pt.S < unit_start);
     pcs.stride = (pt.list_heads == 1) ? hk : 1;
     pcs.offset = (pt.list_heads == 1) ? kvh : 0;
     return pcs;
@@ -255,22 +287,28 @@ __device__ __forceinline__ void walk_share(const DecodeParams &p, const Partitio
     int64_t pos = share * pt.S;
     const int64_t end = min(pt.W, pos + pt.S);
     if (pos >= end) return;
-    UnitPos up = locate_row(p, s_pref, pt.seg, pos, pt.M, pt.list_heads);
+    UnitPos up = locate_row(p, s_pref, pt.seg, pos, pt.M, pt.list_heads, pt.cost);
     UnitRange ur = unit_range(p, up.b, pt.M);
     const int64_t row_start = (int64_t)up.pref * pt.list_heads;   // list position of unit (b, 0)
-    int kvh = (int)((pos - row_start) / ur.nchunks);
-    int offset = (int)((pos - row_start) - (int64_t)kvh * ur.nchunks);  // chunks into the unit
+    int ucost = unit_cost(ur.nchunks, pt.cost);
+    int kvh = (int)((pos - row_start) / ucost);
+    int cost_off = (int)((pos - row_start) - (int64_t)kvh * ucost);  // offset into the unit's interval
     bool first = true;
     while (pos < end) {
-        const int take = (int)min((int64_t)(ur.nchunks - offset), end - pos);
-        const bool whole = (offset == 0) && (take == ur.nchunks);
-        const int c_lo = ur.c0 + offset;
-        const int range_lo = max(ur.lo, c_lo * kChunk);
-        const int range_hi = min(ur.hi, (c_lo + take) * kChunk);
-        piece(up.b, inter ? fixed_kvh : kvh, ur, range_lo, range_hi, whole, worker * 2 + (first ? 0 : 1));
-        first = false;
-        pos += take;
-        offset = 0;
+        const int take_cost = (int)min((int64_t)(ucost - cost_off), end - pos);
+        // the chunks of the unit that this stretch of its interval holds
+        const int off_lo = max(0, cost_off - pt.cost);
+        const int off_hi = max(0, cost_off + take_cost - pt.cost);
+        if (off_hi > off_lo) {
+            const bool whole = (off_lo == 0) && (off_hi == ur.nchunks);
+            const int c_lo = ur.c0 + off_lo;
+            const int range_lo = max(ur.lo, c_lo * kChunk);
+            const int range_hi = min(ur.hi, (ur.c0 + off_hi) * kChunk);
+            piece(up.b, inter ? fixed_kvh : kvh, ur, range_lo, range_hi, whole, worker * 2 + (first ? 0 : 1));
+            first = false;
+        }
+        pos += take_cost;
+        cost_off = 0;
         if (++kvh == pt.list_heads) {
             kvh = 0;
             do {
@@ -278,6 +316,7 @@ __device__ __forceinline__ void walk_share(const DecodeParams &p, const Partitio
                 if (up.b < p.batch) ur = unit_range(p, up.b, pt.M);
             } while (up.b < p.batch && ur.nchunks == 0);
             if (up.b >= p.batch) break;
+            ucost = unit_cost(ur.nchunks, pt.cost);
         }
     }
 }

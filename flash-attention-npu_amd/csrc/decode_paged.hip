@@ -565,8 +565,8 @@ __global__ void __launch_bounds__(256) splitkv_combine_balanced_kernel(const Dec
     const UnitRange ur = unit_range(p, b, pt.M);
     if (ur.nchunks == 0) return;   // the decode kernel initialised this unit
     const int64_t start = (int64_t)chunks_before(p, pt, s_pref, b) * pt.list_heads +
-                          (pt.list_heads == 1 ? 0 : (int64_t)kvh * ur.nchunks);
-    const UnitPieces pcs = unit_pieces(pt, start, ur.nchunks, kvh, p.nheads_k);
+                          (pt.list_heads == 1 ? 0 : (int64_t)kvh * unit_cost(ur.nchunks, pt.cost));
+    const UnitPieces pcs = unit_pieces(pt, start, ur.nchunks, kvh, p.nheads_k, pt.cost);
     if (pcs.ns == 1) return;       // written whole by one worker
     if (pcs.ns <= 16) {
         // few pieces: the four waves merge four rows side by side, no barrier and one chain of

@@ -45,6 +45,7 @@ struct DecodeParams {
     int32_t num_workers, min_share;  // workers sharing the chunk list (workgroups, or waves), least chunks per share
     int32_t wave_workers;          // 1: every wave is a worker (num_workers = 4 * num_wgs)
     int32_t head_interleave;       // 1: worker w streams share w / Hk of the per-head list for kv head w % Hk
+    int32_t piece_cost;            // balanced mode: list length charged for starting on a unit, in chunks (decode_common.h)
     int32_t split_adaptive;        // grid mode: keys per split = adaptive_split_keys(longest sequence, nsplits), not split_keys
     int32_t units_per_token;       // latent int8 cache: 64-head groups per query token (nheads_k = seqlen_q * this); else 0
 };

@@ -7,6 +7,7 @@
 // depends on shapes only, per-row lengths are read by the kernels.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
@@ -518,6 +519,12 @@ static int fwd_kvcache_impl(const fa_kvcache_args *a, void *stream_, void *const
     p.min_share = plan.min_share;
     p.wave_workers = plan.num_workers != plan.num_wgs;
     // wave workers of neighbouring kv heads walk the same token range together
+    // Fixed cost of starting on a unit, in chunk times.  Latent kernel: ~15 us of q staging and pipeline
+    // fill against ~2 us per chunk; charging 7 chunks takes the workgroups that start a second unit off
+    // the critical path (c4 kernel 150 -> 145 us).  Wave-level kernel: ~6 us against ~5 us per chunk;
+    // charging 1-3 chunks measured within +-1 %, so it is not charged.
+    p.piece_cost = is_mla_i8(a) ? 7 : 0;
+    if (const char *env = std::getenv("FA_ROCM_PIECE_COST")) p.piece_cost = std::max(0, std::atoi(env));
     p.head_interleave = p.wave_workers && a->nheads_k > 1 && plan.num_workers % a->nheads_k == 0 &&
                         !std::getenv("FA_ROCM_NO_HEAD_INTERLEAVE");
     const bool needs_combine = need > 0;

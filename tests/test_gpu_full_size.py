@@ -202,3 +202,19 @@ def test_c5_packed_prefill_full_size():
             ref, ref_lse = O.flash_attn_varlen(w["q"][a:e].cpu(), w["k"][a:e].cpu(), w["v"][a:e].cpu(), hcu, hcu, e - a,
                                                e - a, causal=True, mode="fp32")
             check_out(out[a:e], ref, lse[:, a:e], ref_lse, f"c5 sequence {b}")
+
+
+@pytest.mark.parametrize("cost", [1, 5])
+def test_c2_partition_charging_unit_starts(cost, monkeypatch):
+    # the balanced partition with a fixed cost per unit start (the latent kernel's default; an
+    # experiment knob for the others): other cuts of the same keys, same appended bytes, same result
+    from bench import decode_workload
+    w = decode_workload("c2", "cuda")
+    k0, v0 = w["k_cache"].clone(), w["v_cache"].clone()
+    base = run_call(w)
+    k1, v1 = w["k_cache"].clone(), w["v_cache"].clone()
+    monkeypatch.setenv("FA_ROCM_PIECE_COST", str(cost))
+    print("full size c2: unit cost", cost, flush=True)
+    got = run_call(w, k_cache=k0, v_cache=v0)
+    close_splits(base, got, f"unit cost {cost}")
+    assert torch.equal(k0, k1) and torch.equal(v0, v1), "appended rows differ"
