@@ -58,7 +58,9 @@ typedef struct fa_kvcache_args {
     const void *k_new;           /* (B, Snew, Hk, Dqk) io dtype or NULL                          */
     const void *v_new;           /* (B, Snew, Hk, Dv)  io dtype or NULL                          */
     const void *rotary_cos;      /* (seqlen_ro, rotary_dim/2) io dtype or NULL                   */
-    const void *rotary_sin;      /* same                                                         */
+    const void *rotary_sin;      /* same.  The caller provides seqlen_ro >= cache_seqlens + Snew; the
+                                    lengths live on the device, so the call cannot check: a position
+                                    past the table uses its last row (no out-of-bounds read)        */
     const int32_t *cache_seqlens;/* (B,) keys already in the cache, per row                      */
     const int32_t *block_table;  /* (B, max_blocks_per_seq) page ids                             */
     void *workspace;             /* >= fa_rocm_kvcache_workspace_bytes(); may be NULL if that is 0 */
