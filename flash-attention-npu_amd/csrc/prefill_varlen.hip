@@ -458,18 +458,40 @@ __global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) prefill_kernel(const 
         }
         return;
     }
-    if (row_ok) {
-        uint16_t *dst = o_row;
+    if (row_ok && lh == 0) *lse_row = (l_run > 0.f) ? (m_run + fast_log2(l_run)) * kLn2 : INFINITY;
+    // The lane owns 8-byte pieces of its row, 16 of them: stored as they are, one instruction would touch
+    // 32 rows of the output.  The wave's 32 x D tile goes through LDS instead (the V tiles are free
+    // after the last barrier of the loop; each wave uses its own part, so no workgroup barrier) and
+    // leaves as whole rows, 16 bytes per lane.
+    constexpr int kStageRow = D * 2 + 16;                      // padded: the 8-byte writes of a column spread over the banks
+    static_assert(4 * 32 * kStageRow <= 2 * Cfg::kVTileBytes, "staging tile must fit the V tiles");
+    uint8_t *stage = &s_v[0][0] + wave * (32 * kStageRow);
 #pragma unroll
-        for (int t = 0; t < Cfg::kMT; ++t)
+    for (int t = 0; t < Cfg::kMT; ++t)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                uint2 o2;
-                o2.x = pack2<T>(o_acc[t][4 * j] * inv, o_acc[t][4 * j + 1] * inv);
-                o2.y = pack2<T>(o_acc[t][4 * j + 2] * inv, o_acc[t][4 * j + 3] * inv);
-                *reinterpret_cast<uint2 *>(dst + t * 32 + 8 * j + 4 * lh) = o2;
-            }
-        if (lh == 0) *lse_row = (l_run > 0.f) ? (m_run + fast_log2(l_run)) * kLn2 : INFINITY;
+        for (int j = 0; j < 4; ++j) {
+            uint2 o2;
+            o2.x = pack2<T>(o_acc[t][4 * j] * inv, o_acc[t][4 * j + 1] * inv);
+            o2.y = pack2<T>(o_acc[t][4 * j + 2] * inv, o_acc[t][4 * j + 3] * inv);
+            *reinterpret_cast<uint2 *>(stage + ln * kStageRow + (t * 32 + 8 * j + 4 * lh) * 2) = o2;
+        }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    constexpr int kLanesPerRow = D * 2 / 16;                   // lanes that cover one row with 16 bytes each
+    constexpr int kStageRows = 64 / kLanesPerRow;              // rows a wave stores per instruction
+    const int piece = lane % kLanesPerRow;
+#pragma unroll
+    for (int r0 = 0; r0 < 32; r0 += kStageRows) {
+        const int rr = r0 + lane / kLanesPerRow;               // row of the wave's tile
+        const int R = R0 + wave * 32 + rr;
+        if (R < n_rows) {
+            const int row = R / pg;
+            const int head = h_base + (R - row * pg);
+            uint16_t *dst = reinterpret_cast<uint16_t *>(p.out) + (int64_t)b * p.o_stride_b + (int64_t)head * p.o_stride_h +
+                            (int64_t)(q0 + row) * p.o_stride_t;
+            store16(dst + piece * 8, *reinterpret_cast<const u32x4_t *>(stage + rr * kStageRow + piece * 16));
+        }
     }
 }
 
