@@ -56,8 +56,10 @@ __global__ void __launch_bounds__(64) append_kv_kernel(const AppendParams p) {
             const float cs = to_float<T>(cosT[(int64_t)rpos * half + c]);
             const float sn = to_float<T>(sinT[(int64_t)rpos * half + c]);
             const float x1 = to_float<T>(o1), x2 = to_float<T>(o2);
-            o1 = from_float<T>(__fsub_rn(__fmul_rn(x1, cs), __fmul_rn(x2, sn)));
-            o2 = from_float<T>(__fadd_rn(__fmul_rn(x1, sn), __fmul_rn(x2, cs)));
+            float r1, r2;
+            rotate_pair(x1, x2, cs, sn, r1, r2);
+            o1 = from_float<T>(r1);
+            o2 = from_float<T>(r2);
         }
         kdst[d1] = o1;
         kdst[d2] = o2;
@@ -145,8 +147,10 @@ __global__ void __launch_bounds__(64) rotate_q_kernel(const RotateQParams p) {
             const float cs = to_float<T>(cosT[(int64_t)rpos * half + c]);
             const float sn = to_float<T>(sinT[(int64_t)rpos * half + c]);
             const float x1 = to_float<T>(o1), x2 = to_float<T>(o2);
-            o1 = from_float<T>(__fsub_rn(__fmul_rn(x1, cs), __fmul_rn(x2, sn)));
-            o2 = from_float<T>(__fadd_rn(__fmul_rn(x1, sn), __fmul_rn(x2, cs)));
+            float r1, r2;
+            rotate_pair(x1, x2, cs, sn, r1, r2);
+            o1 = from_float<T>(r1);
+            o2 = from_float<T>(r2);
         }
         dst[d1] = o1;
         dst[d2] = o2;

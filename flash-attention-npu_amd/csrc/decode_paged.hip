@@ -203,8 +203,8 @@ __device__ __forceinline__ void process_piece(const DecodeParams &p, const int b
                     const float cs = to_float<T>(cosT[(int64_t)pos * half + c]);
                     const float sn = to_float<T>(sinT[(int64_t)pos * half + c]);
                     const float x1 = to_float<T>(o1), x2 = to_float<T>(o2);
-                    const float r1 = __fsub_rn(__fmul_rn(x1, cs), __fmul_rn(x2, sn));
-                    const float r2 = __fadd_rn(__fmul_rn(x1, sn), __fmul_rn(x2, cs));
+                    float r1, r2;
+                    rotate_pair(x1, x2, cs, sn, r1, r2);
                     o1 = from_float<T>(r1);
                     o2 = from_float<T>(r2);
                 }

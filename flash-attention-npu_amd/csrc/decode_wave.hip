@@ -67,8 +67,10 @@ __device__ __forceinline__ void stage_q_wave(const DecodeParams &p, int b, int k
             for (int j = 0; j < 4; ++j) {
                 const float c = to_float<T>(cs[d0 / 2 + j]), s = to_float<T>(sn[d0 / 2 + j]);
                 const float x1 = to_float<T>(x[2 * j]), x2 = to_float<T>(x[2 * j + 1]);
-                o[2 * j] = from_float<T>(__fsub_rn(__fmul_rn(x1, c), __fmul_rn(x2, s)));
-                o[2 * j + 1] = from_float<T>(__fadd_rn(__fmul_rn(x1, s), __fmul_rn(x2, c)));
+                float r1, r2;
+                rotate_pair(x1, x2, c, s, r1, r2);
+                o[2 * j] = from_float<T>(r1);
+                o[2 * j + 1] = from_float<T>(r2);
             }
             *reinterpret_cast<u32x4_t *>(dst) = *reinterpret_cast<const u32x4_t *>(o);
         } else if (d0 < half) {
@@ -83,8 +85,10 @@ __device__ __forceinline__ void stage_q_wave(const DecodeParams &p, int b, int k
             for (int j = 0; j < 8; ++j) {
                 const float c = to_float<T>(cs[d0 + j]), s = to_float<T>(sn[d0 + j]);
                 const float x1 = to_float<T>(x1v[j]), x2 = to_float<T>(x2v[j]);
-                o1[j] = from_float<T>(__fsub_rn(__fmul_rn(x1, c), __fmul_rn(x2, s)));
-                o2[j] = from_float<T>(__fadd_rn(__fmul_rn(x1, s), __fmul_rn(x2, c)));
+                float r1, r2;
+                rotate_pair(x1, x2, c, s, r1, r2);
+                o1[j] = from_float<T>(r1);
+                o2[j] = from_float<T>(r2);
             }
             *reinterpret_cast<u32x4_t *>(dst) = *reinterpret_cast<const u32x4_t *>(o1);
             *reinterpret_cast<u32x4_t *>(dst + half) = *reinterpret_cast<const u32x4_t *>(o2);
@@ -134,8 +138,10 @@ __device__ __forceinline__ void append_rows_wave(const DecodeParams &p, int b, i
                 const float cs = to_float<T>(cosT[(int64_t)rpos * half + c]);
                 const float sn = to_float<T>(sinT[(int64_t)rpos * half + c]);
                 const float x1 = to_float<T>(o1), x2 = to_float<T>(o2);
-                o1 = from_float<T>(__fsub_rn(__fmul_rn(x1, cs), __fmul_rn(x2, sn)));
-                o2 = from_float<T>(__fadd_rn(__fmul_rn(x1, sn), __fmul_rn(x2, cs)));
+                float r1, r2;
+                rotate_pair(x1, x2, cs, sn, r1, r2);
+                o1 = from_float<T>(r1);
+                o2 = from_float<T>(r2);
             }
             kdst[d1] = o1;
             kdst[d2] = o2;

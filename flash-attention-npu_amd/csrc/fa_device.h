@@ -117,6 +117,18 @@ __device__ __forceinline__ float quad_rows_sum(float v) {
     return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
+// One rotary pair: (x1, x2) turned by the angle whose cosine and sine are c and s.  The two products and
+// the sum or difference of each result are separately rounded fp32 operations.  hipcc would otherwise fuse
+// a product into the addition (and, for fp16 results, the conversion as well), which rounds differently on
+// rare inputs; rotated rows are defined to be bit-identical to the unfused evaluation on a CPU.
+__device__ __forceinline__ void rotate_pair(float x1, float x2, float c, float s, float &r1, float &r2) {
+#pragma clang fp contract(off)
+    const float a = x1 * c, b = x2 * s;
+    const float e = x1 * s, f = x2 * c;
+    r1 = a - b;
+    r2 = e + f;
+}
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 

@@ -123,6 +123,57 @@ def test_append_rotary_bit_exact(interleaved, rot):
     check_out(out, ref, lse, ref_lse, "append+rotary")
 
 
+def double_rounding_pairs(count, seed=0):
+    """fp16 rotary inputs (x1, x2, sin; cos = 1) whose fp32 result x1 - x2*sin lies exactly half way between
+    two fp16 values while the unrounded result does not: rounding once (a multiply-add that writes fp16
+    directly) and rounding twice (fp32, then fp16) then disagree for about half of them."""
+    g = torch.Generator().manual_seed(seed)
+    n = 1 << 21
+    x1 = (1 + torch.rand(n, generator=g)).to(torch.float16)
+    x2 = (1 + torch.rand(n, generator=g)).to(torch.float16)
+    sn = ((1 + torch.rand(n, generator=g)) * 2.0 ** -11).to(torch.float16)
+    r32 = x1.float() - x2.float() * sn.float()                      # both operations exact or rounded once, unfused
+    exact = x1.double() - x2.double() * sn.double()
+    tie = ((r32.view(torch.int32) & 0x1FFF) == 0x1000) & (exact != r32.double())
+    idx = tie.nonzero()[:count, 0]
+    assert idx.numel() == count
+    return x1[idx], x2[idx], sn[idx]
+
+
+@pytest.mark.parametrize("num_splits", [0, 2])        # 0: rows appended by the attention kernel, 2: by the append kernel
+@pytest.mark.parametrize("interleaved", [False, True])
+def test_append_rotary_fp16_rounds_in_fp32_first(interleaved, num_splits):
+    # the rotated row is defined as separately rounded fp32 operations followed by one conversion to fp16
+    from flash_attn_npu import flash_attn_with_kvcache
+    snew, half = 2, 64
+    x1, x2, sn = double_rounding_pairs(snew * half)
+    case = make_paged_case(1, 4, 1, 128, 64, [5], seqlen_q=snew, seqlen_new=snew, dtype=torch.float16, seed=21)
+    k = case["k"]
+    if interleaved:
+        k[0, :, 0, 0::2] = x1.view(snew, half)
+        k[0, :, 0, 1::2] = x2.view(snew, half)
+    else:
+        k[0, :, 0, :half] = x1.view(snew, half)
+        k[0, :, 0, half:] = x2.view(snew, half)
+    cos = torch.ones(16, half, dtype=torch.float16)
+    sin = torch.zeros(16, half, dtype=torch.float16)
+    sin[5:5 + snew] = sn.view(snew, half)
+    dev = to_dev(case)
+    flash_attn_with_kvcache(dev["q"], dev["k_cache"], dev["v_cache"], dev["k"], dev["v"], rotary_cos=cos.cuda(),
+                            rotary_sin=sin.cuda(), cache_seqlens=dev["cache_seqlens"], block_table=dev["block_table"],
+                            causal=True, rotary_interleaved=interleaved, num_splits=num_splits)
+    torch.cuda.synchronize()
+    kc, vc = case["k_cache"].clone(), case["v_cache"].clone()
+    O.append_kv(kc, vc, case["k"], case["v"], case["cache_seqlens"], case["block_table"], cos, sin, interleaved)
+    rows = kc[case["block_table"][0, 0].item(), 5:5 + snew, 0]
+    first = rows[:, 0::2] if interleaved else rows[:, :half]
+    # numpy converts float64 to float16 in one rounding (torch goes through float32)
+    once = torch.from_numpy((x1.double() - x2.double() * sn.double()).numpy().astype("float16")).view(snew, half)
+    assert (first != once).sum() >= 16, "the inputs no longer tell one rounding from two"
+    assert torch.equal(dev["k_cache"].cpu().view(torch.int16), kc.view(torch.int16)), "rotated K bytes differ"
+    assert torch.equal(dev["v_cache"].cpu().view(torch.int16), vc.view(torch.int16))
+
+
 def test_append_multi_token_crosses_page():
     case = make_paged_case(2, 8, 2, 128, 256, [254, 510], seqlen_q=3, seqlen_new=3, seed=12)
     got, ref, gold, (dev, kc, vc) = run_both(case, causal=True)
