@@ -8,6 +8,8 @@ import torch
 
 import fa_oracle as O
 from helpers import check_out, make_paged_case, rotary_tables, to_dev
+from test_gpu_dense import make_dense_case, run_dense
+from test_gpu_mla import mla_case
 from test_gpu_prefill import run_varlen, varlen_case
 
 pytestmark = pytest.mark.gpu
@@ -36,10 +38,36 @@ def draw_kvcache(seed):
                 num_splits=num_splits, dtype=dtype, rot=rot, interleaved=interleaved)
 
 
-@pytest.mark.parametrize("seed", range(60))
+def draw_tall(seed):
+    """Query blocks up to 257 tokens x 16 heads per kv head and batches up to 24 rows: the blocks that leave the
+    decode kernels for the tiled one, its packed heads and its key-range split.  Sized so the oracle takes ~0.1 s."""
+    r = random.Random(seed)
+    while True:
+        d = r.choice([64, 128, 128, 256])
+        hk = r.choice([1, 2, 4, 8])
+        group = r.choice([1, 2, 4, 8, 16])
+        sq = r.choice([2, 5, 8, 16, 17, 33, 64, 100, 128, 130, 257])
+        page = r.choice([32, 64, 128, 256])
+        B = r.randint(1, 24)
+        lens = [r.choice([0, 1, 33, r.randint(1, 300), r.randint(300, 2000), r.randint(2000, 6000)]) for _ in range(B)]
+        if hk * group * sq * (sum(lens) + B * sq) * d <= 3e9:
+            break
+    snew = r.choice([0, 0, sq, 1, 3])
+    causal = r.random() < 0.7
+    window = r.choice([(-1, -1), (-1, -1), (-1, -1), (r.randint(0, 500), 0), (r.randint(0, 500), r.randint(0, 100)),
+                       (-1, r.randint(0, 64)), (r.randint(0, 64), -1)])
+    softcap = r.choice([0.0, 0.0, 0.0, 15.0])
+    num_splits = r.choice([0, 0, 0, 1, 2, 4, 9])
+    dtype = r.choice([torch.bfloat16, torch.bfloat16, torch.float16])
+    rot = r.choice([0, 0, 32, d]) if snew else 0
+    return dict(B=B, hq=hk * group, hk=hk, d=d, page=page, lens=lens, sq=sq, snew=snew, causal=causal, window=window,
+                softcap=softcap, num_splits=num_splits, dtype=dtype, rot=rot, interleaved=r.random() < 0.5)
+
+
+@pytest.mark.parametrize("seed", [*range(60), 324, *range(2000, 2060)])     # 324: an fp16 rotary result on an exact tie
 def test_random_kvcache(seed):
     from flash_attn_npu import flash_attn_with_kvcache
-    c = draw_kvcache(1000 + seed)
+    c = draw_kvcache(1000 + seed) if seed < 2000 else draw_tall(seed - 2000)
     print("random kvcache", seed, c, flush=True)
     case = make_paged_case(c["B"], c["hq"], c["hk"], c["d"], c["page"], c["lens"], seqlen_q=c["sq"], seqlen_new=c["snew"],
                            dtype=c["dtype"], seed=seed, extra_table_cols=seed % 2)
@@ -77,3 +105,62 @@ def test_random_varlen(seed):
     c = varlen_case(seqs_q, seqs_k, hq, hk, d, dtype=dtype, seed=seed)
     got, ref, gold = run_varlen(c, causal=causal, window_size=window, softcap=softcap)
     check_out(got[0], ref[0], got[1], ref[1], f"random varlen {seed}")
+
+
+@pytest.mark.parametrize("seed", range(30))
+def test_random_int8_latent(seed):
+    from flash_attn_npu import flash_attn_with_kvcache
+    r = random.Random(7000 + seed)
+    B = r.randint(1, 40)
+    hq = r.choice([64, 128])
+    sq = r.choice([1, 1, 1, 2, 3, 4])
+    page = r.choice([64, 128, 256])
+    lens = [r.choice([0, 1, 255, 257, r.randint(1, 600), r.randint(600, 5000)]) for _ in range(B)]
+    snew = r.choice([0, 0, sq])
+    kw = dict(softmax_scale=192 ** -0.5, causal=r.random() < 0.7,
+              window_size=r.choice([(-1, -1), (-1, -1), (r.randint(0, 600), 0), (-1, r.randint(0, 8))]), softcap=r.choice([0.0, 0.0, 20.0]))
+    num_splits = r.choice([0, 0, 1, 3])
+    print("random int8 latent", seed, dict(B=B, hq=hq, sq=sq, page=page, lens=lens, snew=snew, num_splits=num_splits), kw, flush=True)
+    case = mla_case(B, hq, [l + snew for l in lens], page=page, seed=seed, spare=seed % 3)
+    case["cache_seqlens"] = torch.tensor(lens, dtype=torch.int32)
+    g = torch.Generator().manual_seed(seed + 7)
+    q = torch.randn(B, sq, hq, 576, generator=g).to(torch.bfloat16)
+    kn = torch.randn(B, snew, 1, 576, generator=g).to(torch.bfloat16) if snew else None
+    kc, ks = case["k_cache"].cuda(), case["k_scale"].cuda()
+    knd = kn.cuda() if snew else None
+    out, lse = flash_attn_with_kvcache(q.cuda(), kc, kc[..., :512], knd, knd[..., :512] if snew else None,
+                                       cache_seqlens=case["cache_seqlens"].cuda(), block_table=case["block_table"].cuda(),
+                                       return_softmax_lse=True, k_scale_cache=ks, num_splits=num_splits, **kw)
+    torch.cuda.synchronize()
+    kc_o, ks_o = case["k_cache"].clone(), case["k_scale"].clone()
+    ref, ref_lse = O.flash_attn_with_kvcache(q, kc_o, kc_o[..., :512], kn, kn[..., :512] if snew else None,
+                                             cache_seqlens=case["cache_seqlens"], block_table=case["block_table"],
+                                             k_scale_cache=ks_o, mode="fp32", **kw)
+    assert torch.equal(kc.cpu(), kc_o), "codes differ"
+    assert torch.equal(ks.cpu().view(torch.int32), ks_o.view(torch.int32)), "scales differ"
+    # the kernel rounds P * v_scale to bf16 (2^-8 relative); a row that sees one or two keys carries that into
+    # elements of magnitude 4 unaveraged, which with the output's own half ulp can pass 2e-2 by a few 1e-3
+    check_out(out, ref, lse, ref_lse, f"random int8 latent {seed}", rel=2.0 ** -8)
+
+
+@pytest.mark.parametrize("seed", range(30))
+def test_random_dense(seed):
+    r = random.Random(9000 + seed)
+    B = r.randint(1, 8)
+    d = r.choice([64, 128, 256])
+    hk = r.choice([1, 2, 8])
+    hq = hk * r.choice([1, 4, 8])
+    sq = r.choice([1, 1, 2, 7, 40])
+    s_cache = r.choice([64, 100, 512, 1111, 3000])
+    snew = r.choice([0, 1, sq])
+    lens = None if (snew == 0 and r.random() < 0.3) else [r.randint(0, s_cache - snew) for _ in range(B)]
+    b_cache = B + r.choice([0, 0, 3])
+    idx = torch.tensor(r.sample(range(b_cache), B), dtype=torch.int32) if r.random() < 0.5 else None
+    causal, num_splits = r.random() < 0.6, r.choice([0, 0, 1, 3])
+    dtype = r.choice([torch.bfloat16, torch.float16])
+    case = make_dense_case(B, hq, hk, d, s_cache, lens, seqlen_q=sq, seqlen_new=snew, dtype=dtype, seed=seed, b_cache=b_cache)
+    got, ref, gold, dev = run_dense(case, cache_batch_idx=idx, causal=causal, num_splits=num_splits)
+    if snew:
+        assert torch.equal(dev["k_cache"].cpu().view(torch.int16), ref[2].view(torch.int16)), "appended K bytes differ"
+        assert torch.equal(dev["v_cache"].cpu().view(torch.int16), ref[3].view(torch.int16)), "appended V bytes differ"
+    check_out(got[0], ref[0], got[1], ref[1], f"random dense {seed}")
