@@ -174,6 +174,33 @@ __device__ __forceinline__ int adaptive_split_keys(int max_keys, int nsplits) {
 }
 
 // 16-byte global load / store through plain vector types
+// Cut of the keys a query block of Sq rows over Sk keys can see (window already normalised) into ranges of
+// `split_keys` keys, counted from the 32-aligned first visible key; at most `nsplits` ranges, the last one
+// takes the rest.  A block that sees nothing has one (empty) range.  The kernel that writes the partial
+// results and the one that merges them derive the cut from this one function.
+struct KeyRanges {
+    int lo, hi;      // visible keys of the block: [lo, hi)
+    int count;       // ranges the block is cut into (>= 1)
+    int first;       // 32-aligned start of range 0
+    __device__ __forceinline__ int begin(int r, int split_keys) const { return max(lo, first + r * split_keys); }
+    __device__ __forceinline__ int end(int r, int split_keys) const {
+        return (r == count - 1) ? hi : min(hi, first + (r + 1) * split_keys);
+    }
+};
+__device__ __forceinline__ KeyRanges key_ranges(int Sq, int Sk, int wl, int wr, int split_keys, int nsplits) {
+    KeyRanges kr;
+    const int off = Sk - Sq;
+    kr.lo = 0;
+    kr.hi = Sk;
+    if (wr >= 0) kr.hi = min(Sk, Sq - 1 + off + wr + 1);
+    if (wl >= 0) kr.lo = max(0, off - wl);
+    const bool empty = Sk <= 0 || kr.hi <= kr.lo;
+    kr.first = kr.lo / 32 * 32;
+    kr.count = empty ? 1 : min(nsplits, (kr.hi - kr.first + split_keys - 1) / split_keys);
+    if (empty) kr.hi = kr.lo;
+    return kr;
+}
+
 __device__ __forceinline__ u32x4_t load16(const void *p) { return *reinterpret_cast<const u32x4_t *>(p); }
 // the same load marked non-temporal: data that is read once (the KV stream) need not stay in the caches
 __device__ __forceinline__ u32x4_t load16_stream(const void *p) {

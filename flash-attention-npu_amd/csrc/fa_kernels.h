@@ -99,6 +99,7 @@ struct PrefillParams {
     const int32_t *block_table;    // NULL: dense K/V
     int32_t batch, nheads, nheads_k, group;
     int32_t pack;                  // set by the launcher: 1, or group when tile rows are (query, head) pairs
+    int32_t pack_short;            // set by the launcher: pack == 1, but a short query block packs its heads on its own
     int32_t num_mb, units8;        // set by the launcher: 128-row blocks per unit, units rounded up to 8
     int32_t seqlen_q_fixed, seqlen_k_add;   // kvcache layout: Sq per row, keys appended this call
     int32_t max_seqlen_q, total_q;
@@ -112,9 +113,10 @@ struct PrefillParams {
     float scale_log2, softcap_pre, softcap_post;
     int32_t causal, window_left, window_right;
     int32_t window_norm_m;                  // key count the window is normalised with; 0 = each row's own
-    // split of the keys (kvcache layout only): blockIdx.z = batch row * nsplits + split, ranges of
-    // adaptive_split_keys() keys; a unit cut into several ranges leaves fp32 partials and base-2 LSEs
-    // in slot (batch row * nheads_k + kv head) * nsplits + split for the split-KV combine kernel
+    // split of the keys (paged K/V): ranges of adaptive_split_keys() keys; a query block cut into several
+    // ranges leaves fp32 partials and base-2 LSEs, in slot (batch row * nheads_k + kv head) * nsplits + split
+    // of `rows` rows each for the split-KV combine kernel (kvcache layout), or at
+    // (token * nheads + head) * nsplits + split for prefill_combine_kernel (token-major q)
     int32_t nsplits, rows;                  // rows = seqlen_q_fixed * group
     float *o_partial;
     float *lse_partial;
@@ -123,6 +125,8 @@ struct PrefillParams {
 // GQA group packed into the tile rows of the tiled forward for query blocks of max_seqlen_q rows
 // (1 = one q head per tile).
 int prefill_pack(int group, int max_seqlen_q);
+// 1 when the blocks of a token-major launch that does not pack (prefill_pack == 1) pack on their own where they are short.
+int prefill_pack_short(int group, int max_seqlen_q, int total_q, int batch);
 // Tiles (workgroups) of the tiled forward per batch row.
 int prefill_tiles(int nheads, int nheads_k, int max_seqlen_q);
 
@@ -135,6 +139,8 @@ hipError_t launch_decode_wave(const DecodeParams &p, int dtype, int headdim, hip
 hipError_t launch_splitkv_combine(const DecodeParams &p, int dtype, int headdim_v, hipStream_t stream);
 hipError_t launch_decode_mla_i8(const DecodeParams &p, int dtype, hipStream_t stream);
 hipError_t launch_prefill(const PrefillParams &p, int dtype, int headdim, hipStream_t stream);
+// merge of the key ranges of token-major query blocks (cu_seqlens_q set, nsplits > 1) after launch_prefill
+hipError_t launch_prefill_combine(const PrefillParams &p, int dtype, int headdim, hipStream_t stream);
 
 // Resident decode workgroups per compute unit for a head dimension / query-block height.
 int decode_wgs_per_cu(int headdim, int rows);

@@ -8,6 +8,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <climits>
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
@@ -591,6 +592,7 @@ int fa_rocm_varlen_validate(const fa_varlen_args *a) {
     if (a->headdim != 64 && a->headdim != 128 && a->headdim != 256) return fail(FA_ERR_SHAPE, "head dimension must be 64, 128 or 256");
     if (a->softcap < 0.f) return fail(FA_ERR_SHAPE, "softcap must be non-negative (0.0 disables softcap)");
     if (a->max_seqlen_q <= 0) return fail(FA_ERR_SHAPE, "max_seqlen_q must be positive");
+    if (a->num_splits < 0) return fail(FA_ERR_SHAPE, "num_splits must be non-negative");
     if (a->block_table && (a->page_size <= 0 || a->page_size % 32 != 0))
         return fail(FA_ERR_SHAPE, "page_block_size must be a positive multiple of 32");
     if (a->block_table && (a->num_blocks <= 0 || a->max_blocks_per_seq <= 0))
@@ -601,9 +603,52 @@ int fa_rocm_varlen_validate(const fa_varlen_args *a) {
     return FA_OK;
 }
 
+int fa_rocm_varlen_num_splits(const fa_varlen_args *a, int num_cus) {
+    if (fa_rocm_varlen_validate(a) != FA_OK) return 1;
+    if (!a->block_table || a->num_splits == 1 || a->total_q <= 0) return 1;
+    if (num_cus <= 0) num_cus = 256;
+    const int group = a->nheads / a->nheads_k;
+    const bool pack_short = fa::prefill_pack_short(group, a->max_seqlen_q, a->total_q, a->batch) != 0;
+    const int pack = pack_short ? group : fa::prefill_pack(group, a->max_seqlen_q);
+    // the lengths of the query blocks stay on the device: sum_b ceil(rows_b / 128) <= rows / 128 + batch
+    const int64_t blocks = ((int64_t)a->total_q * pack + 127) / 128 + a->batch;
+    const int64_t tiles = blocks * (pack > 1 ? a->nheads_k : a->nheads);
+    int64_t n = 1;
+    if (a->num_splits > 1) {
+        n = a->num_splits;
+    } else {
+        const int64_t slots = (int64_t)num_cus * (a->headdim <= 128 ? 2 : 1);
+        // query blocks far shorter than the longest one on average (a prompt chunk among decode rows): the
+        // longest block is the critical path long before the tiles fill the device, so it is cut earlier
+        const bool uneven = (int64_t)a->total_q * 4 <= (int64_t)a->batch * a->max_seqlen_q;
+        if (uneven) {
+            if (tiles < 2 * slots) n = (2 * slots + tiles - 1) / tiles;
+        } else if (tiles * 2 <= slots) {
+            n = (slots + tiles - 1) / tiles;
+        }
+    }
+    const int64_t bound = std::min<int64_t>(a->max_seqlen_k > 0 ? a->max_seqlen_k : INT32_MAX,
+                                            (int64_t)a->max_blocks_per_seq * a->page_size);
+    const int64_t most = (bound + 255) / 256;   // at least 256 keys (four tiles) per range
+    n = std::min<int64_t>(std::min<int64_t>(n, most), 64);
+    return (int)std::max<int64_t>(n, 1);
+}
+
+size_t fa_rocm_varlen_workspace_bytes(const fa_varlen_args *a, int num_cus) {
+    const int n = fa_rocm_varlen_num_splits(a, num_cus);
+    if (n <= 1) return 0;
+    return (size_t)a->total_q * a->nheads * n * ((size_t)a->headdim + 1) * sizeof(float);
+}
+
 int fa_rocm_varlen_fwd(const fa_varlen_args *a, void *stream_) {
     const int rc = fa_rocm_varlen_validate(a);
     if (rc != FA_OK) return rc;
+    int cus = device_cus();
+    if (cus <= 0) cus = 256;
+    const int nsplits = fa_rocm_varlen_num_splits(a, cus);
+    const size_t ws_bytes = fa_rocm_varlen_workspace_bytes(a, cus);
+    if (ws_bytes > 0 && (!a->workspace || a->workspace_bytes < ws_bytes))
+        return fail(FA_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", ws_bytes, a->workspace ? a->workspace_bytes : (size_t)0);
     fa::PrefillParams pp;
     std::memset(&pp, 0, sizeof(pp));
     pp.q = a->q;
@@ -647,8 +692,15 @@ int fa_rocm_varlen_fwd(const fa_varlen_args *a, void *stream_) {
     pp.window_left = a->window_left;
     pp.window_right = a->window_right;
     pp.window_norm_m = a->max_seqlen_k;
+    if (nsplits > 1) {
+        pp.nsplits = nsplits;
+        pp.o_partial = static_cast<float *>(a->workspace);
+        pp.lse_partial = pp.o_partial + (size_t)a->total_q * a->nheads * nsplits * a->headdim;
+    }
     const hipError_t e = fa::launch_prefill(pp, a->io_dtype, a->headdim, static_cast<hipStream_t>(stream_));
     if (e != hipSuccess) return fail(FA_ERR_LAUNCH, "prefill launch failed: %s", hipGetErrorString(e));
+    const hipError_t ec = fa::launch_prefill_combine(pp, a->io_dtype, a->headdim, static_cast<hipStream_t>(stream_));
+    if (ec != hipSuccess) return fail(FA_ERR_LAUNCH, "combine launch failed: %s", hipGetErrorString(ec));
     return FA_OK;
 }
 

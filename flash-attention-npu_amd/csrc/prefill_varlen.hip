@@ -59,8 +59,7 @@ __global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) prefill_kernel(const 
     // mix of tall and short causal blocks whatever the number of blocks is, and the heads that share
     // a unit's K/V meet in one L2.
     const int nsplits = EXT ? max(p.nsplits, 1) : 1;
-    const int pg = EXT ? p.pack : 1;               // tile row R is query R / pg of head h_base + R % pg
-    const int heads_per_unit = (pg > 1) ? 1 : p.group;
+    const int heads_per_unit = (EXT && p.pack > 1) ? 1 : p.group;
     int mb, unit, head_in_unit;
     if (p.num_mb > 2) {
         const int per_block = p.units8 * heads_per_unit;
@@ -82,7 +81,6 @@ __global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) prefill_kernel(const 
     const int hk = unit - z * p.nheads_k;
     const int b = z / nsplits;
     const int split = z - b * nsplits;
-    const int h_base = hk * p.group + ((pg > 1) ? 0 : head_in_unit);
 
     int q0, Sq, k0 = 0, Sk;
     if (p.cu_seqlens_q) {
@@ -92,6 +90,20 @@ __global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) prefill_kernel(const 
         q0 = 0;
         Sq = p.seqlen_q_fixed;
     }
+    // tile row R is query R / pg of head h_base + R % pg.  pg is the launch's (every block packs the heads
+    // of its group, or none does) unless the launch lets short blocks pack on their own: a block whose
+    // (query, head) rows take at most three quarters of the tiles its heads would take one by one is
+    // computed by the tiles of its first head alone, the tiles of the other heads leave
+    int pg = EXT ? p.pack : 1;
+    if (EXT && p.pack_short && pg == 1 && p.group > 1) {
+        const int packed = (Sq * p.group + kBM - 1) / kBM;
+        const int plain = p.group * ((Sq + kBM - 1) / kBM);
+        if (packed * 4 <= plain * 3 && packed <= p.num_mb) {
+            if (head_in_unit != 0) return;
+            pg = p.group;
+        }
+    }
+    const int h_base = hk * p.group + ((pg > 1) ? 0 : head_in_unit);
     if constexpr (PAGED) {
         Sk = p.seqused_k[b] + p.seqlen_k_add;
         Sk = min(Sk, p.max_blocks * p.page_size);
@@ -124,19 +136,14 @@ __global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) prefill_kernel(const 
     bool whole = true;
     int64_t slot = 0;
     if (nsplits > 1) {
-        int u_lo = 0, u_hi = Sk;
-        if (wr_eff >= 0) u_hi = min(Sk, Sq - 1 + off + wr_eff + 1);
-        if (wl >= 0) u_lo = max(0, off - wl);
-        const bool empty = Sk <= 0 || u_hi <= u_lo;
-        const int lo_al = u_lo / 32 * 32;
         const int sk = adaptive_split_keys(batch_max, nsplits);
-        const int ns_row = empty ? 1 : min(nsplits, (u_hi - lo_al + sk - 1) / sk);
-        if (split >= ns_row) return;
-        if (!empty) {
-            range_lo = max(u_lo, lo_al + split * sk);
-            range_hi = (split == ns_row - 1) ? u_hi : min(u_hi, lo_al + (split + 1) * sk);
+        const KeyRanges kr = key_ranges(Sq, Sk, wl, wr_eff, sk, nsplits);
+        if (split >= kr.count) return;
+        if (kr.hi > kr.lo) {
+            range_lo = kr.begin(split, sk);
+            range_hi = kr.end(split, sk);
         }
-        whole = ns_row == 1;
+        whole = kr.count == 1;
         slot = ((int64_t)b * p.nheads_k + hk) * nsplits + split;
     }
 
@@ -161,7 +168,9 @@ __global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) prefill_kernel(const 
     // where this lane's row goes when the unit is cut: row (query, head of the group) of the slot
     float *part_row = nullptr, *part_lse = nullptr;
     if (!whole) {
-        const int64_t prow = slot * p.rows + (int64_t)my_row * p.group + (my_head - hk * p.group);
+        // kvcache layout: (batch row, kv head, range, query x head of the group); token-major q: (token, head, range)
+        const int64_t prow = p.cu_seqlens_q ? ((int64_t)(q0 + my_row) * p.nheads + my_head) * nsplits + split
+                                            : slot * p.rows + (int64_t)my_row * p.group + (my_head - hk * p.group);
         part_row = p.o_partial + prow * D;
         part_lse = p.lse_partial + prow;
     }
@@ -495,11 +504,71 @@ __global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) prefill_kernel(const 
     }
 }
 
+// Merge of the key ranges of token-major query blocks over a paged cache: one wave per (token, head).
+// Partials are laid out (token, head, range): normalised fp32 rows and base-2 log-sum-exps, -inf for a
+// range in which the row saw nothing.  out = sum_r e^{lse_r - LSE} O_r, LSE = log sum_r e^{lse_r}.
+// grid: total_q * nheads workgroups of 64 threads.
+template <typename T, int D>
+__global__ void __launch_bounds__(64) prefill_combine_kernel(const PrefillParams p) {
+    const int tok = blockIdx.x / p.nheads;
+    const int head = blockIdx.x - tok * p.nheads;
+    const int lane = threadIdx.x;
+    // the sequence of this token: last b with cu_seqlens_q[b] <= tok (empty sequences repeat an offset)
+    int lo = 0, hi = p.batch;
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (p.cu_seqlens_q[mid] <= tok) lo = mid; else hi = mid;
+    }
+    const int b = lo;
+    const int Sq = p.cu_seqlens_q[b + 1] - p.cu_seqlens_q[b];
+    const int Sk = min(p.seqused_k[b] + p.seqlen_k_add, p.max_blocks * p.page_size);
+    const int longest = block_max_keys(p.seqused_k, p.batch, p.seqlen_k_add);
+    int wl = p.window_left, wr = p.window_right;
+    int norm_m = p.window_norm_m;
+    if (norm_m <= 0 && (wl >= 0 || wr >= 0)) norm_m = longest;
+    if (norm_m <= 0) norm_m = max(Sk, 1);
+    normalize_window(wl, wr, p.causal, norm_m);
+    const int sk = adaptive_split_keys(min(longest, p.max_blocks * p.page_size), p.nsplits);
+    const KeyRanges kr = key_ranges(Sq, Sk, wl, wr, sk, p.nsplits);
+    if (kr.count == 1) return;   // the tile that computed this row wrote it
+    const int64_t base = ((int64_t)tok * p.nheads + head) * p.nsplits;
+
+    float mx = -INFINITY;
+    for (int r = lane; r < kr.count; r += 64) mx = fmaxf(mx, p.lse_partial[base + r]);
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) mx = fmaxf(mx, __shfl_xor(mx, d, 64));
+    const float mx_use = (mx == -INFINITY) ? 0.f : mx;
+    constexpr int C = D / 64;        // columns per lane
+    float acc[C];
+#pragma unroll
+    for (int c = 0; c < C; ++c) acc[c] = 0.f;
+    float tot = 0.f;
+    for (int r = 0; r < kr.count; ++r) {
+        const float w = fast_exp2(p.lse_partial[base + r] - mx_use);
+        tot += w;
+        const float *o = p.o_partial + (base + r) * D + lane * C;
+#pragma unroll
+        for (int c = 0; c < C; ++c) acc[c] += w * o[c];
+    }
+    const float inv = (tot > 0.f) ? 1.f / tot : 0.f;
+    uint16_t *dst = reinterpret_cast<uint16_t *>(p.out) + (int64_t)tok * p.o_stride_t + (int64_t)head * p.o_stride_h + lane * C;
+#pragma unroll
+    for (int c = 0; c < C; ++c) dst[c] = from_float<T>(acc[c] * inv);
+    if (lane == 0) p.lse[(int64_t)head * p.lse_stride_h + tok] = (tot > 0.f) ? (mx + fast_log2(tot)) * kLn2 : INFINITY;
+}
+
 // pack the heads of a GQA group into the tile rows when that saves at least a quarter of the tiles
 int prefill_pack(int group, int max_seqlen_q) {
     const int tiles_plain = group * ((max_seqlen_q + kBM - 1) / kBM);
     const int tiles_packed = (max_seqlen_q * group + kBM - 1) / kBM;
     return (group > 1 && tiles_packed * 4 <= tiles_plain * 3) ? group : 1;
+}
+
+// token-major q whose blocks differ in length and whose average block would pack: every block decides
+// for itself (mixed prefill / decode batches)
+int prefill_pack_short(int group, int max_seqlen_q, int total_q, int batch) {
+    if (group <= 1 || batch <= 0 || total_q <= 0 || prefill_pack(group, max_seqlen_q) > 1) return 0;
+    return prefill_pack(group, (total_q + batch - 1) / batch) > 1 ? 1 : 0;
 }
 
 int prefill_tiles(int nheads, int nheads_k, int max_seqlen_q) {
@@ -511,7 +580,7 @@ template <typename T, int D> static hipError_t launch_prefill_d(const PrefillPar
     PrefillParams p = p_in;
     p.pack = prefill_pack(p.group, p.max_seqlen_q);
     p.num_mb = (p.max_seqlen_q * p.pack + kBM - 1) / kBM;
-    if (p.nsplits > 1 && (!p.block_table || p.cu_seqlens_q || !p.o_partial)) return hipErrorInvalidValue;
+    if (p.nsplits > 1 && (!p.block_table || !p.o_partial || !p.lse_partial)) return hipErrorInvalidValue;
     const int64_t units = (int64_t)p.batch * max(p.nsplits, 1) * p.nheads_k;
     p.units8 = (int32_t)((units + 7) / 8 * 8);
     const int64_t wgs = (int64_t)p.num_mb * p.units8 * (p.pack > 1 ? 1 : p.group);
@@ -520,7 +589,8 @@ template <typename T, int D> static hipError_t launch_prefill_d(const PrefillPar
     dim3 block(256);
     const bool softcap = p.softcap_post != 0.f;
     const bool paged = p.block_table != nullptr;
-    const bool ext = p.pack > 1 || p.nsplits > 1;
+    p.pack_short = p.cu_seqlens_q ? prefill_pack_short(p.group, p.max_seqlen_q, p.total_q, p.batch) : 0;
+    const bool ext = p.pack > 1 || p.nsplits > 1 || p.pack_short;
     auto launch = [&](auto paged_c, auto softcap_c, auto ext_c) {
         hipLaunchKernelGGL((prefill_kernel<T, D, decltype(paged_c)::value, decltype(softcap_c)::value, decltype(ext_c)::value>),
                            grid, block, 0, stream, p);
@@ -542,6 +612,25 @@ template <typename T> static hipError_t launch_prefill_t(const PrefillParams &p,
         case 256: return launch_prefill_d<T, 256>(p, stream);
         default: return hipErrorInvalidValue;
     }
+}
+
+template <typename T> static hipError_t launch_prefill_combine_t(const PrefillParams &p, int headdim, hipStream_t stream) {
+    const int64_t wgs = (int64_t)p.total_q * p.nheads;
+    if (wgs <= 0 || wgs >= (1ll << 31)) return hipErrorInvalidValue;
+    dim3 grid((unsigned)wgs), block(64);
+    switch (headdim) {
+        case 64: hipLaunchKernelGGL((prefill_combine_kernel<T, 64>), grid, block, 0, stream, p); break;
+        case 128: hipLaunchKernelGGL((prefill_combine_kernel<T, 128>), grid, block, 0, stream, p); break;
+        case 256: hipLaunchKernelGGL((prefill_combine_kernel<T, 256>), grid, block, 0, stream, p); break;
+        default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_prefill_combine(const PrefillParams &p, int dtype, int headdim, hipStream_t stream) {
+    if (p.nsplits <= 1 || p.total_q <= 0) return hipSuccess;
+    if (!p.cu_seqlens_q || !p.block_table || !p.o_partial || !p.lse_partial) return hipErrorInvalidValue;
+    return dtype == 0 ? launch_prefill_combine_t<BF16>(p, headdim, stream) : launch_prefill_combine_t<FP16>(p, headdim, stream);
 }
 
 hipError_t launch_prefill(const PrefillParams &p, int dtype, int headdim, hipStream_t stream) {

@@ -44,7 +44,7 @@ class VarlenArgs(C.Structure):
         + [(n, _i64) for n in ("q_stride_t", "q_stride_h", "k_stride_t", "k_stride_h", "v_stride_t", "v_stride_h",
                                "k_stride_block", "v_stride_block", "o_stride_t", "o_stride_h", "bt_stride_b")]
         + [("io_dtype", _i32), ("softmax_scale", _f32), ("softcap", _f32), ("causal", _i32), ("window_left", _i32),
-           ("window_right", _i32)]
+           ("window_right", _i32), ("num_splits", _i32), ("workspace", _vp), ("workspace_bytes", _sz)]
     )
 
 
@@ -68,6 +68,8 @@ EXPORTS = {
     "fa_rocm_fwd_kvcache": (C.c_int, [C.POINTER(KvcacheArgs), _vp]),
     "fa_rocm_fwd_kvcache_profiled": (C.c_int, [C.POINTER(KvcacheArgs), _vp, C.POINTER(_vp)]),
     "fa_rocm_varlen_fwd": (C.c_int, [C.POINTER(VarlenArgs), _vp]),
+    "fa_rocm_varlen_num_splits": (C.c_int, [C.POINTER(VarlenArgs), C.c_int]),
+    "fa_rocm_varlen_workspace_bytes": (_sz, [C.POINTER(VarlenArgs), C.c_int]),
     "fa_rocm_append_kv": (C.c_int, [C.POINTER(KvcacheArgs), _vp]),
 }
 

@@ -273,8 +273,10 @@ def bind_kvcache(q, kcache, vcache, k_, v_, seqlens_k_, rotary_cos_, rotary_sin_
 
 def varlen_fwd(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k_, leftpad_k_, block_table_, alibi_slopes_,
                max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale, zero_tensors, is_causal, window_size_left,
-               window_size_right, softcap, return_softmax, gen_) -> List[torch.Tensor]:
-    """mha_varlen_fwd (flash_api.cpp:848-1089).  Returns [out, softmax_lse (Hq, total_q), p, rng_state]."""
+               window_size_right, softcap, return_softmax, gen_, *, num_splits: int = 0) -> List[torch.Tensor]:
+    """mha_varlen_fwd (flash_api.cpp:848-1089).  Returns [out, softmax_lse (Hq, total_q), p, rng_state].
+    num_splits (paged K/V only; not an argument of the reference's function): 0 cuts every sequence's keys into
+    as many ranges as it takes to fill the device when the query tiles alone cannot, 1 never, n at most n."""
     lib = _lib.load()
     _require(q.dtype in (torch.bfloat16, torch.float16), "FlashAttention only supports FP16 and BF16 data types")
     _require(k.dtype == q.dtype, "query and key must have the same dtype")
@@ -333,8 +335,14 @@ def varlen_fwd(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k_, leftpad_k_
     a.softmax_scale, a.softcap = float(softmax_scale), float(softcap)
     a.causal = int(bool(is_causal))
     a.window_left, a.window_right = int(window_size_left), int(window_size_right)
+    _require(num_splits >= 0, "num_splits must be non-negative")
+    a.num_splits = int(num_splits)
     if total_q > 0:
         with torch.cuda.device(q.device):
+            need = lib.fa_rocm_varlen_workspace_bytes(C.byref(a), lib.fa_rocm_num_cus())
+            if need:
+                ws = torch.empty(((need + 3) // 4,), dtype=torch.float32, device=q.device)
+                a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel() * 4
             _lib.check(lib.fa_rocm_varlen_fwd(C.byref(a), _stream(q)))
     p = torch.empty((0,), dtype=q.dtype, device=q.device)
     rng_state = torch.empty((2,), dtype=torch.int64, device=q.device)

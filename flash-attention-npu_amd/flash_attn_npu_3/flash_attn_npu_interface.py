@@ -411,7 +411,7 @@ def flash_attn_with_kvcache(
             _require(k_cache.shape[1] % 32 == 0 or table.shape[1] == 1, "page_block_size must be a positive multiple of 32")
             out, lse, _, _ = _op.varlen_fwd(q, k_cache, v_cache, None, cu_seqlens_q, None, cache_seqlens, None, table, None,
                                             int(max_seqlen_q), 0, 0.0, common[0], False, common[1], wl, wr, common[4],
-                                            False, None)
+                                            False, None, num_splits=common[6])
         else:
             _require(k_cache.dim() == 3 and not paged, "a packed cache must be (total_k, nheads_k, headdim) without page_table")
             _require(cache_batch_idx is None, "cache_batch_idx needs a dense (batch_cache, seqlen_cache, ...) cache")

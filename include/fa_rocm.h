@@ -123,6 +123,15 @@ typedef struct fa_varlen_args {
     float softcap;
     int32_t causal;
     int32_t window_left, window_right;
+    /* Paged K/V only: cut of every sequence's keys into ranges when the query tiles alone cannot fill the
+     * device (few sequences, short query blocks, long contexts: chunked prefill, mixed prefill / decode
+     * batches).  0 = as many ranges as it takes, 1 = never, n = at most n.  The ranges leave fp32
+     * partials in `workspace` (fa_rocm_varlen_workspace_bytes), merged by a second kernel.  The
+     * reference's third-generation surface takes num_splits for token-major q the same way
+     * (flash_attn_npu_3/flash_attn_npu_interface.py:965-996). */
+    int32_t num_splits;
+    void *workspace;
+    size_t workspace_bytes;
 } fa_varlen_args;
 
 /* Library / device facts. */
@@ -196,6 +205,12 @@ int fa_rocm_fwd_kvcache_profiled(const fa_kvcache_args *args, void *stream, void
  * (csrc/ascend910/flash_attn_npu/flash_api.cpp:848-1089).
  */
 int fa_rocm_varlen_fwd(const fa_varlen_args *args, void *stream);
+
+/* Ranges the varlen call cuts every sequence's keys into (1 = no cut), from shapes alone, and the bytes
+ * of workspace it then needs (0 when nothing is cut).  Pure host integer code: needs no GPU.
+ * `num_cus` <= 0 means 256. */
+int fa_rocm_varlen_num_splits(const fa_varlen_args *args, int num_cus);
+size_t fa_rocm_varlen_workspace_bytes(const fa_varlen_args *args, int num_cus);
 
 /*
  * The in-place append on its own (k_new/v_new -> pages, rotary on k_new).  The reference

@@ -276,3 +276,33 @@ def test_varlen_empty_sequences():
     cu0 = torch.zeros(3, dtype=torch.int32, device="cuda")
     out = flash_attn_varlen_func(total0, c["k"].cuda(), c["v"].cuda(), cu0, c["cu_k"].cuda()[:3], 1, 70)
     assert out.shape == (0, 8, 128)
+
+
+def paged_ragged(lens_q, lens_k, hq, hk, d, page, seed, dtype=torch.bfloat16):
+    case = make_paged_case(len(lens_k), hq, hk, d, page, lens_k, dtype=dtype, seed=seed)
+    g = torch.Generator().manual_seed(seed + 1)
+    q = torch.randn(sum(lens_q), hq, d, generator=g).to(dtype)
+    cu_q = torch.tensor([0] + torch.tensor(lens_q).cumsum(0).tolist(), dtype=torch.int32)
+    cu_k = torch.tensor([0] + torch.tensor(lens_k).cumsum(0).tolist(), dtype=torch.int32)
+    kl = torch.cat([O.gather_paged(case["k_cache"], case["block_table"][b], lens_k[b]) for b in range(len(lens_k))])
+    vl = torch.cat([O.gather_paged(case["v_cache"], case["block_table"][b], lens_k[b]) for b in range(len(lens_k))])
+    return case, q, cu_q, cu_k, kl, vl
+
+
+@pytest.mark.parametrize("num_splits", [0, 1, 3, 64])
+@pytest.mark.parametrize("hq,hk,d", [(8, 2, 128), (4, 4, 64), (6, 1, 256)])
+@pytest.mark.parametrize("causal,window", [(True, (-1, -1)), (False, (-1, -1)), (True, (900, 0)), (False, (2000, 100))])
+def test_varlen_paged_ragged_blocks_split_keys(hq, hk, d, causal, window, num_splits):
+    # a mixed batch over a paged cache: single-token rows, a chunk of a long prompt, an empty query block, a
+    # sequence shorter than one range; every sequence's keys are cut into ranges and merged per token
+    from flash_attn_npu.flash_attn_npu import varlen_fwd
+    lens_q = [1, 300, 1, 0, 17, 40]
+    lens_k = [5000, 3100, 40, 700, 2100, 0]
+    case, q, cu_q, cu_k, kl, vl = paged_ragged(lens_q, lens_k, hq, hk, d, 64, seed=31)
+    print("ragged split", hq, hk, d, causal, window, num_splits, flush=True)
+    out, lse, _, _ = varlen_fwd(q.cuda(), case["k_cache"].cuda(), case["v_cache"].cuda(), None, cu_q.cuda(), None,
+                                case["cache_seqlens"].cuda(), None, case["block_table"].cuda(), None, max(lens_q), max(lens_k),
+                                0.0, d ** -0.5, False, causal, window[0], window[1], 0.0, False, None, num_splits=num_splits)
+    torch.cuda.synchronize()
+    ref, ref_lse = O.flash_attn_varlen(q, kl, vl, cu_q, cu_k, max(lens_q), max(lens_k), causal=causal, window_size=window, mode="fp32")
+    check_out(out, ref, lse, ref_lse, "ragged split")

@@ -107,6 +107,27 @@ def test_v3_kvcache_tnd_paged(case, num_splits):
     check_vs_golden(out, gold.reshape(B * sq, hq, d), lse, gold_lse.permute(1, 0, 2).reshape(hq, B * sq), str(case))
 
 
+@pytest.mark.parametrize("num_splits", [0, 1, 4])
+def test_v3_kvcache_tnd_mixed_batch_long_contexts(num_splits):
+    # decode rows and a prompt chunk in one token-major batch over long paged contexts: the keys of every
+    # sequence are cut into ranges (num_splits 0 / 4) or not (1); same result either way
+    from flash_attn_npu_3 import flash_attn_with_kvcache
+    q_lens, k_lens = [1, 1, 200, 1], [6000, 129, 4500, 3000]
+    B, hq, hk, d = 4, 16, 2, 128
+    c = make_paged_case(B, hq, hk, d, 256, k_lens, seqlen_q=1, seed=93)
+    g = torch.Generator().manual_seed(94)
+    q = torch.randn(sum(q_lens), hq, d, generator=g).to(BF)
+    k_packed, v_packed = packed_from_pages(c, k_lens)
+    cu_q, cu_k = cu(q_lens), cu(k_lens)
+    print("v3 mixed batch", num_splits, flush=True)
+    out, lse, *_ = flash_attn_with_kvcache(q.cuda(), c["k_cache"].cuda(), c["v_cache"].cuda(), page_table=c["block_table"].cuda(),
+                                           cache_seqlens=c["cache_seqlens"].cuda(), cu_seqlens_q=cu_q.cuda(), max_seqlen_q=max(q_lens),
+                                           causal=True, num_splits=num_splits, return_softmax_lse=True)
+    torch.cuda.synchronize()
+    ref, ref_lse = O.flash_attn_varlen(q, k_packed, v_packed, cu_q, cu_k, max(q_lens), max(k_lens), causal=True, mode="fp32")
+    check_out(out, ref, lse, ref_lse, "v3 mixed batch")
+
+
 @pytest.mark.parametrize("layout", ["paged", "packed", "dense"])
 @pytest.mark.parametrize("causal,window", [(False, (-1, -1)), (True, (-1, -1)), (False, (300, 40))])
 def test_v3_kvcache_tnd_ragged(layout, causal, window):

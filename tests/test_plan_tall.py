@@ -43,3 +43,38 @@ def test_tall_plan():
     q_bytes = 1 * 24 * 16 * 128 * 2
     p = plan_of(1, 24, 16, 2, 128, 32, rotary=True)
     assert p.nsplits == 32 and p.workspace_bytes == q_bytes + 1 * 2 * 32 * (24 * 8) * 129 * 4
+
+
+def test_varlen_split_plan():
+    # the planner: paged only, never with num_splits = 1, at least 256 keys per range, at most 64 ranges
+    import ctypes as C
+    from flash_attn_npu import _lib
+    lib = _lib.load()
+    a = _lib.VarlenArgs()
+    fake = 0x1000        # the planner and the checks never follow a pointer
+    for f in ("q", "k", "v", "out", "softmax_lse", "cu_seqlens_q", "seqused_k", "block_table"):
+        setattr(a, f, fake)
+    a.batch, a.total_q, a.nheads, a.nheads_k, a.headdim = 2, 300, 8, 2, 128
+    a.max_seqlen_q, a.max_seqlen_k, a.page_size, a.max_blocks_per_seq, a.num_blocks = 299, 100000, 64, 2000, 4000
+    a.q_stride_t = a.o_stride_t = 1024
+    a.q_stride_h = a.o_stride_h = a.k_stride_h = a.v_stride_h = 128
+    a.k_stride_t = a.v_stride_t = 256
+    a.io_dtype = 0
+    n = lib.fa_rocm_varlen_num_splits(C.byref(a), 256)
+    assert 1 < n <= 64
+    assert lib.fa_rocm_varlen_workspace_bytes(C.byref(a), 256) == 300 * 8 * n * 129 * 4
+    a.num_splits = 1
+    assert lib.fa_rocm_varlen_num_splits(C.byref(a), 256) == 1 and lib.fa_rocm_varlen_workspace_bytes(C.byref(a), 256) == 0
+    a.num_splits = 500
+    assert lib.fa_rocm_varlen_num_splits(C.byref(a), 256) == 64
+    a.num_splits, a.max_seqlen_k = 0, 700
+    assert lib.fa_rocm_varlen_num_splits(C.byref(a), 256) == 3
+    a.max_seqlen_k, a.total_q, a.max_seqlen_q = 100000, 40000, 20000          # the tiles fill the device: no cut
+    assert lib.fa_rocm_varlen_num_splits(C.byref(a), 256) == 1
+    a.total_q, a.block_table = 300, None
+    a.cu_seqlens_k = fake
+    assert lib.fa_rocm_varlen_num_splits(C.byref(a), 256) == 1
+    # a workspace that is too small is refused before anything is launched
+    a.block_table, a.num_splits = fake, 4
+    a.workspace, a.workspace_bytes = fake, 16
+    assert lib.fa_rocm_varlen_fwd(C.byref(a), None) == -5 and b"workspace" in lib.fa_rocm_last_error()
