@@ -277,6 +277,7 @@ __global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) prefill_kernel(const 
 
     const int kt_begin = k_lo / kBN;
     const int kt_end = (k_hi + kBN - 1) / kBN;
+    const bool wave_live = __builtin_amdgcn_readfirstlane(R0 + wave * 32 < n_rows);
     fetch_tile(kt_begin);
     stash_tile(0);
     __syncthreads();
@@ -287,6 +288,9 @@ __global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) prefill_kernel(const 
         if (more) fetch_tile(kt + 1);
         __builtin_amdgcn_sched_barrier(0);
 
+        // a wave whose 32 rows all lie past the block's end (short blocks: a decode row among prompt chunks
+        // fills four rows of one wave) only helps to move the tiles, and leaves the matrix pipe to the others
+        if (wave_live) {
         // ---- S^T = K Q^T for the two 32-key halves of the tile
         float16_t s[2];
 #pragma unroll
@@ -443,6 +447,7 @@ __global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) prefill_kernel(const 
 #pragma unroll
                 for (int t = 0; t < Cfg::kMT; ++t) o_acc[t] = mfma32<T>(va[t], pk[tt][ks], o_acc[t]);
             }
+        }   // wave_live
 
         if (more) stash_tile(cur ^ 1);
         __syncthreads();
