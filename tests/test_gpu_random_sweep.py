@@ -164,3 +164,47 @@ def test_random_dense(seed):
         assert torch.equal(dev["k_cache"].cpu().view(torch.int16), ref[2].view(torch.int16)), "appended K bytes differ"
         assert torch.equal(dev["v_cache"].cpu().view(torch.int16), ref[3].view(torch.int16)), "appended V bytes differ"
     check_out(got[0], ref[0], got[1], ref[1], f"random dense {seed}")
+
+
+def draw_ragged_paged(seed):
+    r = random.Random(11000 + seed)
+    B = r.randint(1, 12)
+    d = r.choice([64, 128, 128, 256])
+    hk = r.choice([1, 2, 4, 8])
+    hq = hk * r.choice([1, 2, 4, 8])
+    page = r.choice([32, 64, 256])
+    while True:
+        lens_k = [r.choice([0, 1, 40, r.randint(1, 600), r.randint(600, 3000), r.randint(3000, 9000)]) for _ in range(B)]
+        lens_q = [r.choice([0, 1, 1, 1, 2, 17, r.randint(1, 150), r.randint(150, 600)]) for _ in range(B)]
+        if sum(lens_q) > 0 and hq * d * sum(q * (k + 1) for q, k in zip(lens_q, lens_k)) <= 3e9:
+            break
+    causal = r.random() < 0.7
+    window = r.choice([(-1, -1), (-1, -1), (-1, -1), (r.randint(0, 2000), 0), (r.randint(0, 2000), r.randint(0, 100)), (-1, r.randint(0, 64))])
+    return dict(B=B, d=d, hk=hk, hq=hq, page=page, lens_k=lens_k, lens_q=lens_q, causal=causal, window=window,
+                softcap=r.choice([0.0, 0.0, 25.0]), num_splits=r.choice([0, 0, 0, 1, 2, 7, 64]),
+                dtype=r.choice([torch.bfloat16, torch.float16]))
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_random_ragged_blocks_over_pages(seed):
+    # token-major query blocks of any length (empty ones, single decode rows, prompt chunks) over a paged cache:
+    # packed heads per block, key ranges, the per-token merge
+    from flash_attn_npu.flash_attn_npu import varlen_fwd
+    c = draw_ragged_paged(seed)
+    print("random ragged paged", seed, c, flush=True)
+    B, d = c["B"], c["d"]
+    case = make_paged_case(B, c["hq"], c["hk"], d, c["page"], c["lens_k"], dtype=c["dtype"], seed=seed, extra_table_cols=seed % 2)
+    g = torch.Generator().manual_seed(seed + 1)
+    q = torch.randn(sum(c["lens_q"]), c["hq"], d, generator=g).to(c["dtype"])
+    cu_q = torch.tensor([0] + torch.tensor(c["lens_q"]).cumsum(0).tolist(), dtype=torch.int32)
+    cu_k = torch.tensor([0] + torch.tensor(c["lens_k"]).cumsum(0).tolist(), dtype=torch.int32)
+    kl = torch.cat([O.gather_paged(case["k_cache"], case["block_table"][b], c["lens_k"][b]) for b in range(B)])
+    vl = torch.cat([O.gather_paged(case["v_cache"], case["block_table"][b], c["lens_k"][b]) for b in range(B)])
+    max_q, max_k = max(c["lens_q"]), max(max(c["lens_k"]), 1)
+    out, lse, _, _ = varlen_fwd(q.cuda(), case["k_cache"].cuda(), case["v_cache"].cuda(), None, cu_q.cuda(), None,
+                                case["cache_seqlens"].cuda(), None, case["block_table"].cuda(), None, max_q, max_k, 0.0, d ** -0.5,
+                                False, c["causal"], c["window"][0], c["window"][1], c["softcap"], False, None, num_splits=c["num_splits"])
+    torch.cuda.synchronize()
+    ref, ref_lse = O.flash_attn_varlen(q, kl, vl, cu_q, cu_k, max_q, max_k, causal=c["causal"], window_size=c["window"],
+                                       softcap=c["softcap"], mode="fp32")
+    check_out(out, ref, lse, ref_lse, f"random ragged paged {seed}")
