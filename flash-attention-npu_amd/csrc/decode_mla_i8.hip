@@ -59,6 +59,7 @@ struct MlaShared {
     __attribute__((aligned(16))) uint8_t k[3][kMlaTileBytes];   // widened key tiles: scores, output, being filled
     __attribute__((aligned(16))) float ks[3][kChunk];            // per-token scales, K side
     __attribute__((aligned(16))) float vs[3][kChunk];            // per-token scales, V side
+    __attribute__((aligned(16))) float vsi[3][kChunk];           // their inverses (0 for a zero scale)
     __attribute__((aligned(16))) u32x4_t pk[2][4][64];           // P^T operands of the four head groups, two chunks
     float alpha[2][4][16];                                       // accumulator rescale per head
     __attribute__((aligned(4))) uint8_t bump[2][4];              // head group saw a new maximum
@@ -155,6 +156,7 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
             if (th < kChunk) {
                 sh.ks[tile][th] = st_ks[set];
                 sh.vs[tile][th] = st_vs[set];
+                sh.vsi[tile][th] = (st_vs[set] > 0.f) ? 1.f / st_vs[set] : 0.f;
             }
         };
         int blk_next;
@@ -164,7 +166,7 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
             fetch(0, b0, 0, tid);
             fetch(1, b1, 1, tid);
         }
-        float m_run = -INFINITY, l_run = 0.f;
+        float m_run = -INFINITY, l_run = 0.f, l_norm = 0.f;
 
         auto score_step = [&](const int j, const int set, const int tile_j) {
             int th = tid;
@@ -177,11 +179,12 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
             const int tile = (tile_j == 0) ? 2 : tile_j - 1;   // (j + 2) % 3: tile of the scores
             float4_t s[2] = {float4_t{0.f, 0.f, 0.f, 0.f}, float4_t{0.f, 0.f, 0.f, 0.f}};
             // per-token scales of the score chunk, read ahead of the products
-            float4 ks4[2], vs4[2];
+            float4 ks4[2], vs4[2], vi4[2];
 #pragma unroll
             for (int tt = 0; tt < 2; ++tt) {
                 ks4[tt] = *reinterpret_cast<const float4 *>(&sh.ks[tile][tt * 16 + lq * 4]);
                 vs4[tt] = *reinterpret_cast<const float4 *>(&sh.vs[tile][tt * 16 + lq * 4]);
+                vi4[tt] = *reinterpret_cast<const float4 *>(&sh.vsi[tile][tt * 16 + lq * 4]);
             }
             if (do_score) {
                 // ---- S^T = K Q^T : two 16-key tiles x this wave's 16 heads; operand reads run kPf
@@ -223,12 +226,13 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
                 const int pb = set ^ 1;                              // (j - 1) & 1
                 // ---- softmax; register i of tile tt is key c*32 + tt*16 + lq*4 + i
                 const int key_base = c * kChunk + lq * 4;
-                float x[8], vsc[8];
+                float x[8], vsc[8], vin[8];
                 float mloc = -INFINITY;
 #pragma unroll
                 for (int tt = 0; tt < 2; ++tt) {
                     const float ksv[4] = {ks4[tt].x, ks4[tt].y, ks4[tt].z, ks4[tt].w};
                     const float vsv[4] = {vs4[tt].x, vs4[tt].y, vs4[tt].z, vs4[tt].w};
+                    const float viv[4] = {vi4[tt].x, vi4[tt].y, vi4[tt].z, vi4[tt].w};
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
                         const int key = key_base + tt * 16 + i;
@@ -242,6 +246,7 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
                         v = (key >= mask_lo && key < mask_hi) ? v : -INFINITY;
                         x[tt * 4 + i] = v;
                         vsc[tt * 4 + i] = vsv[i];
+                        vin[tt * 4 + i] = viv[i];
                         mloc = fmaxf(mloc, v);
                     }
                 }
@@ -264,6 +269,18 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
                 pk[1] = pack2<T>(x[2], x[3]);
                 pk[2] = pack2<T>(x[4], x[5]);
                 pk[3] = pack2<T>(x[6], x[7]);
+                // The weight a key really gets is round16(P * v_scale) / v_scale = P (1 + eps), |eps| <= 2^-8 (bf16).
+                // The output is divided by the sum of THOSE weights, so that it stays a convex combination of
+                // the dequantised values (a row that sees one key returns that key exactly); the LSE keeps the
+                // sum of the unrounded P.
+                float pcorr = 0.f;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const uint32_t w = pk[e >> 1];
+                    const float xr = to_float<T>((uint16_t)((e & 1) ? (w >> 16) : (w & 0xffffu)));
+                    pcorr = __builtin_fmaf(xr - x[e], vin[e], pcorr);
+                }
+                l_norm = l_norm * alpha + (psum + pcorr);
                 sh.pk[pb][w4][lane] = pk;
                 if (lq == 0) sh.alpha[pb][w4][ln] = alpha;
                 const int wave_bump = __any(bump) ? 1 : 0;
@@ -283,10 +300,11 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
 
         // ---- publish the sums, write the LSE
         l_run = quad_rows_sum(l_run);
+        l_norm = quad_rows_sum(l_norm);
         const int lane = tid & 63;
         const int ln = lane & 15;
         if ((lane >> 4) == 0) {
-            sh.l[w4][ln] = l_run;
+            sh.l[w4][ln] = (l_run > 0.f) ? l_norm : 0.f;
             const int row = w4 * 16 + ln;
             if (write_final)
                 p.lse[((int64_t)b * p.nheads + head) * p.seqlen_q + qi] = (l_run > 0.f) ? (m_run + fast_log2(l_run)) * kLn2 : INFINITY;

@@ -173,3 +173,22 @@ def test_mla_batch_larger_than_prefix_segments():
     case = mla_case(270, 64, lens, page=64, seed=10)
     got, ref, gold = run(case)
     check_out(got[0], ref[0], got[1], ref[1], "mla B=270")
+
+
+def test_mla_one_key_returns_that_key():
+    # the output is a convex combination of the dequantised rows: the kernel rounds P * v_scale to bf16 and divides by
+    # the sum of the weights it really applied, so a row that sees a single key gives that key's values, to the
+    # rounding of the output alone
+    from flash_attn_npu import flash_attn_with_kvcache
+    case = mla_case(6, 128, [1, 1, 1, 1, 1, 1], seed=12)
+    kc = case["k_cache"].cuda()
+    out = flash_attn_with_kvcache(case["q"].cuda(), kc, kc[..., :512], cache_seqlens=case["cache_seqlens"].cuda(),
+                                  block_table=case["block_table"].cuda(), softmax_scale=192 ** -0.5, causal=True,
+                                  k_scale_cache=case["k_scale"].cuda())
+    torch.cuda.synchronize()
+    for b in range(6):
+        blk = int(case["block_table"][b, 0])
+        want = O.dequantize_per_token(case["k_cache"][blk, 0, 0, :512], case["k_scale"][blk, 0, 0]).to(torch.bfloat16)
+        diff = (out[b, 0].cpu().float() - want.float().expand(128, 512)).abs()
+        # 1 / sum and the product are two more fp32 roundings: an element within 1e-7 of a bf16 tie may land on the other side
+        assert (diff <= want.float().abs() * 2.0 ** -7).all() and int((diff != 0).sum()) <= 8, f"row {b}: {int((diff != 0).sum())} differ"
