@@ -5,7 +5,7 @@ import math
 
 import torch
 
-# parity bars (BASELINE north_star): 16-bit outputs vs the fp32 reference, LSE relative
+# parity bars: 16-bit outputs vs the fp32 reference, LSE relative
 OUT_MAX_ABS = 2e-2
 OUT_MEAN_ABS = 2e-3
 LSE_REL = 1e-3
@@ -64,7 +64,7 @@ def to_dev(case, device="cuda"):
 
 
 def check_out(out, ref_fp32, lse, ref_lse, what=""):
-    """north_star bars: max-abs 2e-2, mean-abs 2e-3 vs fp32; LSE 1e-3 relative."""
+    """Parity bars: max-abs 2e-2, mean-abs 2e-3 vs fp32; LSE 1e-3 relative."""
     out = out.detach().float().cpu()
     ref = ref_fp32.detach().float().cpu()
     err = (out - ref).abs()
