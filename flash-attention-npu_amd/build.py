@@ -21,6 +21,7 @@ SOURCES = [
     "decode_wave.hip",
     "decode_mla_i8.hip",
     "prefill_varlen.hip",
+    "ragged_rows.hip",
 ]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")

@@ -603,6 +603,108 @@ int fa_rocm_varlen_validate(const fa_varlen_args *a) {
     return FA_OK;
 }
 
+}  // extern "C"
+
+namespace {
+
+size_t align256(size_t n) { return (n + 255) / 256 * 256; }
+
+// Where the pieces of a varlen call's workspace lie: the partials of the key ranges first, then the
+// batch-major rows of the one-token query blocks and the workspace of the decode launch over them.
+struct VarlenWorkspace {
+    int nsplits;
+    bool single_rows;
+    size_t partials, q_rows, out_rows, lse_rows, lens_rows, decode_ws, decode_ws_bytes, total;
+};
+
+// The decode launch over the one-token blocks of a token-major batch: batch row b is sequence b, with
+// lens_rows[b] keys (0 for the sequences the tiled kernel computes).  `base` may be NULL for planning.
+fa_kvcache_args single_rows_call(const fa_varlen_args *a, char *base, const VarlenWorkspace &w) {
+    fa_kvcache_args k;
+    std::memset(&k, 0, sizeof(k));
+    char *b = base ? base : reinterpret_cast<char *>(uintptr_t(256));   // never followed when planning
+    k.q = b + w.q_rows;
+    k.out = b + w.out_rows;
+    k.softmax_lse = reinterpret_cast<float *>(b + w.lse_rows);
+    k.cache_seqlens = reinterpret_cast<const int32_t *>(b + w.lens_rows);
+    k.k_cache = const_cast<void *>(a->k);
+    k.v_cache = const_cast<void *>(a->v);
+    k.block_table = a->block_table;
+    k.workspace = w.decode_ws_bytes ? b + w.decode_ws : nullptr;
+    k.workspace_bytes = w.decode_ws_bytes;
+    k.batch = a->batch;
+    k.seqlen_q = 1;
+    k.nheads = a->nheads;
+    k.nheads_k = a->nheads_k;
+    k.headdim_qk = k.headdim_v = a->headdim;
+    k.num_blocks = a->num_blocks;
+    k.page_size = a->page_size;
+    k.max_blocks_per_seq = a->max_blocks_per_seq;
+    k.q_stride_h = k.o_stride_h = a->headdim;
+    k.q_stride_s = k.o_stride_s = k.q_stride_b = k.o_stride_b = (int64_t)a->nheads * a->headdim;
+    k.k_stride_block = a->k_stride_block;
+    k.k_stride_row = a->k_stride_t;
+    k.k_stride_h = a->k_stride_h;
+    k.v_stride_block = a->v_stride_block;
+    k.v_stride_row = a->v_stride_t;
+    k.v_stride_h = a->v_stride_h;
+    k.bt_stride_b = a->bt_stride_b;
+    k.io_dtype = k.kv_dtype = a->io_dtype;
+    k.softmax_scale = a->softmax_scale;
+    k.softcap = a->softcap;
+    k.causal = a->causal;
+    k.window_left = a->window_left;
+    k.window_right = a->window_right;
+    return k;
+}
+
+// A token-major batch over a paged cache whose query blocks are far shorter than the longest one on average
+// is taken for a prompt chunk among decode rows: its one-token blocks go to the decode kernels (which stream
+// their keys at memory speed), the tiled forward computes the rest.  Decided from shapes; which block has
+// one token is decided on the device.
+bool routes_single_rows(const fa_varlen_args *a) {
+    if (!a->block_table || a->batch < 2 || a->max_seqlen_q <= 1 || a->total_q <= 0) return false;
+    if (a->nheads / a->nheads_k > fa::kDecodeMaxRows) return false;
+    if ((int64_t)a->total_q * 4 > (int64_t)a->batch * a->max_seqlen_q) return false;
+    return std::getenv("FA_ROCM_NO_SINGLE_ROWS") == nullptr;
+}
+
+VarlenWorkspace varlen_workspace(const fa_varlen_args *a, int num_cus) {
+    VarlenWorkspace w;
+    std::memset(&w, 0, sizeof(w));
+    w.nsplits = fa_rocm_varlen_num_splits(a, num_cus);
+    size_t off = 0;
+    if (w.nsplits > 1) off = align256((size_t)a->total_q * a->nheads * w.nsplits * ((size_t)a->headdim + 1) * sizeof(float));
+    w.single_rows = routes_single_rows(a);
+    if (w.single_rows) {
+        const size_t rows = (size_t)a->batch * a->nheads;
+        w.q_rows = off;
+        off += align256(rows * a->headdim * 2);
+        w.out_rows = off;
+        off += align256(rows * a->headdim * 2);
+        w.lse_rows = off;
+        off += align256(rows * sizeof(float));
+        w.lens_rows = off;
+        off += align256((size_t)a->batch * sizeof(int32_t));
+        const fa_kvcache_args k = single_rows_call(a, nullptr, w);
+        fa_split_plan plan;
+        if (fa_rocm_kvcache_validate(&k) != FA_OK || fa_rocm_plan_kvcache(&k, num_cus, &plan) != FA_OK) {
+            w.single_rows = false;     // a cache the decode kernels do not take: everything stays on the tiled kernel
+            off = w.q_rows;
+        } else {
+            w.decode_ws = off;
+            w.decode_ws_bytes = plan.workspace_bytes;
+            off += align256(plan.workspace_bytes);
+        }
+    }
+    w.total = off;
+    return w;
+}
+
+}  // namespace
+
+extern "C" {
+
 int fa_rocm_varlen_num_splits(const fa_varlen_args *a, int num_cus) {
     if (fa_rocm_varlen_validate(a) != FA_OK) return 1;
     if (!a->block_table || a->num_splits == 1 || a->total_q <= 0) return 1;
@@ -635,9 +737,8 @@ int fa_rocm_varlen_num_splits(const fa_varlen_args *a, int num_cus) {
 }
 
 size_t fa_rocm_varlen_workspace_bytes(const fa_varlen_args *a, int num_cus) {
-    const int n = fa_rocm_varlen_num_splits(a, num_cus);
-    if (n <= 1) return 0;
-    return (size_t)a->total_q * a->nheads * n * ((size_t)a->headdim + 1) * sizeof(float);
+    if (fa_rocm_varlen_validate(a) != FA_OK) return 0;
+    return varlen_workspace(a, num_cus <= 0 ? 256 : num_cus).total;
 }
 
 int fa_rocm_varlen_fwd(const fa_varlen_args *a, void *stream_) {
@@ -645,10 +746,40 @@ int fa_rocm_varlen_fwd(const fa_varlen_args *a, void *stream_) {
     if (rc != FA_OK) return rc;
     int cus = device_cus();
     if (cus <= 0) cus = 256;
-    const int nsplits = fa_rocm_varlen_num_splits(a, cus);
-    const size_t ws_bytes = fa_rocm_varlen_workspace_bytes(a, cus);
-    if (ws_bytes > 0 && (!a->workspace || a->workspace_bytes < ws_bytes))
-        return fail(FA_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", ws_bytes, a->workspace ? a->workspace_bytes : (size_t)0);
+    const VarlenWorkspace w = varlen_workspace(a, cus);
+    const int nsplits = w.nsplits;
+    if (w.total > 0 && (!a->workspace || a->workspace_bytes < w.total))
+        return fail(FA_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", w.total, a->workspace ? a->workspace_bytes : (size_t)0);
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    fa::SingleRowsParams sr;
+    std::memset(&sr, 0, sizeof(sr));
+    if (w.single_rows) {
+        // the one-token blocks: gathered into batch-major rows, computed by the decode kernels with every other
+        // sequence's key count set to 0, scattered back after the tiled kernel (which skips them) has been queued
+        char *base = static_cast<char *>(a->workspace);
+        sr.q = a->q;
+        sr.out = a->out;
+        sr.lse = a->softmax_lse;
+        sr.cu_seqlens_q = a->cu_seqlens_q;
+        sr.seqused_k = a->seqused_k;
+        sr.q_rows = base + w.q_rows;
+        sr.out_rows = base + w.out_rows;
+        sr.lse_rows = reinterpret_cast<float *>(base + w.lse_rows);
+        sr.lens_rows = reinterpret_cast<int32_t *>(base + w.lens_rows);
+        sr.batch = a->batch;
+        sr.total_q = a->total_q;
+        sr.nheads = a->nheads;
+        sr.headdim = a->headdim;
+        sr.q_stride_t = a->q_stride_t;
+        sr.q_stride_h = a->q_stride_h;
+        sr.o_stride_t = a->o_stride_t;
+        sr.o_stride_h = a->o_stride_h;
+        const hipError_t eg = fa::launch_gather_single_rows(sr, stream);
+        if (eg != hipSuccess) return fail(FA_ERR_LAUNCH, "gather launch failed: %s", hipGetErrorString(eg));
+        const fa_kvcache_args k = single_rows_call(a, base, w);
+        const int rk = fa_rocm_fwd_kvcache(&k, stream_);
+        if (rk != FA_OK) return rk;
+    }
     fa::PrefillParams pp;
     std::memset(&pp, 0, sizeof(pp));
     pp.q = a->q;
@@ -697,10 +828,15 @@ int fa_rocm_varlen_fwd(const fa_varlen_args *a, void *stream_) {
         pp.o_partial = static_cast<float *>(a->workspace);
         pp.lse_partial = pp.o_partial + (size_t)a->total_q * a->nheads * nsplits * a->headdim;
     }
-    const hipError_t e = fa::launch_prefill(pp, a->io_dtype, a->headdim, static_cast<hipStream_t>(stream_));
+    pp.skip_single = w.single_rows ? 1 : 0;
+    const hipError_t e = fa::launch_prefill(pp, a->io_dtype, a->headdim, stream);
     if (e != hipSuccess) return fail(FA_ERR_LAUNCH, "prefill launch failed: %s", hipGetErrorString(e));
-    const hipError_t ec = fa::launch_prefill_combine(pp, a->io_dtype, a->headdim, static_cast<hipStream_t>(stream_));
+    const hipError_t ec = fa::launch_prefill_combine(pp, a->io_dtype, a->headdim, stream);
     if (ec != hipSuccess) return fail(FA_ERR_LAUNCH, "combine launch failed: %s", hipGetErrorString(ec));
+    if (w.single_rows) {
+        const hipError_t es = fa::launch_scatter_single_rows(sr, stream);
+        if (es != hipSuccess) return fail(FA_ERR_LAUNCH, "scatter launch failed: %s", hipGetErrorString(es));
+    }
     return FA_OK;
 }
 

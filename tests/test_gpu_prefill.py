@@ -306,3 +306,38 @@ def test_varlen_paged_ragged_blocks_split_keys(hq, hk, d, causal, window, num_sp
     torch.cuda.synchronize()
     ref, ref_lse = O.flash_attn_varlen(q, kl, vl, cu_q, cu_k, max(lens_q), max(lens_k), causal=causal, window_size=window, mode="fp32")
     check_out(out, ref, lse, ref_lse, "ragged split")
+
+
+@pytest.mark.parametrize("causal,window,softcap", [(True, (-1, -1), 0.0), (False, (-1, -1), 0.0), (True, (1500, 0), 0.0),
+                                                     (False, (3000, 7), 0.0), (True, (-1, -1), 20.0)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_varlen_paged_one_token_blocks_on_the_decode_kernels(causal, window, softcap, dtype):
+    # a prompt chunk among decode rows: the one-token blocks are computed by the decode kernels, the others by the
+    # tiled kernel; both against the oracle, and against the same call with the routing switched off
+    import os
+    from flash_attn_npu.flash_attn_npu import varlen_fwd
+    lens_q = [1, 1, 400, 1, 0, 1, 2, 1]
+    lens_k = [4000, 1, 2500, 0, 300, 777, 64, 6000]
+    hq, hk, d = 16, 4, 128
+    case, q, cu_q, cu_k, kl, vl = paged_ragged(lens_q, lens_k, hq, hk, d, 128, seed=41, dtype=dtype)
+    dev = [q.cuda(), case["k_cache"].cuda(), case["v_cache"].cuda(), cu_q.cuda(), case["cache_seqlens"].cuda(), case["block_table"].cuda()]
+
+    def call():
+        out, lse, _, _ = varlen_fwd(dev[0], dev[1], dev[2], None, dev[3], None, dev[4], None, dev[5], None, max(lens_q), max(lens_k),
+                                    0.0, d ** -0.5, False, causal, window[0], window[1], softcap, False, None)
+        torch.cuda.synchronize()
+        return out, lse
+
+    print("one-token blocks", causal, window, softcap, dtype, flush=True)
+    out, lse = call()
+    ref, ref_lse = O.flash_attn_varlen(q, kl, vl, cu_q, cu_k, max(lens_q), max(lens_k), causal=causal, window_size=window,
+                                       softcap=softcap, mode="fp32")
+    check_out(out, ref, lse, ref_lse, "one-token blocks")
+    os.environ["FA_ROCM_NO_SINGLE_ROWS"] = "1"
+    try:
+        out2, lse2 = call()
+    finally:
+        del os.environ["FA_ROCM_NO_SINGLE_ROWS"]
+    check_out(out2, ref, lse2, ref_lse, "one-token blocks, tiled kernel only")
+    single = torch.tensor([n == 1 for n in lens_q for _ in range(n)])
+    assert torch.equal(out[~single].cpu(), out2[~single].cpu()), "rows of the tiled kernel changed with the routing"
