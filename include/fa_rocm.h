@@ -128,7 +128,12 @@ typedef struct fa_varlen_args {
      * batches).  0 = as many ranges as it takes, 1 = never, n = at most n.  The ranges leave fp32
      * partials in `workspace` (fa_rocm_varlen_workspace_bytes), merged by a second kernel.  The
      * reference's third-generation surface takes num_splits for token-major q the same way
-     * (flash_attn_npu_3/flash_attn_npu_interface.py:965-996). */
+     * (flash_attn_npu_3/flash_attn_npu_interface.py:965-996).
+     * When the query blocks are far shorter than the longest one on average
+     * (4 * total_q <= batch * max_seqlen_q: a prompt chunk among decode rows), the blocks of exactly one
+     * token are computed by the decode kernels of fa_rocm_fwd_kvcache instead; their batch-major rows and
+     * that launch's own workspace are part of `workspace` too.  Which blocks those are is decided on the
+     * device, so the call records into a graph like every other. */
     int32_t num_splits;
     void *workspace;
     size_t workspace_bytes;
