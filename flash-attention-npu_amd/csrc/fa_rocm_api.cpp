@@ -663,19 +663,25 @@ fa_kvcache_args single_rows_call(const fa_varlen_args *a, char *base, const Varl
 // their keys at memory speed), the tiled forward computes the rest.  Decided from shapes; which block has
 // one token is decided on the device.
 bool routes_single_rows(const fa_varlen_args *a) {
-    if (!a->block_table || a->batch < 2 || a->max_seqlen_q <= 1 || a->total_q <= 0) return false;
+    if (!a->block_table || a->total_q <= 0) return false;
     if (a->nheads / a->nheads_k > fa::kDecodeMaxRows) return false;
-    if ((int64_t)a->total_q * 4 > (int64_t)a->batch * a->max_seqlen_q) return false;
+    // max_seqlen_q == 1: every block that is not empty has one token, and nothing is left for the tiled kernel
+    if (a->max_seqlen_q > 1 && (a->batch < 2 || (int64_t)a->total_q * 4 > (int64_t)a->batch * a->max_seqlen_q)) return false;
     return std::getenv("FA_ROCM_NO_SINGLE_ROWS") == nullptr;
 }
 
 VarlenWorkspace varlen_workspace(const fa_varlen_args *a, int num_cus) {
     VarlenWorkspace w;
     std::memset(&w, 0, sizeof(w));
-    w.nsplits = fa_rocm_varlen_num_splits(a, num_cus);
+    w.single_rows = routes_single_rows(a);
+    if (w.single_rows) {
+        const fa_kvcache_args probe = single_rows_call(a, nullptr, w);
+        if (fa_rocm_kvcache_validate(&probe) != FA_OK) w.single_rows = false;   // a cache the decode kernels do not take
+    }
+    const bool decode_only = w.single_rows && a->max_seqlen_q == 1;
+    w.nsplits = decode_only ? 1 : fa_rocm_varlen_num_splits(a, num_cus);
     size_t off = 0;
     if (w.nsplits > 1) off = align256((size_t)a->total_q * a->nheads * w.nsplits * ((size_t)a->headdim + 1) * sizeof(float));
-    w.single_rows = routes_single_rows(a);
     if (w.single_rows) {
         const size_t rows = (size_t)a->batch * a->nheads;
         w.q_rows = off;
@@ -688,14 +694,10 @@ VarlenWorkspace varlen_workspace(const fa_varlen_args *a, int num_cus) {
         off += align256((size_t)a->batch * sizeof(int32_t));
         const fa_kvcache_args k = single_rows_call(a, nullptr, w);
         fa_split_plan plan;
-        if (fa_rocm_kvcache_validate(&k) != FA_OK || fa_rocm_plan_kvcache(&k, num_cus, &plan) != FA_OK) {
-            w.single_rows = false;     // a cache the decode kernels do not take: everything stays on the tiled kernel
-            off = w.q_rows;
-        } else {
-            w.decode_ws = off;
-            w.decode_ws_bytes = plan.workspace_bytes;
-            off += align256(plan.workspace_bytes);
-        }
+        if (fa_rocm_plan_kvcache(&k, num_cus, &plan) != FA_OK) plan.workspace_bytes = 0;   // cannot fail after the check above
+        w.decode_ws = off;
+        w.decode_ws_bytes = plan.workspace_bytes;
+        off += align256(plan.workspace_bytes);
     }
     w.total = off;
     return w;
@@ -829,10 +831,12 @@ int fa_rocm_varlen_fwd(const fa_varlen_args *a, void *stream_) {
         pp.lse_partial = pp.o_partial + (size_t)a->total_q * a->nheads * nsplits * a->headdim;
     }
     pp.skip_single = w.single_rows ? 1 : 0;
-    const hipError_t e = fa::launch_prefill(pp, a->io_dtype, a->headdim, stream);
-    if (e != hipSuccess) return fail(FA_ERR_LAUNCH, "prefill launch failed: %s", hipGetErrorString(e));
-    const hipError_t ec = fa::launch_prefill_combine(pp, a->io_dtype, a->headdim, stream);
-    if (ec != hipSuccess) return fail(FA_ERR_LAUNCH, "combine launch failed: %s", hipGetErrorString(ec));
+    if (!(w.single_rows && a->max_seqlen_q == 1)) {
+        const hipError_t e = fa::launch_prefill(pp, a->io_dtype, a->headdim, stream);
+        if (e != hipSuccess) return fail(FA_ERR_LAUNCH, "prefill launch failed: %s", hipGetErrorString(e));
+        const hipError_t ec = fa::launch_prefill_combine(pp, a->io_dtype, a->headdim, stream);
+        if (ec != hipSuccess) return fail(FA_ERR_LAUNCH, "combine launch failed: %s", hipGetErrorString(ec));
+    }
     if (w.single_rows) {
         const hipError_t es = fa::launch_scatter_single_rows(sr, stream);
         if (es != hipSuccess) return fail(FA_ERR_LAUNCH, "scatter launch failed: %s", hipGetErrorString(es));

@@ -341,3 +341,19 @@ def test_varlen_paged_one_token_blocks_on_the_decode_kernels(causal, window, sof
     check_out(out2, ref, lse2, ref_lse, "one-token blocks, tiled kernel only")
     single = torch.tensor([n == 1 for n in lens_q for _ in range(n)])
     assert torch.equal(out[~single].cpu(), out2[~single].cpu()), "rows of the tiled kernel changed with the routing"
+
+
+@pytest.mark.parametrize("causal,window", [(True, (-1, -1)), (False, (-1, -1)), (False, (500, 3))])
+def test_varlen_paged_all_blocks_one_token(causal, window):
+    # max_seqlen_q = 1: the whole call runs on the decode kernels (empty blocks have no rows to write)
+    from flash_attn_npu.flash_attn_npu import varlen_fwd
+    lens_q = [1, 1, 0, 1, 1]
+    lens_k = [3000, 1, 500, 0, 1025]
+    hq, hk, d = 8, 2, 128
+    case, q, cu_q, cu_k, kl, vl = paged_ragged(lens_q, lens_k, hq, hk, d, 64, seed=43)
+    out, lse, _, _ = varlen_fwd(q.cuda(), case["k_cache"].cuda(), case["v_cache"].cuda(), None, cu_q.cuda(), None,
+                                case["cache_seqlens"].cuda(), None, case["block_table"].cuda(), None, 1, max(lens_k),
+                                0.0, d ** -0.5, False, causal, window[0], window[1], 0.0, False, None)
+    torch.cuda.synchronize()
+    ref, ref_lse = O.flash_attn_varlen(q, kl, vl, cu_q, cu_k, 1, max(lens_k), causal=causal, window_size=window, mode="fp32")
+    check_out(out, ref, lse, ref_lse, "all blocks one token")
