@@ -85,19 +85,20 @@ struct RotateQParams {
     int64_t q_stride_b, q_stride_s, q_stride_h;
 };
 
-// One-token query blocks of a token-major batch between the token-major tensors of the call and the
-// batch-major rows (B, 1, Hq, D) / (B, Hq) that the decode kernels work on.
-struct SingleRowsParams {
+// Short query blocks (1 .. slots tokens) of a token-major batch between the token-major tensors of the call
+// and the batch-major blocks (B, slots, Hq, D) / (B, Hq, slots) that the decode kernels work on; a block of n
+// tokens occupies the last n slots.
+struct ShortBlocksParams {
     const void *q;                 // (total_q, Hq, D)
     void *out;                     // (total_q, Hq, D)
     float *lse;                    // (Hq, total_q)
     const int32_t *cu_seqlens_q;   // (B + 1,)
     const int32_t *seqused_k;      // (B,)
-    void *q_rows;                  // (B, Hq, D) contiguous
-    const void *out_rows;          // (B, Hq, D) contiguous
-    const float *lse_rows;         // (B, Hq)
-    int32_t *lens_rows;            // (B,): seqused_k of the one-token sequences, 0 for the others
-    int32_t batch, total_q, nheads, headdim;
+    void *q_rows;                  // (B, slots, Hq, D) contiguous
+    const void *out_rows;          // (B, slots, Hq, D) contiguous
+    const float *lse_rows;         // (B, Hq, slots)
+    int32_t *lens_rows;            // (B,): seqused_k of the short blocks' sequences, 0 for the others
+    int32_t batch, total_q, nheads, headdim, slots;
     int64_t q_stride_t, q_stride_h, o_stride_t, o_stride_h;
 };
 
@@ -116,7 +117,7 @@ struct PrefillParams {
     int32_t batch, nheads, nheads_k, group;
     int32_t pack;                  // set by the launcher: 1, or group when tile rows are (query, head) pairs
     int32_t pack_short;            // set by the launcher: pack == 1, but a short query block packs its heads on its own
-    int32_t skip_single;           // token-major q: sequences with exactly one query token are computed elsewhere
+    int32_t skip_short;            // token-major q: sequences with 1 .. skip_short query tokens are computed elsewhere (0 = none)
     int32_t num_mb, units8;        // set by the launcher: 128-row blocks per unit, units rounded up to 8
     int32_t seqlen_q_fixed, seqlen_k_add;   // kvcache layout: Sq per row, keys appended this call
     int32_t max_seqlen_q, total_q;
@@ -159,8 +160,8 @@ hipError_t launch_prefill(const PrefillParams &p, int dtype, int headdim, hipStr
 // merge of the key ranges of token-major query blocks (cu_seqlens_q set, nsplits > 1) after launch_prefill
 hipError_t launch_prefill_combine(const PrefillParams &p, int dtype, int headdim, hipStream_t stream);
 
-hipError_t launch_gather_single_rows(const SingleRowsParams &p, hipStream_t stream);
-hipError_t launch_scatter_single_rows(const SingleRowsParams &p, hipStream_t stream);
+hipError_t launch_gather_short_blocks(const ShortBlocksParams &p, hipStream_t stream);
+hipError_t launch_scatter_short_blocks(const ShortBlocksParams &p, hipStream_t stream);
 
 // Resident decode workgroups per compute unit for a head dimension / query-block height.
 int decode_wgs_per_cu(int headdim, int rows);

@@ -613,13 +613,15 @@ size_t align256(size_t n) { return (n + 255) / 256 * 256; }
 // batch-major rows of the one-token query blocks and the workspace of the decode launch over them.
 struct VarlenWorkspace {
     int nsplits;
-    bool single_rows;
+    bool short_blocks;
+    int slots;           // query positions per sequence in the decode launch over the short blocks
+    bool decode_only;    // no block is longer than `slots`: the tiled kernel has nothing to do
     size_t partials, q_rows, out_rows, lse_rows, lens_rows, decode_ws, decode_ws_bytes, total;
 };
 
 // The decode launch over the one-token blocks of a token-major batch: batch row b is sequence b, with
 // lens_rows[b] keys (0 for the sequences the tiled kernel computes).  `base` may be NULL for planning.
-fa_kvcache_args single_rows_call(const fa_varlen_args *a, char *base, const VarlenWorkspace &w) {
+fa_kvcache_args short_blocks_call(const fa_varlen_args *a, char *base, const VarlenWorkspace &w) {
     fa_kvcache_args k;
     std::memset(&k, 0, sizeof(k));
     char *b = base ? base : reinterpret_cast<char *>(uintptr_t(256));   // never followed when planning
@@ -633,7 +635,7 @@ fa_kvcache_args single_rows_call(const fa_varlen_args *a, char *base, const Varl
     k.workspace = w.decode_ws_bytes ? b + w.decode_ws : nullptr;
     k.workspace_bytes = w.decode_ws_bytes;
     k.batch = a->batch;
-    k.seqlen_q = 1;
+    k.seqlen_q = w.slots;
     k.nheads = a->nheads;
     k.nheads_k = a->nheads_k;
     k.headdim_qk = k.headdim_v = a->headdim;
@@ -641,7 +643,8 @@ fa_kvcache_args single_rows_call(const fa_varlen_args *a, char *base, const Varl
     k.page_size = a->page_size;
     k.max_blocks_per_seq = a->max_blocks_per_seq;
     k.q_stride_h = k.o_stride_h = a->headdim;
-    k.q_stride_s = k.o_stride_s = k.q_stride_b = k.o_stride_b = (int64_t)a->nheads * a->headdim;
+    k.q_stride_s = k.o_stride_s = (int64_t)a->nheads * a->headdim;
+    k.q_stride_b = k.o_stride_b = (int64_t)w.slots * a->nheads * a->headdim;
     k.k_stride_block = a->k_stride_block;
     k.k_stride_row = a->k_stride_t;
     k.k_stride_h = a->k_stride_h;
@@ -658,32 +661,42 @@ fa_kvcache_args single_rows_call(const fa_varlen_args *a, char *base, const Varl
     return k;
 }
 
+// Query positions per sequence of the decode launch over the short blocks: as many tokens as fit the 16 rows
+// (tokens x q heads per kv head) of the wave-level decode kernel's one tile, so the launch costs the same
+// whether the blocks hold one token or several (decode rows, or speculative decoding's few tokens).
+int short_block_slots(const fa_varlen_args *a) {
+    const int group = a->nheads / a->nheads_k;
+    return std::max(1, std::min(16 / std::max(group, 1), 8));
+}
+
 // A token-major batch over a paged cache whose query blocks are far shorter than the longest one on average
-// is taken for a prompt chunk among decode rows: its one-token blocks go to the decode kernels (which stream
-// their keys at memory speed), the tiled forward computes the rest.  Decided from shapes; which block has
-// one token is decided on the device.
-bool routes_single_rows(const fa_varlen_args *a) {
+// is taken for prompt chunks among decode rows: its short blocks go to the decode kernels (which stream
+// their keys at memory speed), the tiled forward computes the rest.  Decided from shapes; which block is
+// short is decided on the device.  When no block can be longer than the slots, the decode kernels do it all.
+bool routes_short_blocks(const fa_varlen_args *a) {
     if (!a->block_table || a->total_q <= 0) return false;
     if (a->nheads / a->nheads_k > fa::kDecodeMaxRows) return false;
-    // max_seqlen_q == 1: every block that is not empty has one token, and nothing is left for the tiled kernel
-    if (a->max_seqlen_q > 1 && (a->batch < 2 || (int64_t)a->total_q * 4 > (int64_t)a->batch * a->max_seqlen_q)) return false;
-    return std::getenv("FA_ROCM_NO_SINGLE_ROWS") == nullptr;
+    if (a->max_seqlen_q > short_block_slots(a) &&
+        (a->batch < 2 || (int64_t)a->total_q * 4 > (int64_t)a->batch * a->max_seqlen_q))
+        return false;
+    return std::getenv("FA_ROCM_NO_SHORT_BLOCKS") == nullptr;
 }
 
 VarlenWorkspace varlen_workspace(const fa_varlen_args *a, int num_cus) {
     VarlenWorkspace w;
     std::memset(&w, 0, sizeof(w));
-    w.single_rows = routes_single_rows(a);
-    if (w.single_rows) {
-        const fa_kvcache_args probe = single_rows_call(a, nullptr, w);
-        if (fa_rocm_kvcache_validate(&probe) != FA_OK) w.single_rows = false;   // a cache the decode kernels do not take
+    w.short_blocks = routes_short_blocks(a);
+    w.slots = std::min(short_block_slots(a), std::max(a->max_seqlen_q, 1));
+    if (w.short_blocks) {
+        const fa_kvcache_args probe = short_blocks_call(a, nullptr, w);
+        if (fa_rocm_kvcache_validate(&probe) != FA_OK) w.short_blocks = false;   // a cache the decode kernels do not take
     }
-    const bool decode_only = w.single_rows && a->max_seqlen_q == 1;
-    w.nsplits = decode_only ? 1 : fa_rocm_varlen_num_splits(a, num_cus);
+    w.decode_only = w.short_blocks && a->max_seqlen_q <= w.slots;
+    w.nsplits = w.decode_only ? 1 : fa_rocm_varlen_num_splits(a, num_cus);
     size_t off = 0;
     if (w.nsplits > 1) off = align256((size_t)a->total_q * a->nheads * w.nsplits * ((size_t)a->headdim + 1) * sizeof(float));
-    if (w.single_rows) {
-        const size_t rows = (size_t)a->batch * a->nheads;
+    if (w.short_blocks) {
+        const size_t rows = (size_t)a->batch * w.slots * a->nheads;
         w.q_rows = off;
         off += align256(rows * a->headdim * 2);
         w.out_rows = off;
@@ -692,7 +705,7 @@ VarlenWorkspace varlen_workspace(const fa_varlen_args *a, int num_cus) {
         off += align256(rows * sizeof(float));
         w.lens_rows = off;
         off += align256((size_t)a->batch * sizeof(int32_t));
-        const fa_kvcache_args k = single_rows_call(a, nullptr, w);
+        const fa_kvcache_args k = short_blocks_call(a, nullptr, w);
         fa_split_plan plan;
         if (fa_rocm_plan_kvcache(&k, num_cus, &plan) != FA_OK) plan.workspace_bytes = 0;   // cannot fail after the check above
         w.decode_ws = off;
@@ -753,9 +766,9 @@ int fa_rocm_varlen_fwd(const fa_varlen_args *a, void *stream_) {
     if (w.total > 0 && (!a->workspace || a->workspace_bytes < w.total))
         return fail(FA_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", w.total, a->workspace ? a->workspace_bytes : (size_t)0);
     hipStream_t stream = static_cast<hipStream_t>(stream_);
-    fa::SingleRowsParams sr;
+    fa::ShortBlocksParams sr;
     std::memset(&sr, 0, sizeof(sr));
-    if (w.single_rows) {
+    if (w.short_blocks) {
         // the one-token blocks: gathered into batch-major rows, computed by the decode kernels with every other
         // sequence's key count set to 0, scattered back after the tiled kernel (which skips them) has been queued
         char *base = static_cast<char *>(a->workspace);
@@ -772,13 +785,14 @@ int fa_rocm_varlen_fwd(const fa_varlen_args *a, void *stream_) {
         sr.total_q = a->total_q;
         sr.nheads = a->nheads;
         sr.headdim = a->headdim;
+        sr.slots = w.slots;
         sr.q_stride_t = a->q_stride_t;
         sr.q_stride_h = a->q_stride_h;
         sr.o_stride_t = a->o_stride_t;
         sr.o_stride_h = a->o_stride_h;
-        const hipError_t eg = fa::launch_gather_single_rows(sr, stream);
+        const hipError_t eg = fa::launch_gather_short_blocks(sr, stream);
         if (eg != hipSuccess) return fail(FA_ERR_LAUNCH, "gather launch failed: %s", hipGetErrorString(eg));
-        const fa_kvcache_args k = single_rows_call(a, base, w);
+        const fa_kvcache_args k = short_blocks_call(a, base, w);
         const int rk = fa_rocm_fwd_kvcache(&k, stream_);
         if (rk != FA_OK) return rk;
     }
@@ -830,15 +844,15 @@ int fa_rocm_varlen_fwd(const fa_varlen_args *a, void *stream_) {
         pp.o_partial = static_cast<float *>(a->workspace);
         pp.lse_partial = pp.o_partial + (size_t)a->total_q * a->nheads * nsplits * a->headdim;
     }
-    pp.skip_single = w.single_rows ? 1 : 0;
-    if (!(w.single_rows && a->max_seqlen_q == 1)) {
+    pp.skip_short = w.short_blocks ? w.slots : 0;
+    if (!w.decode_only) {
         const hipError_t e = fa::launch_prefill(pp, a->io_dtype, a->headdim, stream);
         if (e != hipSuccess) return fail(FA_ERR_LAUNCH, "prefill launch failed: %s", hipGetErrorString(e));
         const hipError_t ec = fa::launch_prefill_combine(pp, a->io_dtype, a->headdim, stream);
         if (ec != hipSuccess) return fail(FA_ERR_LAUNCH, "combine launch failed: %s", hipGetErrorString(ec));
     }
-    if (w.single_rows) {
-        const hipError_t es = fa::launch_scatter_single_rows(sr, stream);
+    if (w.short_blocks) {
+        const hipError_t es = fa::launch_scatter_short_blocks(sr, stream);
         if (es != hipSuccess) return fail(FA_ERR_LAUNCH, "scatter launch failed: %s", hipGetErrorString(es));
     }
     return FA_OK;

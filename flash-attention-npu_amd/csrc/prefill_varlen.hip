@@ -90,7 +90,7 @@ __global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) prefill_kernel(const 
         q0 = 0;
         Sq = p.seqlen_q_fixed;
     }
-    if (EXT && p.skip_single && Sq == 1) return;   // the decode kernels compute this sequence
+    if (EXT && Sq >= 1 && Sq <= p.skip_short) return;   // the decode kernels compute this sequence
     // tile row R is query R / pg of head h_base + R % pg.  pg is the launch's (every block packs the heads
     // of its group, or none does) unless the launch lets short blocks pack on their own: a block whose
     // (query, head) rows take at most three quarters of the tiles its heads would take one by one is
@@ -529,7 +529,7 @@ __global__ void __launch_bounds__(64) prefill_combine_kernel(const PrefillParams
     const int Sq = p.cu_seqlens_q[b + 1] - p.cu_seqlens_q[b];
     const int Sk = min(p.seqused_k[b] + p.seqlen_k_add, p.max_blocks * p.page_size);
     const int longest = block_max_keys(p.seqused_k, p.batch, p.seqlen_k_add);
-    if (p.skip_single && Sq == 1) return;
+    if (Sq >= 1 && Sq <= p.skip_short) return;
     int wl = p.window_left, wr = p.window_right;
     int norm_m = p.window_norm_m;
     if (norm_m <= 0 && (wl >= 0 || wr >= 0)) norm_m = longest;
@@ -597,7 +597,7 @@ template <typename T, int D> static hipError_t launch_prefill_d(const PrefillPar
     const bool softcap = p.softcap_post != 0.f;
     const bool paged = p.block_table != nullptr;
     p.pack_short = p.cu_seqlens_q ? prefill_pack_short(p.group, p.max_seqlen_q, p.total_q, p.batch) : 0;
-    const bool ext = p.pack > 1 || p.nsplits > 1 || p.pack_short || p.skip_single;
+    const bool ext = p.pack > 1 || p.nsplits > 1 || p.pack_short || p.skip_short > 0;
     auto launch = [&](auto paged_c, auto softcap_c, auto ext_c) {
         hipLaunchKernelGGL((prefill_kernel<T, D, decltype(paged_c)::value, decltype(softcap_c)::value, decltype(ext_c)::value>),
                            grid, block, 0, stream, p);

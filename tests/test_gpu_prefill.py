@@ -311,13 +311,14 @@ def test_varlen_paged_ragged_blocks_split_keys(hq, hk, d, causal, window, num_sp
 @pytest.mark.parametrize("causal,window,softcap", [(True, (-1, -1), 0.0), (False, (-1, -1), 0.0), (True, (1500, 0), 0.0),
                                                      (False, (3000, 7), 0.0), (True, (-1, -1), 20.0)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-def test_varlen_paged_one_token_blocks_on_the_decode_kernels(causal, window, softcap, dtype):
-    # a prompt chunk among decode rows: the one-token blocks are computed by the decode kernels, the others by the
-    # tiled kernel; both against the oracle, and against the same call with the routing switched off
+def test_varlen_paged_short_blocks_on_the_decode_kernels(causal, window, softcap, dtype):
+    # a prompt chunk among decode rows and speculative blocks: blocks of 1 .. 4 tokens (16 rows of 4 q heads per kv
+    # head) are computed by the decode kernels, the others by the tiled kernel; both against the oracle, and against
+    # the same call with the routing switched off
     import os
     from flash_attn_npu.flash_attn_npu import varlen_fwd
-    lens_q = [1, 1, 400, 1, 0, 1, 2, 1]
-    lens_k = [4000, 1, 2500, 0, 300, 777, 64, 6000]
+    lens_q = [1, 1, 400, 1, 0, 4, 2, 1, 5, 3, 1, 2]
+    lens_k = [4000, 1, 2500, 0, 300, 777, 64, 6000, 900, 2, 130, 1]
     hq, hk, d = 16, 4, 128
     case, q, cu_q, cu_k, kl, vl = paged_ragged(lens_q, lens_k, hq, hk, d, 128, seed=41, dtype=dtype)
     dev = [q.cuda(), case["k_cache"].cuda(), case["v_cache"].cuda(), cu_q.cuda(), case["cache_seqlens"].cuda(), case["block_table"].cuda()]
@@ -328,32 +329,34 @@ def test_varlen_paged_one_token_blocks_on_the_decode_kernels(causal, window, sof
         torch.cuda.synchronize()
         return out, lse
 
-    print("one-token blocks", causal, window, softcap, dtype, flush=True)
+    print("short blocks", causal, window, softcap, dtype, flush=True)
     out, lse = call()
     ref, ref_lse = O.flash_attn_varlen(q, kl, vl, cu_q, cu_k, max(lens_q), max(lens_k), causal=causal, window_size=window,
                                        softcap=softcap, mode="fp32")
-    check_out(out, ref, lse, ref_lse, "one-token blocks")
-    os.environ["FA_ROCM_NO_SINGLE_ROWS"] = "1"
+    check_out(out, ref, lse, ref_lse, "short blocks")
+    os.environ["FA_ROCM_NO_SHORT_BLOCKS"] = "1"
     try:
         out2, lse2 = call()
     finally:
-        del os.environ["FA_ROCM_NO_SINGLE_ROWS"]
-    check_out(out2, ref, lse2, ref_lse, "one-token blocks, tiled kernel only")
-    single = torch.tensor([n == 1 for n in lens_q for _ in range(n)])
-    assert torch.equal(out[~single].cpu(), out2[~single].cpu()), "rows of the tiled kernel changed with the routing"
+        del os.environ["FA_ROCM_NO_SHORT_BLOCKS"]
+    check_out(out2, ref, lse2, ref_lse, "short blocks, tiled kernel only")
+    short = torch.tensor([1 <= n <= 4 for n in lens_q for _ in range(n)])
+    assert torch.equal(out[~short].cpu(), out2[~short].cpu()), "rows of the tiled kernel changed with the routing"
+    assert not torch.equal(out[short].cpu(), out2[short].cpu()), "the short blocks did not take the other path"
 
 
 @pytest.mark.parametrize("causal,window", [(True, (-1, -1)), (False, (-1, -1)), (False, (500, 3))])
-def test_varlen_paged_all_blocks_one_token(causal, window):
-    # max_seqlen_q = 1: the whole call runs on the decode kernels (empty blocks have no rows to write)
+@pytest.mark.parametrize("lens_q,hq,hk", [([1, 1, 0, 1, 1], 8, 2), ([2, 4, 0, 1, 3], 8, 2), ([2, 1, 0, 2, 2], 16, 2), ([8, 3, 0, 1, 5], 4, 4)])
+def test_varlen_paged_all_blocks_short(causal, window, lens_q, hq, hk):
+    # no block is longer than the decode launch's slots: the whole call runs on the decode kernels (empty blocks
+    # have no rows to write)
     from flash_attn_npu.flash_attn_npu import varlen_fwd
-    lens_q = [1, 1, 0, 1, 1]
     lens_k = [3000, 1, 500, 0, 1025]
-    hq, hk, d = 8, 2, 128
+    d = 128
     case, q, cu_q, cu_k, kl, vl = paged_ragged(lens_q, lens_k, hq, hk, d, 64, seed=43)
     out, lse, _, _ = varlen_fwd(q.cuda(), case["k_cache"].cuda(), case["v_cache"].cuda(), None, cu_q.cuda(), None,
-                                case["cache_seqlens"].cuda(), None, case["block_table"].cuda(), None, 1, max(lens_k),
+                                case["cache_seqlens"].cuda(), None, case["block_table"].cuda(), None, max(lens_q), max(lens_k),
                                 0.0, d ** -0.5, False, causal, window[0], window[1], 0.0, False, None)
     torch.cuda.synchronize()
-    ref, ref_lse = O.flash_attn_varlen(q, kl, vl, cu_q, cu_k, 1, max(lens_k), causal=causal, window_size=window, mode="fp32")
-    check_out(out, ref, lse, ref_lse, "all blocks one token")
+    ref, ref_lse = O.flash_attn_varlen(q, kl, vl, cu_q, cu_k, max(lens_q), max(lens_k), causal=causal, window_size=window, mode="fp32")
+    check_out(out, ref, lse, ref_lse, "all blocks short")

@@ -80,7 +80,7 @@ def test_varlen_split_plan():
     assert lib.fa_rocm_varlen_fwd(C.byref(a), None) == -5 and b"workspace" in lib.fa_rocm_last_error()
 
 
-def test_varlen_single_rows_workspace():
+def test_varlen_short_blocks_workspace():
     # a prompt chunk among decode rows: the one-token blocks are computed by the decode kernels, whose batch-major
     # rows and own workspace follow the partials in the caller's workspace
     lib = _lib.load()
