@@ -91,6 +91,19 @@ def test_rotary_closed_form_and_special_cases():
     assert torch.equal(a, b)
 
 
+def test_rotary_rounds_to_fp32_then_to_the_io_dtype():
+    # known answer on an exact tie: x1 - x2 * sin = -1.559082081... lies just past the middle of the fp16 neighbours
+    # -1.5595703125 and -1.55859375; the product and the difference each rounded to fp32 give the middle exactly
+    # (-1.55908203125), which rounds to the even neighbour.  One rounding of the unrounded value gives the other one.
+    x = torch.tensor([[[-1.560546875, -0.994140625]]], dtype=torch.float16)
+    cos = torch.tensor([[1.0]], dtype=torch.float16)
+    sin = torch.tensor([[0.0014734268188476562]], dtype=torch.float16)
+    assert float(sin[0, 0]) == 0.0014734268188476562 and float(x[0, 0, 1]) == -0.994140625      # inputs are exact in fp16
+    for inter in (False, True):
+        y = O.apply_rotary(x, cos, sin, torch.tensor([0]), inter)
+        assert float(y[0, 0, 0]) == -1.55859375
+
+
 def test_rotary_q_positions_follow_docstring():
     # q at cache_seqlens + i when causal/local, all at cache_seqlens otherwise (interface docstring :1469-1474)
     c = make_paged_case(1, 2, 1, 32, 32, [10], seqlen_q=3, seqlen_new=3, dtype=torch.float32, seed=5)
