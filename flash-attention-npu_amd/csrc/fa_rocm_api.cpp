@@ -769,8 +769,9 @@ int fa_rocm_varlen_fwd(const fa_varlen_args *a, void *stream_) {
     fa::ShortBlocksParams sr;
     std::memset(&sr, 0, sizeof(sr));
     if (w.short_blocks) {
-        // the one-token blocks: gathered into batch-major rows, computed by the decode kernels with every other
-        // sequence's key count set to 0, scattered back after the tiled kernel (which skips them) has been queued
+        // the short blocks: gathered into batch-major blocks of `slots` query positions, computed by the decode kernels
+        // with every other sequence's key count set to 0, scattered back after the tiled kernel (which skips them) has
+        // been queued
         char *base = static_cast<char *>(a->workspace);
         sr.q = a->q;
         sr.out = a->out;
