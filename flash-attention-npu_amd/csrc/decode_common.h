@@ -23,6 +23,12 @@ __device__ __forceinline__ int window_norm_m(const DecodeParams &p) {
     return block_max_keys(p.cache_seqlens, p.batch, p.seqlen_new);
 }
 
+// Rows of batch row b's query block that nobody reads (padding in front of the real query tokens): the
+// kernels compute them with the others but skip their stores and their merge.
+__device__ __forceinline__ int dead_rows(const DecodeParams &p, int b) {
+    return p.q_live ? max(p.seqlen_q - p.q_live[b], 0) * p.group : 0;
+}
+
 struct UnitRange {
     int len_cache, Lk, lo, hi;
     int wl, wr;       // window after normalisation (-1 = unbounded); causal gives wr = 0

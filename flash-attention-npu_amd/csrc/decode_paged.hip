@@ -568,16 +568,17 @@ __global__ void __launch_bounds__(256) splitkv_combine_balanced_kernel(const Dec
                           (pt.list_heads == 1 ? 0 : (int64_t)kvh * unit_cost(ur.nchunks, pt.cost));
     const UnitPieces pcs = unit_pieces(pt, start, ur.nchunks, kvh, p.nheads_k, pt.cost);
     if (pcs.ns == 1) return;       // written whole by one worker
+    const int row0 = dead_rows(p, b);
     if (pcs.ns <= 16) {
         // few pieces: the four waves merge four rows side by side, no barrier and one chain of
         // dependent loads per row
         const int wave = threadIdx.x >> 6;
-        for (int row = blockIdx.x * 4 + wave; row < p.rows; row += gridDim.x * 4)
+        for (int row = row0 + blockIdx.x * 4 + wave; row < p.rows; row += gridDim.x * 4)
             combine_row_wave<T, D>(p, b, kvh, row, pcs.ns, [&](int s) { return pcs.slot(s); });
         return;
     }
     // many pieces: the whole workgroup on one row at a time
-    for (int row = blockIdx.x; row < p.rows; row += gridDim.x) combine_row_block<T, D>(p, b, kvh, row, pcs);
+    for (int row = row0 + blockIdx.x; row < p.rows; row += gridDim.x) combine_row_block<T, D>(p, b, kvh, row, pcs);
 }
 
 template <typename T, int D, int RT>

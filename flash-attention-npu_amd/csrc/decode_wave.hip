@@ -362,7 +362,7 @@ __device__ __forceinline__ void wave_piece(const DecodeParams &p, const int b, c
     // ---- write.  Register i of column tile t = hh*kVW + w is column hh*128 + (lq*4 + i)*kVW + w
     //      of query row ln: kVW consecutive columns per (hh, i).
     l_run = quad_rows_sum(l_run);
-    if (ln < p.rows) {
+    if (ln < p.rows && ln >= dead_rows(p, b)) {
         const float inv = (l_run > 0.f) ? 1.f / l_run : 0.f;
         const int qi = ln / p.group;
         const int head = kvh * p.group + (ln - qi * p.group);

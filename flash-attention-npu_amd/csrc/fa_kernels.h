@@ -23,6 +23,8 @@ struct DecodeParams {
     const void *rotary_sin;
     const int32_t *cache_seqlens;
     const int32_t *block_table;
+    const int32_t *q_live;   // per batch row: how many query tokens, at the END of the block, are real; the rows of the
+                             // others are computed but neither written nor merged.  NULL: all (balanced wave-level launch only)
     float *o_partial;    // (B, Hk, nsplits, rows, Dv) fp32, each normalised by its own sum
     float *lse_partial;  // (B, Hk, nsplits, rows)     fp32, base-2 log-sum-exp, -inf when empty
     int32_t batch, seqlen_q, nheads, nheads_k, group, rows;  // rows = seqlen_q * group
@@ -98,6 +100,7 @@ struct ShortBlocksParams {
     const void *out_rows;          // (B, slots, Hq, D) contiguous
     const float *lse_rows;         // (B, Hq, slots)
     int32_t *lens_rows;            // (B,): seqused_k of the short blocks' sequences, 0 for the others
+    int32_t *live_rows;            // (B,): tokens of the short blocks (their real query positions), 0 for the others
     int32_t batch, total_q, nheads, headdim, slots;
     int64_t q_stride_t, q_stride_h, o_stride_t, o_stride_h;
 };

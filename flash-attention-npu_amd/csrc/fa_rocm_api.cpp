@@ -301,7 +301,7 @@ int fa_rocm_append_kv(const fa_kvcache_args *a, void *stream) {
     return FA_OK;
 }
 
-static int fwd_kvcache_impl(const fa_kvcache_args *a, void *stream_, void *const *events);
+static int fwd_kvcache_impl(const fa_kvcache_args *a, void *stream_, void *const *events, const int32_t *q_live = nullptr);
 
 int fa_rocm_fwd_kvcache(const fa_kvcache_args *a, void *stream_) { return fwd_kvcache_impl(a, stream_, nullptr); }
 
@@ -310,7 +310,7 @@ int fa_rocm_fwd_kvcache_profiled(const fa_kvcache_args *a, void *stream_, void *
     return fwd_kvcache_impl(a, stream_, events);
 }
 
-static int fwd_kvcache_impl(const fa_kvcache_args *a, void *stream_, void *const *events) {
+static int fwd_kvcache_impl(const fa_kvcache_args *a, void *stream_, void *const *events, const int32_t *q_live) {
     int rc = fa_rocm_kvcache_validate(a);
     if (rc != FA_OK) return rc;
     hipStream_t stream = static_cast<hipStream_t>(stream_);
@@ -475,6 +475,7 @@ static int fwd_kvcache_impl(const fa_kvcache_args *a, void *stream_, void *const
     p.rotary_sin = a->k_new ? a->rotary_sin : nullptr;
     p.cache_seqlens = a->cache_seqlens;
     p.block_table = a->block_table;
+    p.q_live = q_live;
     p.batch = a->batch;
     p.seqlen_q = a->seqlen_q;
     p.nheads = a->nheads;
@@ -616,7 +617,7 @@ struct VarlenWorkspace {
     bool short_blocks;
     int slots;           // query positions per sequence in the decode launch over the short blocks
     bool decode_only;    // no block is longer than `slots`: the tiled kernel has nothing to do
-    size_t partials, q_rows, out_rows, lse_rows, lens_rows, decode_ws, decode_ws_bytes, total;
+    size_t partials, q_rows, out_rows, lse_rows, lens_rows, live_rows, decode_ws, decode_ws_bytes, total;
 };
 
 // The decode launch over the one-token blocks of a token-major batch: batch row b is sequence b, with
@@ -705,6 +706,8 @@ VarlenWorkspace varlen_workspace(const fa_varlen_args *a, int num_cus) {
         off += align256(rows * sizeof(float));
         w.lens_rows = off;
         off += align256((size_t)a->batch * sizeof(int32_t));
+        w.live_rows = off;
+        off += align256((size_t)a->batch * sizeof(int32_t));
         const fa_kvcache_args k = short_blocks_call(a, nullptr, w);
         fa_split_plan plan;
         if (fa_rocm_plan_kvcache(&k, num_cus, &plan) != FA_OK) plan.workspace_bytes = 0;   // cannot fail after the check above
@@ -782,6 +785,7 @@ int fa_rocm_varlen_fwd(const fa_varlen_args *a, void *stream_) {
         sr.out_rows = base + w.out_rows;
         sr.lse_rows = reinterpret_cast<float *>(base + w.lse_rows);
         sr.lens_rows = reinterpret_cast<int32_t *>(base + w.lens_rows);
+        sr.live_rows = reinterpret_cast<int32_t *>(base + w.live_rows);
         sr.batch = a->batch;
         sr.total_q = a->total_q;
         sr.nheads = a->nheads;
@@ -794,7 +798,8 @@ int fa_rocm_varlen_fwd(const fa_varlen_args *a, void *stream_) {
         const hipError_t eg = fa::launch_gather_short_blocks(sr, stream);
         if (eg != hipSuccess) return fail(FA_ERR_LAUNCH, "gather launch failed: %s", hipGetErrorString(eg));
         const fa_kvcache_args k = short_blocks_call(a, base, w);
-        const int rk = fa_rocm_fwd_kvcache(&k, stream_);
+        // the padded query positions in front of a block's tokens are computed with them but neither stored nor merged
+        const int rk = fwd_kvcache_impl(&k, stream_, nullptr, w.slots > 1 ? sr.live_rows : nullptr);
         if (rk != FA_OK) return rk;
     }
     fa::PrefillParams pp;

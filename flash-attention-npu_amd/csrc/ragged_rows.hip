@@ -22,7 +22,10 @@ __global__ void __launch_bounds__(256) gather_short_blocks_kernel(const ShortBlo
     const int q0 = p.cu_seqlens_q[b];
     const int n = p.cu_seqlens_q[b + 1] - q0;
     const bool is_short = n >= 1 && n <= p.slots;
-    if (threadIdx.x == 0) p.lens_rows[b] = is_short ? p.seqused_k[b] : 0;
+    if (threadIdx.x == 0) {
+        p.lens_rows[b] = is_short ? p.seqused_k[b] : 0;
+        p.live_rows[b] = is_short ? n : 0;
+    }
     const int pieces_per_head = p.headdim / 8;
     const int pieces_per_token = p.nheads * pieces_per_head;
     const int pad = is_short ? p.slots - n : p.slots;
