@@ -665,6 +665,12 @@ fa_kvcache_args short_blocks_call(const fa_varlen_args *a, char *base, const Var
 // Query positions per sequence of the decode launch over the short blocks: as many tokens as fit the 16 rows
 // (tokens x q heads per kv head) of the wave-level decode kernel's one tile, so the launch costs the same
 // whether the blocks hold one token or several (decode rows, or speculative decoding's few tokens).
+// The query blocks other than the longest one are, on average, at most a quarter of it: a prompt chunk (or a
+// few) among decode rows.  From shapes alone; the block lengths themselves stay on the device.
+bool uneven_blocks(const fa_varlen_args *a) {
+    return a->batch >= 2 && ((int64_t)a->total_q - a->max_seqlen_q) * 4 <= (int64_t)(a->batch - 1) * a->max_seqlen_q;
+}
+
 int short_block_slots(const fa_varlen_args *a) {
     const int group = a->nheads / a->nheads_k;
     return std::max(1, std::min(16 / std::max(group, 1), 8));
@@ -677,9 +683,7 @@ int short_block_slots(const fa_varlen_args *a) {
 bool routes_short_blocks(const fa_varlen_args *a) {
     if (!a->block_table || a->total_q <= 0) return false;
     if (a->nheads / a->nheads_k > fa::kDecodeMaxRows) return false;
-    if (a->max_seqlen_q > short_block_slots(a) &&
-        (a->batch < 2 || (int64_t)a->total_q * 4 > (int64_t)a->batch * a->max_seqlen_q))
-        return false;
+    if (a->max_seqlen_q > short_block_slots(a) && !uneven_blocks(a)) return false;
     return std::getenv("FA_ROCM_NO_SHORT_BLOCKS") == nullptr;
 }
 
@@ -740,7 +744,7 @@ int fa_rocm_varlen_num_splits(const fa_varlen_args *a, int num_cus) {
         const int64_t slots = (int64_t)num_cus * (a->headdim <= 128 ? 2 : 1);
         // query blocks far shorter than the longest one on average (a prompt chunk among decode rows): the
         // longest block is the critical path long before the tiles fill the device, so it is cut earlier
-        const bool uneven = (int64_t)a->total_q * 4 <= (int64_t)a->batch * a->max_seqlen_q;
+        const bool uneven = uneven_blocks(a);
         if (uneven) {
             if (tiles < 2 * slots) n = (2 * slots + tiles - 1) / tiles;
         } else if (tiles * 2 <= slots) {

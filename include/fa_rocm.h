@@ -130,7 +130,7 @@ typedef struct fa_varlen_args {
      * reference's third-generation surface takes num_splits for token-major q the same way
      * (flash_attn_npu_3/flash_attn_npu_interface.py:965-996).
      * When the query blocks are far shorter than the longest one on average
-     * (4 * total_q <= batch * max_seqlen_q: prompt chunks among decode rows), the short blocks - as many
+     * (4 * (total_q - max_seqlen_q) <= (batch - 1) * max_seqlen_q: prompt chunks among decode rows), the short blocks - as many
      * tokens as fit 16 rows of tokens x q heads per kv head, at most 8 - are computed by the decode kernels
      * of fa_rocm_fwd_kvcache instead, and so is a whole call whose max_seqlen_q is that short; their
      * batch-major copies and that launch's own workspace are part of `workspace` too.  Which blocks are

@@ -360,3 +360,18 @@ def test_varlen_paged_all_blocks_short(causal, window, lens_q, hq, hk):
     torch.cuda.synchronize()
     ref, ref_lse = O.flash_attn_varlen(q, kl, vl, cu_q, cu_k, max(lens_q), max(lens_k), causal=causal, window_size=window, mode="fp32")
     check_out(out, ref, lse, ref_lse, "all blocks short")
+
+
+def test_varlen_paged_small_mixed_batch():
+    # one prompt chunk and two decode rows: the rule that calls a batch uneven looks at the blocks other than the longest
+    import ctypes as C
+    from flash_attn_npu.flash_attn_npu import varlen_fwd
+    lens_q, lens_k = [1, 300, 1], [5000, 4000, 129]
+    hq, hk, d = 8, 2, 128
+    case, q, cu_q, cu_k, kl, vl = paged_ragged(lens_q, lens_k, hq, hk, d, 64, seed=47)
+    out, lse, _, _ = varlen_fwd(q.cuda(), case["k_cache"].cuda(), case["v_cache"].cuda(), None, cu_q.cuda(), None,
+                                case["cache_seqlens"].cuda(), None, case["block_table"].cuda(), None, max(lens_q), max(lens_k),
+                                0.0, d ** -0.5, False, True, -1, -1, 0.0, False, None)
+    torch.cuda.synchronize()
+    ref, ref_lse = O.flash_attn_varlen(q, kl, vl, cu_q, cu_k, max(lens_q), max(lens_k), causal=True, mode="fp32")
+    check_out(out, ref, lse, ref_lse, "small mixed batch")

@@ -54,7 +54,7 @@ def test_varlen_split_plan():
     fake = 0x1000        # the planner and the checks never follow a pointer
     for f in ("q", "k", "v", "out", "softmax_lse", "cu_seqlens_q", "seqused_k", "block_table"):
         setattr(a, f, fake)
-    a.batch, a.total_q, a.nheads, a.nheads_k, a.headdim = 2, 300, 8, 2, 128
+    a.batch, a.total_q, a.nheads, a.nheads_k, a.headdim = 2, 598, 8, 2, 128      # two blocks of 299 tokens
     a.max_seqlen_q, a.max_seqlen_k, a.page_size, a.max_blocks_per_seq, a.num_blocks = 299, 100000, 64, 2000, 4000
     a.q_stride_t = a.o_stride_t = 1024
     a.q_stride_h = a.o_stride_h = a.k_stride_h = a.v_stride_h = 128
@@ -62,7 +62,7 @@ def test_varlen_split_plan():
     a.io_dtype = 0
     n = lib.fa_rocm_varlen_num_splits(C.byref(a), 256)
     assert 1 < n <= 64
-    assert 0 <= lib.fa_rocm_varlen_workspace_bytes(C.byref(a), 256) - 300 * 8 * n * 129 * 4 < 256
+    assert 0 <= lib.fa_rocm_varlen_workspace_bytes(C.byref(a), 256) - 598 * 8 * n * 129 * 4 < 256
     a.num_splits = 1
     assert lib.fa_rocm_varlen_num_splits(C.byref(a), 256) == 1 and lib.fa_rocm_varlen_workspace_bytes(C.byref(a), 256) == 0
     a.num_splits = 500
@@ -71,7 +71,7 @@ def test_varlen_split_plan():
     assert lib.fa_rocm_varlen_num_splits(C.byref(a), 256) == 3
     a.max_seqlen_k, a.total_q, a.max_seqlen_q = 100000, 40000, 20000          # the tiles fill the device: no cut
     assert lib.fa_rocm_varlen_num_splits(C.byref(a), 256) == 1
-    a.total_q, a.block_table = 300, None
+    a.total_q, a.max_seqlen_q, a.block_table = 598, 299, None
     a.cu_seqlens_k = fake
     assert lib.fa_rocm_varlen_num_splits(C.byref(a), 256) == 1
     # a workspace that is too small is refused before anything is launched
@@ -101,7 +101,11 @@ def test_varlen_short_blocks_workspace():
     least = partials + 2 * rows * 128 * 2 + rows * 4 + 16 * 4
     with_rows = lib.fa_rocm_varlen_workspace_bytes(C.byref(a), 256)
     assert with_rows > least
-    a.max_seqlen_q, a.total_q = 40, 527                 # blocks of similar length: nothing is routed
+    a.batch, a.total_q, a.max_seqlen_q = 3, 302, 300     # one chunk, two decode rows: uneven as well
+    small = lib.fa_rocm_varlen_workspace_bytes(C.byref(a), 256)
+    n3 = lib.fa_rocm_varlen_num_splits(C.byref(a), 256)
+    assert small > (302 * 32 * n3 * 129 * 4 if n3 > 1 else 0) + 2 * 3 * 4 * 32 * 128 * 2
+    a.batch, a.total_q, a.max_seqlen_q = 16, 527, 40     # blocks of similar length: nothing is routed
     assert lib.fa_rocm_varlen_workspace_bytes(C.byref(a), 256) < with_rows - partials + 527 * 32 * 64 * 129 * 4
     a.max_seqlen_q = 512
     a.nheads, a.nheads_k = 64, 1                       # 64 q heads per kv head: taller than the decode kernels take
