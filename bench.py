@@ -28,7 +28,7 @@ for _p in (os.path.join(ROOT, "flash-attention-npu_amd"), os.path.join(ROOT, "or
 HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E
 # HBM bytes per launch of the attention kernel from the FETCH_SIZE / WRITE_SIZE counter passes
 # (calibrated against a 1 GiB device copy); the workloads are seeded, so these are constants.
-MEASURED_TRAFFIC_BYTES = {"c2": 1241.7e6, "c3a": 2156.7e6, "c4": 399.7e6}
+MEASURED_TRAFFIC_BYTES = {"c2": 1241.6e6, "c3a": 2156.7e6, "c4": 399.7e6}
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
 
 
