@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the paged KV-cache attention path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2|c2_8k|c3a|c3b|c4|c5] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2|c2_8k|c3a|c3b|c4|c5|mixed] [--no-cpu]
 
 A step is one call of the hot path (append + rotary + attention + split combine for the decode
 configs, one varlen forward for c5) on synthetic inputs that are resident in HBM before the
@@ -401,6 +401,65 @@ def run_prefill(args):
     return res
 
 
+def run_mixed(args):
+    """Not a BASELINE.json config: a token-major serving step over a paged cache through the varlen call, 63 decode
+    rows (contexts uniform in [1024, 8191]) and one 1024-token prompt chunk at the end of a 16384-key context,
+    32 q / 8 kv heads, d = 128, bf16, causal.  The decode rows are bound by HBM, the chunk by the matrix pipe: the
+    line reports the time against the sum of the two roofs."""
+    import torch
+    from flash_attn_npu import flash_attn_npu as ops
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    hq, hk, d, page = 32, 8, 128, 256
+    g = torch.Generator(device="cpu").manual_seed(0)
+    lens_k = torch.randint(1024, 8192, (63,), generator=g).tolist() + [16384]
+    lens_q = [1] * 63 + [1024]
+    pages = [(n + page - 1) // page for n in lens_k]
+    pool = sum(pages)
+    table = torch.zeros(64, max(pages), dtype=torch.int32)
+    perm = torch.randperm(pool, generator=g).to(torch.int32)
+    o = 0
+    for b in range(64):
+        table[b, :pages[b]] = perm[o:o + pages[b]]
+        o += pages[b]
+    gd = torch.Generator(device=dev).manual_seed(1)
+
+    def rn(*shape):
+        return torch.randn(*shape, generator=gd, device=dev, dtype=torch.float32).to(torch.bfloat16)
+
+    sets = [(rn(pool, page, hk, d), rn(pool, page, hk, d)) for _ in range(2)]     # two pools alternated: cold caches
+    q = rn(sum(lens_q), hq, d)
+    out = torch.empty_like(q)
+    cu_q = torch.tensor([0] + torch.tensor(lens_q).cumsum(0).tolist(), dtype=torch.int32, device=dev)
+    used = torch.tensor(lens_k, dtype=torch.int32, device=dev)
+    table = table.to(dev)
+    scale = d ** -0.5
+
+    def step(i):
+        kc, vc = sets[i & 1]
+        return ops.varlen_fwd(q, kc, vc, out, cu_q, None, used, None, table, None, max(lens_q), max(lens_k), 0.0, scale,
+                              False, True, -1, -1, 0.0, False, None)
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i)
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / args.steps * 1e3
+    decode_bytes = sum(lens_k[:63]) * hk * d * 2 * 2
+    chunk_flops = 4.0 * 1024 * (16384 - 1024 + 1024 / 2.0) * d * hq
+    at_roofs_us = decode_bytes / (HBM_PEAK_GBPS * 1e9) * 1e6 + chunk_flops / (MFMA_BF16_PEAK_TFLOPS * 1e12) * 1e6
+    return {"metric": "mixed_batch_step_us", "value": ms * 1e3, "unit": "us", "n_gpus": 1, "steps": args.steps,
+            "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+            "dtype": "bf16", "data": "synthetic",
+            "config": {"workload": "mixed: token-major step over a paged cache, 63 decode rows (contexts U[1024,8191]) + one "
+                                   "1024-token chunk ending a 16384-key context, 32q/8kv d=128 page=256 causal",
+                       "decode_bytes": decode_bytes, "chunk_flops": chunk_flops},
+            "us_per_call": ms * 1e3, "us_at_both_roofs": at_roofs_us, "frac_of_both_roofs": at_roofs_us / (ms * 1e3)}
+
+
 def run_copy(args):
     """Plain device copy of known size (1 GiB read + 1 GiB written per step): the calibration
     workload for the FETCH_SIZE / WRITE_SIZE counters and a practical bandwidth yardstick."""
@@ -443,6 +502,8 @@ def main():
         out = run_decode(args, args.config)
     elif args.config == "c5":
         out = run_prefill(args)
+    elif args.config == "mixed":
+        out = run_mixed(args)
     elif args.config == "copy":
         out = run_copy(args)
     else:

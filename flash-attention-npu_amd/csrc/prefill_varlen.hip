@@ -513,23 +513,26 @@ __global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) prefill_kernel(const 
 // Merge of the key ranges of token-major query blocks over a paged cache: one wave per (token, head).
 // Partials are laid out (token, head, range): normalised fp32 rows and base-2 log-sum-exps, -inf for a
 // range in which the row saw nothing.  out = sum_r e^{lse_r - LSE} O_r, LSE = log sum_r e^{lse_r}.
-// grid: total_q * nheads workgroups of 64 threads.
+// grid: total_q * ceil(nheads / 4) workgroups of 256 threads: the four waves take four heads of one token,
+// so what depends on the token alone (its sequence, the cut of that sequence's keys) is found once per
+// workgroup and every early exit is taken by the whole workgroup.
 template <typename T, int D>
-__global__ void __launch_bounds__(64) prefill_combine_kernel(const PrefillParams p) {
-    const int tok = blockIdx.x / p.nheads;
-    const int head = blockIdx.x - tok * p.nheads;
-    const int lane = threadIdx.x;
-    // the sequence of this token: last b with cu_seqlens_q[b] <= tok (empty sequences repeat an offset)
-    int lo = 0, hi = p.batch;
-    while (hi - lo > 1) {
-        const int mid = (lo + hi) >> 1;
-        if (p.cu_seqlens_q[mid] <= tok) lo = mid; else hi = mid;
-    }
-    const int b = lo;
+__global__ void __launch_bounds__(256) prefill_combine_kernel(const PrefillParams p) {
+    const int head_groups = (p.nheads + 3) >> 2;
+    const int tok = blockIdx.x / head_groups;
+    const int head = (blockIdx.x - tok * head_groups) * 4 + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    // the sequence of this token: last b with cu_seqlens_q[b] <= tok (empty sequences repeat an offset), counted by
+    // the lanes side by side: one trip to memory where a bisection makes log2(batch) dependent ones
+    int below = 0;
+    for (int i = lane; i < p.batch; i += 64) below += (p.cu_seqlens_q[i] <= tok) ? 1 : 0;
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) below += __shfl_xor(below, d, 64);
+    const int b = max(below - 1, 0);
     const int Sq = p.cu_seqlens_q[b + 1] - p.cu_seqlens_q[b];
     const int Sk = min(p.seqused_k[b] + p.seqlen_k_add, p.max_blocks * p.page_size);
+    if (Sq >= 1 && Sq <= p.skip_short) return;   // computed by the decode kernels (the whole workgroup: one token)
     const int longest = block_max_keys(p.seqused_k, p.batch, p.seqlen_k_add);
-    if (Sq >= 1 && Sq <= p.skip_short) return;
     int wl = p.window_left, wr = p.window_right;
     int norm_m = p.window_norm_m;
     if (norm_m <= 0 && (wl >= 0 || wr >= 0)) norm_m = longest;
@@ -538,6 +541,7 @@ __global__ void __launch_bounds__(64) prefill_combine_kernel(const PrefillParams
     const int sk = adaptive_split_keys(min(longest, p.max_blocks * p.page_size), p.nsplits);
     const KeyRanges kr = key_ranges(Sq, Sk, wl, wr, sk, p.nsplits);
     if (kr.count == 1) return;   // the tile that computed this row wrote it
+    if (head >= p.nheads) return;
     const int64_t base = ((int64_t)tok * p.nheads + head) * p.nsplits;
 
     float mx = -INFINITY;
@@ -622,9 +626,9 @@ template <typename T> static hipError_t launch_prefill_t(const PrefillParams &p,
 }
 
 template <typename T> static hipError_t launch_prefill_combine_t(const PrefillParams &p, int headdim, hipStream_t stream) {
-    const int64_t wgs = (int64_t)p.total_q * p.nheads;
+    const int64_t wgs = (int64_t)p.total_q * ((p.nheads + 3) / 4);
     if (wgs <= 0 || wgs >= (1ll << 31)) return hipErrorInvalidValue;
-    dim3 grid((unsigned)wgs), block(64);
+    dim3 grid((unsigned)wgs), block(256);
     switch (headdim) {
         case 64: hipLaunchKernelGGL((prefill_combine_kernel<T, 64>), grid, block, 0, stream, p); break;
         case 128: hipLaunchKernelGGL((prefill_combine_kernel<T, 128>), grid, block, 0, stream, p); break;
