@@ -101,6 +101,8 @@ struct ShortBlocksParams {
     const float *lse_rows;         // (B, Hq, slots)
     int32_t *lens_rows;            // (B,): seqused_k of the short blocks' sequences, 0 for the others
     int32_t *live_rows;            // (B,): tokens of the short blocks (their real query positions), 0 for the others
+    int32_t *long_ids;             // (B,): the sequences with more than `slots` tokens, in batch order
+    int32_t *list_state;           // [0] = how many, [1..8] = 0 (block counters of the tiled launch that follows)
     int32_t batch, total_q, nheads, headdim, slots;
     int64_t q_stride_t, q_stride_h, o_stride_t, o_stride_h;
 };
@@ -121,6 +123,12 @@ struct PrefillParams {
     int32_t pack;                  // set by the launcher: 1, or group when tile rows are (query, head) pairs
     int32_t pack_short;            // set by the launcher: pack == 1, but a short query block packs its heads on its own
     int32_t skip_short;            // token-major q: sequences with 1 .. skip_short query tokens are computed elsewhere (0 = none)
+    // token-major q whose live sequences are listed on the device (with skip_short): the sequences with more than
+    // skip_short tokens, list_state[0] of them; list_state[1..8] are the per-XCD block counters of the launch, zero
+    // when it starts; list_wgs workgroups are launched (as many as the device holds)
+    const int32_t *long_ids;
+    int32_t *list_state;
+    int32_t list_wgs;
     int32_t num_mb, units8;        // set by the launcher: 128-row blocks per unit, units rounded up to 8
     int32_t seqlen_q_fixed, seqlen_k_add;   // kvcache layout: Sq per row, keys appended this call
     int32_t max_seqlen_q, total_q;

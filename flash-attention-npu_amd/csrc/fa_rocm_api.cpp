@@ -617,7 +617,7 @@ struct VarlenWorkspace {
     bool short_blocks;
     int slots;           // query positions per sequence in the decode launch over the short blocks
     bool decode_only;    // no block is longer than `slots`: the tiled kernel has nothing to do
-    size_t partials, q_rows, out_rows, lse_rows, lens_rows, live_rows, decode_ws, decode_ws_bytes, total;
+    size_t partials, q_rows, out_rows, lse_rows, lens_rows, live_rows, long_ids, list_state, decode_ws, decode_ws_bytes, total;
 };
 
 // The decode launch over the one-token blocks of a token-major batch: batch row b is sequence b, with
@@ -712,6 +712,10 @@ VarlenWorkspace varlen_workspace(const fa_varlen_args *a, int num_cus) {
         off += align256((size_t)a->batch * sizeof(int32_t));
         w.live_rows = off;
         off += align256((size_t)a->batch * sizeof(int32_t));
+        w.long_ids = off;
+        off += align256((size_t)a->batch * sizeof(int32_t));
+        w.list_state = off;
+        off += 256;
         const fa_kvcache_args k = short_blocks_call(a, nullptr, w);
         fa_split_plan plan;
         if (fa_rocm_plan_kvcache(&k, num_cus, &plan) != FA_OK) plan.workspace_bytes = 0;   // cannot fail after the check above
@@ -790,6 +794,10 @@ int fa_rocm_varlen_fwd(const fa_varlen_args *a, void *stream_) {
         sr.lse_rows = reinterpret_cast<float *>(base + w.lse_rows);
         sr.lens_rows = reinterpret_cast<int32_t *>(base + w.lens_rows);
         sr.live_rows = reinterpret_cast<int32_t *>(base + w.live_rows);
+        if (!w.decode_only) {
+            sr.long_ids = reinterpret_cast<int32_t *>(base + w.long_ids);
+            sr.list_state = reinterpret_cast<int32_t *>(base + w.list_state);
+        }
         sr.batch = a->batch;
         sr.total_q = a->total_q;
         sr.nheads = a->nheads;
@@ -855,6 +863,12 @@ int fa_rocm_varlen_fwd(const fa_varlen_args *a, void *stream_) {
         pp.lse_partial = pp.o_partial + (size_t)a->total_q * a->nheads * nsplits * a->headdim;
     }
     pp.skip_short = w.short_blocks ? w.slots : 0;
+    if (w.short_blocks && !w.decode_only) {
+        // the sequences left to the tiled kernel are listed on the device by the gather kernel
+        pp.long_ids = sr.long_ids;
+        pp.list_state = sr.list_state;
+        pp.list_wgs = cus * (a->headdim <= 128 ? 2 : 1);
+    }
     if (!w.decode_only) {
         const hipError_t e = fa::launch_prefill(pp, a->io_dtype, a->headdim, stream);
         if (e != hipSuccess) return fail(FA_ERR_LAUNCH, "prefill launch failed: %s", hipGetErrorString(e));

@@ -41,12 +41,14 @@ template <int D> struct PrefillCfg {
 };
 
 // EXT: packed heads and / or a split of the keys (p.pack, p.nsplits); without it both are compiled out
+// One 128-row block of one (sequence, key range, kv head, q head) of the launch: `bid` is its place in the
+// launch's order.  n_long < 0: the units are the launch's batch rows; otherwise they are the first n_long entries of
+// p.long_ids (the sequences the tiled kernel computes, listed on the device).
 template <typename T, int D, bool PAGED, bool SOFTCAP, bool EXT>
-__global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) prefill_kernel(const PrefillParams p) {
+__device__ __forceinline__ void prefill_block(const PrefillParams &p, const unsigned bid, const int n_long,
+                                              uint8_t (&s_k)[2][PrefillCfg<D>::kTileBytes],
+                                              uint8_t (&s_v)[2][PrefillCfg<D>::kVTileBytes]) {
     using Cfg = PrefillCfg<D>;
-    __shared__ __attribute__((aligned(16))) uint8_t s_k[2][Cfg::kTileBytes];
-    __shared__ __attribute__((aligned(16))) uint8_t s_v[2][Cfg::kVTileBytes];
-
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -60,27 +62,31 @@ __global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) prefill_kernel(const 
     // a unit's K/V meet in one L2.
     const int nsplits = EXT ? max(p.nsplits, 1) : 1;
     const int heads_per_unit = (EXT && p.pack > 1) ? 1 : p.group;
+    const bool listed = EXT && n_long >= 0;
+    const int n_units = (listed ? n_long : p.batch) * nsplits * p.nheads_k;
+    const int units8 = listed ? (n_units + 7) / 8 * 8 : p.units8;
     int mb, unit, head_in_unit;
     if (p.num_mb > 2) {
-        const int per_block = p.units8 * heads_per_unit;
-        mb = p.num_mb - 1 - (int)(blockIdx.x / per_block);
-        const int e = blockIdx.x % per_block;
+        const int per_block = units8 * heads_per_unit;
+        mb = p.num_mb - 1 - (int)(bid / per_block);
+        const int e = bid % per_block;
         unit = ((e >> 3) / heads_per_unit) * 8 + (e & 7);
         head_in_unit = (e >> 3) % heads_per_unit;
     } else {
         // one or two blocks per unit (short sequences, all equally light): a unit's blocks stay
         // neighbours in their XCD's queue, so its K/V are fetched into that L2 once
         const int per_unit = p.num_mb * heads_per_unit;
-        const int r = blockIdx.x >> 3;
-        unit = (r / per_unit) * 8 + (blockIdx.x & 7);
+        const int r = bid >> 3;
+        unit = (r / per_unit) * 8 + (bid & 7);
         head_in_unit = (r % per_unit) / p.num_mb;
         mb = p.num_mb - 1 - r % p.num_mb;
     }
-    if (unit >= p.batch * nsplits * p.nheads_k) return;
+    if (unit >= n_units) return;
     const int z = unit / p.nheads_k;
     const int hk = unit - z * p.nheads_k;
-    const int b = z / nsplits;
-    const int split = z - b * nsplits;
+    const int zb = z / nsplits;
+    const int split = z - zb * nsplits;
+    const int b = listed ? p.long_ids[zb] : zb;
 
     int q0, Sq, k0 = 0, Sk;
     if (p.cu_seqlens_q) {
@@ -510,6 +516,42 @@ __global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) prefill_kernel(const 
     }
 }
 
+template <typename T, int D, bool PAGED, bool SOFTCAP, bool EXT>
+__global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) prefill_kernel(const PrefillParams p) {
+    using Cfg = PrefillCfg<D>;
+    __shared__ __attribute__((aligned(16))) uint8_t s_k[2][Cfg::kTileBytes];
+    __shared__ __attribute__((aligned(16))) uint8_t s_v[2][Cfg::kVTileBytes];
+    prefill_block<T, D, PAGED, SOFTCAP, EXT>(p, blockIdx.x, -1, s_k, s_v);
+}
+
+// The same blocks for a launch whose live sequences are known on the device only (token-major batches whose
+// short blocks went to the decode kernels: p.long_ids, p.list_state[0] of them).  A grid sized for every batch
+// row would be mostly workgroups that find nothing to do, and dispatching those costs as much time as the live
+// ones' work once the batch has many decode rows.  Here as many workgroups as the device holds take blocks from
+// the ordered list until it ends: workgroup w (on XCD w % 8) takes the blocks congruent to w % 8, so that the heads
+// of a unit still meet in one L2, through one counter per XCD (p.list_state[1 + x], zeroed by the kernel that
+// wrote the list).  Every workgroup leaves when its counter passes the end of the list.
+template <typename T, int D, bool SOFTCAP>
+__global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) prefill_list_kernel(const PrefillParams p) {
+    using Cfg = PrefillCfg<D>;
+    __shared__ __attribute__((aligned(16))) uint8_t s_k[2][Cfg::kTileBytes];
+    __shared__ __attribute__((aligned(16))) uint8_t s_v[2][Cfg::kVTileBytes];
+    __shared__ int s_item;
+    const int n_long = p.list_state[0];
+    const int heads_per_unit = (p.pack > 1) ? 1 : p.group;
+    const int64_t units8 = ((int64_t)n_long * max(p.nsplits, 1) * p.nheads_k + 7) / 8 * 8;
+    const int64_t total = (int64_t)p.num_mb * units8 * heads_per_unit;     // a multiple of 8
+    const int x = blockIdx.x & 7;
+    for (;;) {
+        __syncthreads();   // the last block's LDS tiles and s_item are free
+        if (threadIdx.x == 0) s_item = atomicAdd(&p.list_state[1 + x], 1);
+        __syncthreads();
+        const int64_t bid = (int64_t)s_item * 8 + x;
+        if (bid >= total) break;
+        prefill_block<T, D, true, SOFTCAP, true>(p, (unsigned)bid, n_long, s_k, s_v);
+    }
+}
+
 // Merge of the key ranges of token-major query blocks over a paged cache: one wave per (token, head).
 // Partials are laid out (token, head, range): normalised fp32 rows and base-2 log-sum-exps, -inf for a
 // range in which the row saw nothing.  out = sum_r e^{lse_r - LSE} O_r, LSE = log sum_r e^{lse_r}.
@@ -602,6 +644,16 @@ template <typename T, int D> static hipError_t launch_prefill_d(const PrefillPar
     const bool paged = p.block_table != nullptr;
     p.pack_short = p.cu_seqlens_q ? prefill_pack_short(p.group, p.max_seqlen_q, p.total_q, p.batch) : 0;
     const bool ext = p.pack > 1 || p.nsplits > 1 || p.pack_short || p.skip_short > 0;
+    if (p.long_ids) {
+        // live sequences listed on the device: workgroups that stay and take blocks from the list
+        if (!paged || !p.list_state || p.list_wgs <= 0 || !p.cu_seqlens_q) return hipErrorInvalidValue;
+        dim3 lgrid((unsigned)std::min<int64_t>(p.list_wgs, wgs));
+        if (softcap)
+            hipLaunchKernelGGL((prefill_list_kernel<T, D, true>), lgrid, block, 0, stream, p);
+        else
+            hipLaunchKernelGGL((prefill_list_kernel<T, D, false>), lgrid, block, 0, stream, p);
+        return hipGetLastError();
+    }
     auto launch = [&](auto paged_c, auto softcap_c, auto ext_c) {
         hipLaunchKernelGGL((prefill_kernel<T, D, decltype(paged_c)::value, decltype(softcap_c)::value, decltype(ext_c)::value>),
                            grid, block, 0, stream, p);

@@ -26,6 +26,26 @@ __global__ void __launch_bounds__(256) gather_short_blocks_kernel(const ShortBlo
         p.lens_rows[b] = is_short ? p.seqused_k[b] : 0;
         p.live_rows[b] = is_short ? n : 0;
     }
+    if (b == 0 && p.long_ids) {
+        // the sequences left to the tiled kernel, in batch order: flags counted wave by wave, 256 sequences a pass
+        __shared__ int s_wave[4];
+        int done = 0;
+        for (int base = 0; base < p.batch; base += 256) {
+            const int i = base + threadIdx.x;
+            const bool is_long = i < p.batch && p.cu_seqlens_q[i + 1] - p.cu_seqlens_q[i] > p.slots;
+            const uint64_t mask = __ballot(is_long);
+            const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+            if (lane == 0) s_wave[wave] = __popcll(mask);
+            __syncthreads();
+            int before = done;
+            for (int w = 0; w < wave; ++w) before += s_wave[w];
+            if (is_long) p.long_ids[before + __popcll(mask & ((1ull << lane) - 1))] = i;
+            done += s_wave[0] + s_wave[1] + s_wave[2] + s_wave[3];
+            __syncthreads();
+        }
+        if (threadIdx.x == 0) p.list_state[0] = done;
+        if (threadIdx.x >= 1 && threadIdx.x <= 8) p.list_state[threadIdx.x] = 0;
+    }
     const int pieces_per_head = p.headdim / 8;
     const int pieces_per_token = p.nheads * pieces_per_head;
     const int pad = is_short ? p.slots - n : p.slots;
