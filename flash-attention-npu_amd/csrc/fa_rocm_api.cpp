@@ -8,6 +8,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <atomic>
 #include <climits>
 #include <cmath>
 #include <cstdarg>
@@ -576,6 +577,65 @@ static int fwd_kvcache_impl(const fa_kvcache_args *a, void *stream_, void *const
     }
     mark(3);
     return FA_OK;
+}
+
+// ---- the kvcache call for callers that cannot allocate: the split workspace is a static device array.
+// Every GPU the library runs on holds its own copy of the array, at its own address, until the process
+// ends; the name below is only a host-side handle, the address comes from hipGetSymbolAddress.
+}  // extern "C"
+
+namespace {
+static __device__ __align__(256) unsigned char scratch[FA_ROCM_STATIC_SCRATCH_BYTES];
+constexpr int kMaxDevices = 64;
+std::atomic<void *> g_scratch_ptr[kMaxDevices];   // device address of `scratch`, per device
+
+// Device address of the current device's copy of `scratch`; looked up on the first call on that device
+// (a symbol query: it allocates nothing, but it must not run while a stream is being captured).
+int static_scratch(void **ptr_out) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
+        return fail(FA_ERR_LAUNCH, "no current HIP device (or a device index beyond %d)", kMaxDevices - 1);
+    void *ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!ptr) {
+        const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr)
+            return fail(FA_ERR_LAUNCH, "hipGetSymbolAddress(scratch) failed on device %d: %s", dev, hipGetErrorString(e));
+        g_scratch_ptr[dev].store(ptr, std::memory_order_release);   // two racing threads store the same address
+    }
+    *ptr_out = ptr;
+    return FA_OK;
+}
+}  // namespace
+
+extern "C" {
+
+int fa_rocm_fwd_kvcache_static(const fa_kvcache_args *args, void *stream) {
+    const int rc = fa_rocm_kvcache_validate(args);
+    if (rc != FA_OK) return rc;
+    int cus = device_cus();
+    if (cus <= 0) cus = 256;
+    fa_split_plan plan;
+    const int rp = fa_rocm_plan_kvcache(args, cus, &plan);
+    if (rp != FA_OK) return rp;
+    if (plan.workspace_bytes > (size_t)FA_ROCM_STATIC_SCRATCH_BYTES)
+        return fail(FA_ERR_WORKSPACE,
+                    "the call needs a workspace of %zu bytes, the static scratch of fa_rocm_fwd_kvcache_static holds %zu: "
+                    "use fa_rocm_fwd_kvcache with a caller-owned workspace",
+                    plan.workspace_bytes, (size_t)FA_ROCM_STATIC_SCRATCH_BYTES);
+    fa_kvcache_args a = *args;
+    a.workspace = nullptr;
+    a.workspace_bytes = 0;
+    if (plan.workspace_bytes > 0) {
+        void *ptr = nullptr;
+        const int rs = static_scratch(&ptr);
+        if (rs != FA_OK) return rs;
+        // Nothing in the scratch has to start at zero: every partial slot a launch merges was written by
+        // that launch (the kernels and the combine derive the same partition), so the contents the last
+        // call left are never read.
+        a.workspace = ptr;
+        a.workspace_bytes = FA_ROCM_STATIC_SCRATCH_BYTES;
+    }
+    return fwd_kvcache_impl(&a, stream, nullptr);
 }
 
 int fa_rocm_varlen_validate(const fa_varlen_args *a) {

@@ -71,6 +71,7 @@ EXPORTS = {
     "fa_rocm_varlen_num_splits": (C.c_int, [C.POINTER(VarlenArgs), C.c_int]),
     "fa_rocm_varlen_workspace_bytes": (_sz, [C.POINTER(VarlenArgs), C.c_int]),
     "fa_rocm_append_kv": (C.c_int, [C.POINTER(KvcacheArgs), _vp]),
+    "fa_rocm_fwd_kvcache_static": (C.c_int, [C.POINTER(KvcacheArgs), _vp]),
 }
 
 _lib: Optional[C.CDLL] = None

@@ -225,6 +225,25 @@ size_t fa_rocm_varlen_workspace_bytes(const fa_varlen_args *args, int num_cus);
  */
 int fa_rocm_append_kv(const fa_kvcache_args *args, void *stream);
 
+/*
+ * fa_rocm_fwd_kvcache for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference, whose
+ * host allocates its workspace on every call (csrc/ascend910/flash_attn_npu/flash_api.cpp:552-567).
+ * Same arguments and results as fa_rocm_fwd_kvcache, except that args->workspace / workspace_bytes are
+ * ignored: the fp32 split partials go to a static device array of FA_ROCM_STATIC_SCRATCH_BYTES that the
+ * library holds on every GPU it runs on until the process ends.  The call allocates and frees nothing.
+ * A call whose plan (fa_rocm_plan_kvcache) needs more than that returns FA_ERR_WORKSPACE and enqueues
+ * nothing (36 MiB holds the partials of every bf16 / fp16 decode launch, i.e. any query block of up to 32
+ * rows = seqlen_q * nheads / nheads_k; the int8 latent kernel's partials at 128 query heads do not fit, and a
+ * taller block over few long sequences may not).
+ * All calls on one GPU share that GPU's array: two such calls that overlap in time on one device (two
+ * streams, two host threads) race on it; calls ordered on one stream do not.  The first call on a
+ * device looks the array's address up (a symbol query) and must not be made while a stream is being
+ * captured; later calls may.
+ */
+#define FA_ROCM_STATIC_SCRATCH_BYTES (36u << 20)
+int fa_rocm_fwd_kvcache_static(const fa_kvcache_args *args, void *stream);
+
 #ifdef __cplusplus
 }
 #endif
