@@ -171,6 +171,7 @@ template <typename T, int DV, typename SlotFn>
 __device__ __forceinline__ void combine_row_wave(const DecodeParams &p, int b, int kvh, int row, int ns, SlotFn slot_of) {
     constexpr int CPL = DV / 64;   // columns per lane (2, 4 or 8)
     static_assert(CPL == 1 || CPL == 2 || CPL == 4 || CPL == 8, "column split");
+    if (row_id(p, kvh, row).head >= p.nheads) return;   // a row of the latent kernel's last, partly empty head group
     const int lane = threadIdx.x & 63;
     float mx = -INFINITY;
     for (int s = lane; s < ns; s += 64) mx = fmaxf(mx, p.lse_partial[slot_of(s) * p.rows + row]);
@@ -211,6 +212,7 @@ template <int DV> __device__ __forceinline__ void init_empty_unit(const DecodePa
         const int piece = idx - row * (DV / 8);
         const RowId rid = row_id(p, kvh, row);
         const int qi = rid.qi, head = rid.head;
+        if (head >= p.nheads) continue;
         uint16_t *dst = reinterpret_cast<uint16_t *>(p.out) + (int64_t)b * p.o_stride_b + (int64_t)qi * p.o_stride_s +
                         (int64_t)head * p.o_stride_h + piece * 8;
         store16(dst, u32x4_t{0, 0, 0, 0});

@@ -1,47 +1,62 @@
 // Latent-attention (MLA) decode over an int8 paged cache with per-token fp32 scales, gfx950.
 //
-// Layout: one latent kv head, 576 key dims, V = the first 512 of them (v_cache aliases k_cache);
-// 128 q heads (any multiple of 64), any seqlen_q (each query token is its own set of units).  The reference has no quantised path
-// (dtypes are limited to fp16/bf16 at csrc/ascend910/flash_attn_npu/flash_api.cpp:386-388 and
-// descales are rejected at flash_attn_npu_3/flash_api.cpp:153-155); the attention arithmetic is
-// the same as the bf16 decode kernel's (mha_fwd_kvcache.cpp:632-969 in the reference) applied to
-// K^ = code * scale[token].
+// Layout: one latent kv head, 576 key dims, V = the first 512 of them (v_cache aliases k_cache); any number of q
+// heads, any seqlen_q (each query token is its own set of units).  The reference has no quantised path (dtypes are
+// limited to fp16/bf16 at csrc/ascend910/flash_attn_npu/flash_api.cpp:386-388 and descales are rejected at
+// flash_attn_npu_3/flash_api.cpp:153-155); the attention arithmetic is the same as the bf16 decode kernel's
+// (mha_fwd_kvcache.cpp:632-969 in the reference) applied to K^ = code * scale[token].
 //
-// A work unit is (batch row, 64-head half).  The 512-thread workgroup streams its share of the
-// unit list (same balanced partition as the bf16 decode kernel): every 32-key chunk is fetched
-// once as int8 with 8-byte loads, widened to the 16-bit type on the way into LDS (a code is an
-// integer of magnitude <= 127, exact in bf16 and fp16) and shared by the eight waves, which come
-// in two kinds, one of each per SIMD:
-//   score waves  (0-3): they also stage the cache (loads two chunks ahead, the widening of chunk
-//            c+2 interleaved with the products of chunk c+1); wave w owns heads 16w..16w+15 with
-//            Q^T resident in registers: S^T = K Q^T over the chunk, per-token scale folded into
-//            the scores, online softmax local to the lane column; P, the rescale factor and a
-//            "new maximum" flag go to LDS;
-//   output waves (4-7): wave w owns a 128-column slice of V for all 64 heads: O^T += V^T P^T, each
-//            transposed V operand (rows read whole from the same LDS tile, v_perm in registers)
-//            feeding four MFMAs; the V side of the dequantisation is folded into P.
-// The kinds run one chunk apart (scores of chunk c+1 beside the output of chunk c), so the
-// LDS-heavy score products, the conversions and the output products of one SIMD overlap instead
-// of taking turns, with one barrier per chunk.
+// A work unit is (batch row, query token, group of 128 heads): ALL heads of a token share one pass over the cache,
+// so every 32-key chunk is fetched from HBM once and widened to the 16-bit type once (a code is an integer of
+// magnitude <= 127, exact in bf16 and fp16).  One 256-thread workgroup per compute unit, one wave per SIMD with the
+// whole register file (512 registers): the fp32 accumulators of 128 heads x 512 columns fill the 256 accumulation
+// registers of every wave, Q^T most of the ordinary ones.
+//
+//   scores  wave w owns heads 32w..32w+31 with Q^T resident (29 operands of the 32x32x16 MFMA in registers, the last
+//           7 in LDS): S^T[32 keys x 32 heads] = K Q^T, the key-side scale folded into the exponent, online softmax local
+//           to the lane column (one exchange between the two half-waves per chunk).  P^T, with the V-side scale folded
+//           in and rounded to the 16-bit type, goes to LDS in MFMA operand order.
+//   output  wave w owns columns 128w..128w+127 of V for ALL 128 heads: O^T[cols x heads] += V^T P^T; every
+//           transposed V operand (ds_read_b64_tr_b16 from the same LDS tile) feeds four MFMAs, one per head group.
+//   staging all four waves: the loads of chunk c+2 leave (global -> registers) piece by piece while chunk c+1 is
+//           widened into LDS beside the score products of chunk c, and the softmax of chunk c stands beside the
+//           output products of chunk c-1; one workgroup barrier per chunk, three LDS tiles.
+// Measured on this machine, vector and matrix instructions of one wave overlap little (a step costs about the sum
+// of the two), so what counts is the instruction count: per chunk and wave 68 MFMAs, ~300 vector instructions.
+//
+// The exponent reference of a head moves only when a chunk's maximum passes it by more than kLazy (the lazy rescale of
+// the reference's fourth-generation kernels, csrc/ascend910/flash_attn_npu_4/online_softmax.hpp:633-666): rescaling
+// the accumulators is then rare, and all of it (masks, the first chunk, a moved reference) lives on a slow path the
+// common chunk never enters.  The weight a key really gets is round16(P * v_scale) / v_scale; the output is divided
+// by the sum of THOSE weights, so it stays a convex combination of the dequantised rows whatever the reference is
+// (a row that sees one key returns that key); the LSE uses the unrounded P.
+#include <utility>
+
 #include "decode_common.h"
 
 namespace fa {
 
 constexpr int kMlaDqk = 576;
 constexpr int kMlaDv = 512;
-constexpr int kMlaThreads = 512;
-// LDS key rows are unpadded; the 16-byte units of a row are XOR-swizzled with (row & 7) inside
-// their aligned groups of eight.  The LDS serves 16-byte reads eight lanes at a time and two
-// neighbouring groups of eight lanes overlap in time, so any 16 consecutive lanes (from a
-// multiple of 8) must hit 16 different units modulo 256 bytes: rows are 1152 = 4.5 * 256 bytes,
-// so odd and even rows sit half a bank cycle apart and the swizzle spreads rows of equal parity.
-constexpr int kMlaRowBytes = kMlaDqk * 2;                // 1152
+constexpr int kMlaThreads = 256;
+constexpr int kMlaUnitHeads = 128;                       // heads of a unit, 32 per wave
+constexpr int kMlaRowBytes = kMlaDqk * 2;                // 1152: a widened key row
 constexpr int kMlaTileBytes = kChunk * kMlaRowBytes;     // 36864
-constexpr int kMlaPiecesPerRow = kMlaDqk / 8;            // 72 8-byte int8 pieces per key = 16-byte units once widened
-constexpr int kMlaStagers = 256;                         // threads of the score waves
-constexpr int kMlaRounds = kChunk * kMlaPiecesPerRow / kMlaStagers;   // 9 pieces per staging thread per chunk
-constexpr int kMlaHeadsPerUnit = 64;
-static_assert(kChunk * kMlaPiecesPerRow == kMlaRounds * kMlaStagers, "chunk must split evenly over the staging threads");
+constexpr int kMlaKSteps = kMlaDqk / 16;                 // 36 k-steps of the score product
+constexpr int kMlaRounds = kMlaDqk / 64;                 // 9 eight-code pieces per staging thread and chunk
+constexpr int kMlaQLds = 7;                              // Q^T operands of the last k-steps wait in LDS, not in registers
+constexpr int kMlaQReg = kMlaKSteps - kMlaQLds;
+static_assert(kMlaThreads / 8 == kChunk, "eight staging threads per key row");
+
+// LDS key rows are unpadded (1152 B = 4.5 x 256 B: odd and even rows sit half a bank cycle apart); the 16-byte units
+// of a row are XOR-swizzled inside their aligned groups of eight with the bit-reversed (row / 2) % 8.  The LDS serves
+// 16 lanes per cycle, so: the 16 rows x same unit of a score operand read land on 16 different units modulo 256 B
+// (eight rows of equal parity get eight different swizzles), and the 4 rows x 4 units of a transposed read as well
+// (rows r and r + 2 differ in swizzle bit 2, i.e. in which aligned group of four units they use).
+__device__ __forceinline__ int mla_swz(int row) {
+    const int t = row >> 1;
+    return ((t & 1) << 2) | (t & 2) | ((t >> 2) & 1);
+}
 
 struct __attribute__((aligned(4))) MlaCodes8 { uint32_t w[2]; };
 
@@ -55,368 +70,570 @@ template <typename T> __device__ __forceinline__ void widen4(uint32_t w, uint32_
     hi = pack2<T>(f2, f3);
 }
 
+template <typename T> struct MlaLazy;
+// P <= 2^kLazy before the V-side scale is folded in: bf16 has the range; fp16 (max 65504) keeps 2^4 x scale inside it
+template <> struct MlaLazy<BF16> { static constexpr float kLog2 = 8.f, kMax = 256.f; };
+template <> struct MlaLazy<FP16> { static constexpr float kLog2 = 4.f, kMax = 16.f; };
+
+// ---- the output accumulators live in the 256 accumulation registers a0..a255, addressed by number.
+// The compiler's register allocator keeps loop-carried vector values in ordinary registers and copies them in and out
+// of every hand-written matrix instruction; 128 heads x 512 columns only fit if they never leave the accumulation
+// file.  So these registers are not C++ values at all: every instruction that touches them is written out with the
+// register number in its text, and lists all 256 as clobbered, which (a) makes the kernel's register count include
+// them and (b) keeps the compiler from parking anything of its own there across these instructions.
+#define MLA_AD(p, d) "a" p #d
+#define MLA_ATEN(p) MLA_AD(p, 0), MLA_AD(p, 1), MLA_AD(p, 2), MLA_AD(p, 3), MLA_AD(p, 4), MLA_AD(p, 5), MLA_AD(p, 6), MLA_AD(p, 7), MLA_AD(p, 8), MLA_AD(p, 9)
+#define MLA_ALL_ACC                                                                                                          \
+    MLA_ATEN(""), MLA_ATEN("1"), MLA_ATEN("2"), MLA_ATEN("3"), MLA_ATEN("4"), MLA_ATEN("5"), MLA_ATEN("6"), MLA_ATEN("7"),        \
+        MLA_ATEN("8"), MLA_ATEN("9"), MLA_ATEN("10"), MLA_ATEN("11"), MLA_ATEN("12"), MLA_ATEN("13"), MLA_ATEN("14"), MLA_ATEN("15"), \
+        MLA_ATEN("16"), MLA_ATEN("17"), MLA_ATEN("18"), MLA_ATEN("19"), MLA_ATEN("20"), MLA_ATEN("21"), MLA_ATEN("22"),          \
+        MLA_ATEN("23"), MLA_ATEN("24"), MLA_AD("25", 0), MLA_AD("25", 1), MLA_AD("25", 2), MLA_AD("25", 3), MLA_AD("25", 4),      \
+        MLA_AD("25", 5)
+
+template <int I, int N, typename F> __device__ __forceinline__ void static_for(F &&f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<I + 1, N>(f);
+    }
+}
+
+// a[BASE : BASE+15] += A * B (32x32x16).  Register numbers are printed digit by digit: an immediate of 64 or more
+// would come out in hexadecimal.
+template <typename T, int BASE> __device__ __forceinline__ void acc_mfma(const u32x4_t &a, const u32x4_t &b) {
+    if constexpr (BASE == 0) {
+        if constexpr (__is_same(T, BF16))
+            asm volatile("v_mfma_f32_32x32x16_bf16 a[0:15], %0, %1, a[0:15]" ::"v"(a), "v"(b) : MLA_ALL_ACC);
+        else
+            asm volatile("v_mfma_f32_32x32x16_f16 a[0:15], %0, %1, a[0:15]" ::"v"(a), "v"(b) : MLA_ALL_ACC);
+    } else {
+        if constexpr (__is_same(T, BF16))
+            asm volatile("v_mfma_f32_32x32x16_bf16 a[%2%3:%4%5], %0, %1, a[%2%3:%4%5]" ::"v"(a), "v"(b), "n"(BASE / 10),
+                         "n"(BASE % 10), "n"((BASE + 15) / 10), "n"((BASE + 15) % 10)
+                         : MLA_ALL_ACC);
+        else
+            asm volatile("v_mfma_f32_32x32x16_f16 a[%2%3:%4%5], %0, %1, a[%2%3:%4%5]" ::"v"(a), "v"(b), "n"(BASE / 10),
+                         "n"(BASE % 10), "n"((BASE + 15) / 10), "n"((BASE + 15) % 10)
+                         : MLA_ALL_ACC);
+    }
+}
+template <int R> __device__ __forceinline__ void acc_zero() {
+    if constexpr (R < 10)
+        asm volatile("v_accvgpr_write_b32 a%0, 0" ::"n"(R) : MLA_ALL_ACC);
+    else
+        asm volatile("v_accvgpr_write_b32 a%0%1, 0" ::"n"(R / 10), "n"(R % 10) : MLA_ALL_ACC);
+}
+template <int R> __device__ __forceinline__ float acc_read() {
+    float v;
+    if constexpr (R < 10)
+        asm volatile("v_accvgpr_read_b32 %0, a%1" : "=v"(v) : "n"(R) : MLA_ALL_ACC);
+    else
+        asm volatile("v_accvgpr_read_b32 %0, a%1%2" : "=v"(v) : "n"(R / 10), "n"(R % 10) : MLA_ALL_ACC);
+    return v;
+}
+template <int R> __device__ __forceinline__ void acc_scale(float f) {
+    float t;
+    if constexpr (R < 10)
+        asm volatile("v_accvgpr_read_b32 %0, a%2\n\tv_mul_f32 %0, %0, %1\n\tv_accvgpr_write_b32 a%2, %0" : "=&v"(t) : "v"(f), "n"(R) : MLA_ALL_ACC);
+    else
+        asm volatile("v_accvgpr_read_b32 %0, a%2%3\n\tv_mul_f32 %0, %0, %1\n\tv_accvgpr_write_b32 a%2%3, %0"
+                     : "=&v"(t)
+                     : "v"(f), "n"(R / 10), "n"(R % 10)
+                     : MLA_ALL_ACC);
+}
+// wait states between a matrix instruction and the first vector instruction that reads or writes its result
+// registers (and back): the hazards the compiler would cover for instructions it knows
+__device__ __forceinline__ void mfma_settle() { asm volatile("s_nop 15\n\ts_nop 3" ::: "memory", MLA_ALL_ACC); }
+
 struct MlaShared {
-    __attribute__((aligned(16))) uint8_t k[3][kMlaTileBytes];   // widened key tiles: scores, output, being filled
-    __attribute__((aligned(16))) float ks[3][kChunk];            // per-token scales, K side
-    __attribute__((aligned(16))) float vs[3][kChunk];            // per-token scales, V side
-    __attribute__((aligned(16))) float vsi[3][kChunk];           // their inverses (0 for a zero scale)
-    __attribute__((aligned(16))) u32x4_t pk[2][4][64];           // P^T operands of the four head groups, two chunks
-    float alpha[2][4][16];                                       // accumulator rescale per head
-    __attribute__((aligned(4))) uint8_t bump[2][4];              // head group saw a new maximum
-    float l[4][16];                                              // final sum per head
+    __attribute__((aligned(16))) uint8_t k[3][kMlaTileBytes];   // widened key tiles
+    struct __attribute__((aligned(16))) Scales {                 // per-token scales of a tile, side by side: one LDS base address
+        float ksl[kChunk];                                       // key-side scale x softmax scale (log2 units)
+        float vs[kChunk];                                        // V-side scale
+        float vsi[kChunk];                                       // its inverse (0 for a zero scale)
+        uint16_t vsi_hi[kChunk];                                 // the inverse as two bf16 terms (hi + lo), for v_dot2_f32_bf16
+        uint16_t vsi_lo[kChunk];
+    } sc[3];
+    __attribute__((aligned(16))) u32x4_t pk[2][4][2][64];        // P^T operands: [chunk parity][head group][k-step][lane]
+    float alpha[2][kMlaUnitHeads];                               // accumulator rescale per head (slow path only)
+    __attribute__((aligned(16))) int32_t moved[2][4];                                         // head group moved its reference in this chunk
+    float l[kMlaUnitHeads];                                      // final normaliser per head
+    __attribute__((aligned(16))) u32x4_t q[4][kMlaQLds][64];     // Q^T operands of the last k-steps: [wave][k-step][lane]
 };
 
 template <typename T, bool SOFTCAP>
 __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, const int unit, const UnitRange &ur,
                                           const int range_lo, const int range_hi, const bool write_final,
                                           const int64_t slot, MlaShared &sh) {
-    // unit = (query token qi, 64-head group `half`); the chunks walked are those of the whole query
-    // block, the keys this token may not see (causal / window bounds of its own row) are masked
+    // unit = (query token qi, 128-head group hgrp); the chunks walked are those of the whole query block, the keys
+    // this token may not see (causal / window bounds of its own row) are masked
     const int qi = unit / p.units_per_token;
-    const int half = unit - qi * p.units_per_token;
+    const int hgrp = unit - qi * p.units_per_token;
     const int row_off = ur.Lk - p.seqlen_q + qi;                       // key aligned with this query token
     const int mask_lo = max(range_lo, ur.wl >= 0 ? row_off - ur.wl : 0);
     const int mask_hi = min(range_hi, ur.wr >= 0 ? row_off + ur.wr + 1 : ur.Lk);
-    constexpr int KSTEPS = kMlaDqk / 32;   // 18
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int role = wave >> 2;   // 0: scores, 1: output
-    const int w4 = wave & 3;      // head group (scores) or 128-column slice (output)
+    const int lane = tid & 63;
+    const int ln = lane & 31;     // MFMA column: head of the wave's group (scores), head of a group (output)
+    const int lh = lane >> 5;     // half-wave
     const int Lk = ur.Lk;
+    const int c_begin = range_lo / kChunk;
+    const int nch = (range_hi + kChunk - 1) / kChunk - c_begin;   // chunks of this piece (>= 1)
 
     const int8_t *kc = reinterpret_cast<const int8_t *>(p.k_cache);
     const int32_t *bt_row = p.block_table + (int64_t)b * p.bt_stride_b;
-    const int c_begin = range_lo / kChunk;
-    const int n = (range_hi + kChunk - 1) / kChunk - c_begin;   // chunks of this piece
 
-    // Step j of a piece (j = 0 .. n + 1): chunk j is widened into tile j % 3 and chunk j + 2 loaded;
-    // the score waves work on chunk j - 1 (tile (j + 2) % 3), the output waves on chunk j - 2
-    // (tile (j + 1) % 3); one barrier ends the step.
-    if (role == 0) {
-        // =========================== score waves ===========================================
-        const int lane0 = tid & 63;
-        const int head = half * kMlaHeadsPerUnit + w4 * 16 + (lane0 & 15);   // head of this lane column
-        // Q^T operand: lane (lq, ln) holds head `head` of query token qi, elements t*32 + lq*8 .. +7
-        u32x4_t qreg[KSTEPS];
-        {
-            const uint16_t *src = reinterpret_cast<const uint16_t *>(p.q) + (int64_t)b * p.q_stride_b +
-                                  (int64_t)qi * p.q_stride_s + (int64_t)head * p.q_stride_h + (lane0 >> 4) * 8;
-#pragma unroll
-            for (int t = 0; t < KSTEPS; ++t) qreg[t] = load16(src + t * 32);
-        }
-        // ---- staging: int8 rows -> registers -> widened LDS tile.  Chunk j of the piece is loaded
-        //      into register set j & 1 two steps before it is widened.  Thread -> (key row, 8-byte
-        //      column): 8 threads per row, nine pieces 64 bytes apart each, so one address per chunk
-        //      serves all loads and one LDS address all stores (the swizzle stays inside a group of
-        //      eight units, the pieces of a thread are eight units apart).  Past the end of the piece the last
-        //      chunk is named again: every step issues the same loads, so the compiler counts the
-        //      loads in flight instead of waiting for all of them.  Page ids are loaded one step
-        //      before the tile loads that use them and ahead of that step's tile loads, so waiting
-        //      for a page id never waits for younger tile loads.  The thread index comes in as an
-        //      argument: the step loop passes a copy the compiler cannot see through, so the few
-        //      address terms are recomputed per chunk instead of held in registers.
-        static_assert(kMlaStagers / 8 == kChunk && kMlaRounds * 8 == kMlaPiecesPerRow, "thread map of the staging");
-        MlaCodes8 st[2][kMlaRounds];
-        float st_ks[2] = {0.f, 0.f}, st_vs[2] = {0.f, 0.f};
-        auto fetch_blk = [&](int j) -> int {
-            int page = ((c_begin + min(j, n - 1)) * kChunk) / p.page_size;
-            page = min(page, p.max_blocks - 1);
-            return min(max(bt_row[page], 0), p.num_blocks - 1);
-        };
-        auto fetch = [&](int j_any, int blk, int set, int th) {
-            const int j = min(j_any, n - 1);
-            const int t_row = th >> 3;
-            const int t_sub = th & 7;
-            const int key0 = (c_begin + j) * kChunk;
-            const int inpage0 = key0 % p.page_size;
-            const int last = Lk - 1 - key0;
-            // wave-uniform 64-bit base + 32-bit per-thread offset
-            const int8_t *src = kc + (int64_t)blk * p.k_stride_block + (int64_t)inpage0 * p.k_stride_row;
-            const uint32_t voff = (uint32_t)min(t_row, last) * (uint32_t)p.k_stride_row + t_sub * 8;
-#pragma unroll
-            for (int i = 0; i < kMlaRounds; ++i) st[set][i] = *reinterpret_cast<const MlaCodes8 *>(src + voff + i * 64);
-            const int64_t so = (int64_t)blk * p.ks_stride_block + (int64_t)inpage0 * p.ks_stride_row;
-            const uint32_t soff = (uint32_t)min(th & (kChunk - 1), last) * (uint32_t)p.ks_stride_row;
-            st_ks[set] = (p.k_scale + so)[soff];
-            st_vs[set] = (p.v_scale + so)[soff];
-        };
-        // piece i (0..8) of the staged chunk: eight codes -> eight 16-bit floats -> one LDS unit
-        auto widen_piece = [&](int tile, int set, int th, int i) {
-            const int row = th >> 3;
-            uint8_t *dst = &sh.k[tile][row * kMlaRowBytes + (((th & 7) ^ (row & 7)) << 4)];
-            u32x4_t w;
-            uint32_t lo, hi;
-            widen4<T>(st[set][i].w[0], lo, hi);
-            w[0] = lo, w[1] = hi;
-            widen4<T>(st[set][i].w[1], lo, hi);
-            w[2] = lo, w[3] = hi;
-            *reinterpret_cast<u32x4_t *>(dst + i * 128) = w;
-        };
-        auto stash_scales = [&](int tile, int set, int th) {
-            if (th < kChunk) {
-                sh.ks[tile][th] = st_ks[set];
-                sh.vs[tile][th] = st_vs[set];
-                sh.vsi[tile][th] = (st_vs[set] > 0.f) ? 1.f / st_vs[set] : 0.f;
-            }
-        };
-        int blk_next;
-        {
-            const int b0 = fetch_blk(0), b1 = fetch_blk(1);
-            blk_next = fetch_blk(2);
-            fetch(0, b0, 0, tid);
-            fetch(1, b1, 1, tid);
-        }
-        float m_run = -INFINITY, l_run = 0.f, l_norm = 0.f;
+    // page ids of the first two chunks: requested first, they come back while Q^T is loaded
+    const int blk_first = bt_row[min((c_begin * kChunk) / p.page_size, p.max_blocks - 1)];
+    const int blk_second = bt_row[min(((c_begin + min(1, nch - 1)) * kChunk) / p.page_size, p.max_blocks - 1)];
 
-        auto score_step = [&](const int j, const int set, const int tile_j) {
-            int th = tid;
-            asm volatile("" : "+v"(th));
-            const int lane = th & 63;
-            const int lq = lane >> 4;
-            const int ln = lane & 15;
-            const bool do_stash = j < n;
-            const bool do_score = j >= 1 && j <= n;
-            const int tile = (tile_j == 0) ? 2 : tile_j - 1;   // (j + 2) % 3: tile of the scores
-            float4_t s[2] = {float4_t{0.f, 0.f, 0.f, 0.f}, float4_t{0.f, 0.f, 0.f, 0.f}};
-            // per-token scales of the score chunk, read ahead of the products
-            float4 ks4[2], vs4[2], vi4[2];
+    // ---- Q^T operands: lane (ln, lh) holds head 32*wave + ln, dims 16t + 8lh .. +7 of k-step t
+    const int row_u = wave * 32 + ln;                                  // row of the unit
+    const int head = hgrp * kMlaUnitHeads + row_u;
+    u32x4_t qreg[kMlaQReg];
+    {
+        const uint16_t *src = reinterpret_cast<const uint16_t *>(p.q) + (int64_t)b * p.q_stride_b + (int64_t)qi * p.q_stride_s +
+                              (int64_t)min(head, p.nheads - 1) * p.q_stride_h + lh * 8;
 #pragma unroll
-            for (int tt = 0; tt < 2; ++tt) {
-                ks4[tt] = *reinterpret_cast<const float4 *>(&sh.ks[tile][tt * 16 + lq * 4]);
-                vs4[tt] = *reinterpret_cast<const float4 *>(&sh.vs[tile][tt * 16 + lq * 4]);
-                vi4[tt] = *reinterpret_cast<const float4 *>(&sh.vsi[tile][tt * 16 + lq * 4]);
-            }
-            if (do_score) {
-                // ---- S^T = K Q^T : two 16-key tiles x this wave's 16 heads; operand reads run kPf
-                //      k-steps ahead of the MFMAs that use them; one piece of the next-but-one chunk
-                //      is widened beside every other k-step (in the last score step that is the last chunk
-                //      once more, into a tile nobody reads: no branch inside the product loop)
-                constexpr int kPf = 8;
-                u32x4_t ka[KSTEPS][2];
-                // unit 4t + lq of rows ln and 16 + ln (same row & 7), swizzled: two lane offsets by parity of t
-                const uint8_t *k_rd = &sh.k[tile][ln * kMlaRowBytes];
-                const int k_off[2] = {(lq ^ (ln & 7)) << 4, ((4 + lq) ^ (ln & 7)) << 4};
-                auto read_k = [&](int t) {
-                    ka[t][0] = *reinterpret_cast<const u32x4_t *>(k_rd + k_off[t & 1] + (t >> 1) * 128);
-                    ka[t][1] = *reinterpret_cast<const u32x4_t *>(k_rd + 16 * kMlaRowBytes + k_off[t & 1] + (t >> 1) * 128);
-                };
+        for (int t = 0; t < kMlaQReg; ++t) qreg[t] = load16(src + t * 16);
 #pragma unroll
-                for (int t = 0; t < kPf; ++t) read_k(t);
-#pragma unroll
-                for (int t = 0; t < KSTEPS; ++t) {
-                    if (t + kPf < KSTEPS) read_k(t + kPf);
-                    s[0] = mfma16<T>(ka[t][0], qreg[t], s[0]);
-                    if (t & 1) widen_piece(tile_j, set, th, t >> 1);
-                    s[1] = mfma16<T>(ka[t][1], qreg[t], s[1]);
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-            } else if (do_stash) {
-#pragma unroll
-                for (int i = 0; i < kMlaRounds; ++i) widen_piece(tile_j, set, th, i);
-            }
-            if (do_stash) stash_scales(tile_j, set, th);
-            {
-                const int blk_after = fetch_blk(j + 3);
-                fetch(j + 2, blk_next, set, th);
-                blk_next = blk_after;
-            }
-            __builtin_amdgcn_sched_barrier(0);
-            if (do_score) {
-                const int c = c_begin + j - 1;
-                const int pb = set ^ 1;                              // (j - 1) & 1
-                // ---- softmax; register i of tile tt is key c*32 + tt*16 + lq*4 + i
-                const int key_base = c * kChunk + lq * 4;
-                float x[8], vsc[8], vin[8];
-                float mloc = -INFINITY;
-#pragma unroll
-                for (int tt = 0; tt < 2; ++tt) {
-                    const float ksv[4] = {ks4[tt].x, ks4[tt].y, ks4[tt].z, ks4[tt].w};
-                    const float vsv[4] = {vs4[tt].x, vs4[tt].y, vs4[tt].z, vs4[tt].w};
-                    const float viv[4] = {vi4[tt].x, vi4[tt].y, vi4[tt].z, vi4[tt].w};
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const int key = key_base + tt * 16 + i;
-                        float v = s[tt][i] * ksv[i];
-                        if constexpr (SOFTCAP) {
-                            const float e2 = __expf(2.f * v * p.softcap_pre);
-                            v = p.softcap_post * (1.f - 2.f / (e2 + 1.f));
-                        } else {
-                            v *= p.scale_log2;
-                        }
-                        v = (key >= mask_lo && key < mask_hi) ? v : -INFINITY;
-                        x[tt * 4 + i] = v;
-                        vsc[tt * 4 + i] = vsv[i];
-                        vin[tt * 4 + i] = viv[i];
-                        mloc = fmaxf(mloc, v);
-                    }
-                }
-                mloc = quad_rows_max(mloc);
-                const bool bump = mloc > m_run;
-                const float m_new = bump ? mloc : m_run;
-                const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-                const float alpha = bump ? fast_exp2(m_run - m_use) : 1.f;
-                m_run = m_new;
-                float psum = 0.f;
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const float pe = fast_exp2(x[e] - m_use);
-                    psum += pe;
-                    x[e] = pe * vsc[e];   // V side of the dequantisation folded into P
-                }
-                l_run = l_run * alpha + psum;
-                u32x4_t pk;
-                pk[0] = pack2<T>(x[0], x[1]);
-                pk[1] = pack2<T>(x[2], x[3]);
-                pk[2] = pack2<T>(x[4], x[5]);
-                pk[3] = pack2<T>(x[6], x[7]);
-                // The weight a key really gets is round16(P * v_scale) / v_scale = P (1 + eps), |eps| <= 2^-8 (bf16).
-                // The output is divided by the sum of THOSE weights, so that it stays a convex combination of
-                // the dequantised values (a row that sees one key returns that key exactly); the LSE keeps the
-                // sum of the unrounded P.
-                float pcorr = 0.f;
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const uint32_t w = pk[e >> 1];
-                    const float xr = to_float<T>((uint16_t)((e & 1) ? (w >> 16) : (w & 0xffffu)));
-                    pcorr = __builtin_fmaf(xr - x[e], vin[e], pcorr);
-                }
-                l_norm = l_norm * alpha + (psum + pcorr);
-                sh.pk[pb][w4][lane] = pk;
-                if (lq == 0) sh.alpha[pb][w4][ln] = alpha;
-                const int wave_bump = __any(bump) ? 1 : 0;
-                if (lane == 0) sh.bump[pb][w4] = (uint8_t)wave_bump;
-            }
-            __syncthreads();
-        };
-        int tile_j = 0;
-        for (int j = 0; j <= n + 1; j += 2) {
-            score_step(j, 0, tile_j);
-            tile_j = (tile_j == 2) ? 0 : tile_j + 1;
-            if (j + 1 <= n + 1) {
-                score_step(j + 1, 1, tile_j);
-                tile_j = (tile_j == 2) ? 0 : tile_j + 1;
-            }
-        }
+        for (int t = kMlaQReg; t < kMlaKSteps; ++t) sh.q[wave][t - kMlaQReg][lane] = load16(src + t * 16);   // wave-private
+    }
 
-        // ---- publish the sums, write the LSE
-        l_run = quad_rows_sum(l_run);
-        l_norm = quad_rows_sum(l_norm);
-        const int lane = tid & 63;
-        const int ln = lane & 15;
-        if ((lane >> 4) == 0) {
-            sh.l[w4][ln] = (l_run > 0.f) ? l_norm : 0.f;
-            const int row = w4 * 16 + ln;
-            if (write_final)
-                p.lse[((int64_t)b * p.nheads + head) * p.seqlen_q + qi] = (l_run > 0.f) ? (m_run + fast_log2(l_run)) * kLn2 : INFINITY;
+    // ---- staging: thread -> (key row tid / 8, eight-code pieces tid % 8 + 8i): one address per chunk serves all
+    //      loads and one LDS address all stores.  Rows past the last key of the sequence re-read the last key
+    //      (never memory nobody wrote); they are masked.
+    MlaCodes8 st[kMlaRounds];
+    float st_ks = 0.f, st_vs = 0.f;
+    auto fetch_blk = [&](int j) -> int {
+        int page = ((c_begin + min(j, nch - 1)) * kChunk) / p.page_size;
+        page = min(page, p.max_blocks - 1);
+        return bt_row[page];   // clamped and made wave-uniform where it is used, an iteration later: no wait here
+    };
+    // the loads of a chunk leave piece by piece (fetch_piece), right behind the widening of the piece that held the
+    // registers before: they have a whole step to come back
+    const int8_t *f_src = nullptr;
+    const float *f_ks = nullptr, *f_vs = nullptr;
+    uint32_t f_voff = 0, f_soff = 0;
+    auto fetch_setup = [&](int j_any, int blk_raw) {
+        const int blk = __builtin_amdgcn_readfirstlane(min(max(blk_raw, 0), p.num_blocks - 1));
+        const int j = min(j_any, nch - 1);
+        const int key0 = (c_begin + j) * kChunk;
+        const int inpage0 = key0 % p.page_size;
+        const int last = Lk - 1 - key0;
+        f_src = kc + (int64_t)blk * p.k_stride_block + (int64_t)inpage0 * p.k_stride_row;
+        f_voff = (uint32_t)min(tid >> 3, last) * (uint32_t)p.k_stride_row + (tid & 7) * 8;
+        const int64_t so = (int64_t)blk * p.ks_stride_block + (int64_t)inpage0 * p.ks_stride_row;
+        f_soff = (uint32_t)min(tid & (kChunk - 1), last) * (uint32_t)p.ks_stride_row;
+        f_ks = p.k_scale + so;
+        f_vs = p.v_scale + so;
+    };
+    auto fetch_piece = [&](int i) { st[i] = *reinterpret_cast<const MlaCodes8 *>(f_src + f_voff + i * 64); };
+    auto fetch_scales = [&]() {
+        st_ks = f_ks[f_soff];
+        st_vs = f_vs[f_soff];
+    };
+    const int st_row = tid >> 3;
+    const int st_off = st_row * kMlaRowBytes + (((tid & 7) ^ mla_swz(st_row)) << 4);
+    // widening of eight-code piece i in four steps (q = 0..3: two codes each ... the last one stores the unit)
+    u32x4_t wide;
+    auto widen_quarter = [&](int tile, int i, int q) {
+        const uint32_t w = st[i].w[q >> 1];
+        if ((q & 1) == 0) {
+            wide[q] = pack2<T>((float)(int8_t)(w & 0xff), (float)(int8_t)((w >> 8) & 0xff));
+        } else {
+            wide[q] = pack2<T>((float)(int8_t)((w >> 16) & 0xff), (float)(int8_t)(w >> 24));
+            if (q == 3) *reinterpret_cast<u32x4_t *>(&sh.k[tile][st_off + i * 128]) = wide;
+        }
+    };
+    auto stash_scales = [&](int tile) {
+        if (tid < kChunk) {
+            sh.sc[tile].ksl[tid] = st_ks * (SOFTCAP ? p.softcap_pre : p.scale_log2);
+            sh.sc[tile].vs[tid] = st_vs;
+            const float inv = (st_vs > 0.f) ? __builtin_amdgcn_rcpf(st_vs) : 0.f;
+            sh.sc[tile].vsi[tid] = inv;
+            const uint16_t hi = from_float<BF16>(inv);
+            sh.sc[tile].vsi_hi[tid] = hi;
+            sh.sc[tile].vsi_lo[tid] = from_float<BF16>(inv - to_float<BF16>(hi));
+        }
+    };
+
+    // All matrix instructions of the loop are written out: the accumulator of the score product is pinned to ordinary
+    // vector registers (the softmax reads it there), and the products stand in the instruction stream exactly where
+    // the vector work beside them is written (the wave issues in order: a product, then the few vector instructions
+    // that run in its shadow).
+    auto mfma_first = [&](float16_t &d, const u32x4_t &a, const u32x4_t &bq) {
+        if constexpr (__is_same(T, BF16))
+            asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=v"(d) : "v"(a), "v"(bq));
+        else
+            asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=v"(d) : "v"(a), "v"(bq));
+    };
+    auto mfma_v = [&](float16_t &d, const u32x4_t &a, const u32x4_t &bq) {
+        if constexpr (__is_same(T, BF16))
+            asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(d) : "v"(a), "v"(bq));
+        else
+            asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(d) : "v"(a), "v"(bq));
+    };
+    // ---- S^T = K Q^T: operand t is unit 2t + lh of key row ln.  A quarter of an eight-code piece of the next chunk is
+    //      widened beside every product.
+    float16_t s_acc;
+    const int sc_row = ln * kMlaRowBytes;
+    int sc_off[4];
+    {
+        const int sw = mla_swz(ln);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) sc_off[k] = sc_row + (((2 * k + lh) ^ sw) << 4);
+    }
+    auto scores = [&](int tile, int tile_w) {
+        constexpr int kPf = 4;
+        const uint8_t *base = &sh.k[tile][0];
+        u32x4_t ka[kMlaKSteps];
+        u32x4_t ql[kMlaQLds];
+        auto issue = [&](int t) {
+            ka[t] = *reinterpret_cast<const u32x4_t *>(base + sc_off[t & 3] + (t >> 2) * 128);
+            if (t >= kMlaQReg) ql[t - kMlaQReg] = sh.q[wave][t - kMlaQReg][lane];
+        };
+#pragma unroll
+        for (int t = 0; t < kPf; ++t) issue(t);
+#pragma unroll
+        for (int t = 0; t < kMlaKSteps; ++t) {
+            if (t + kPf < kMlaKSteps) issue(t + kPf);
+            const u32x4_t &bq = (t < kMlaQReg) ? qreg[t < kMlaQReg ? t : 0] : ql[t >= kMlaQReg ? t - kMlaQReg : 0];
+            if (t == 0)
+                mfma_first(s_acc, ka[t], bq);
             else
-                p.lse_partial[slot * p.rows + row] = (l_run > 0.f) ? m_run + fast_log2(l_run) : -INFINITY;
+                mfma_v(s_acc, ka[t], bq);
+            widen_quarter(tile_w, t >> 2, t & 3);
+            if ((t & 3) == 3) fetch_piece(t >> 2);   // chunk i+2 into the registers just widened
+            __builtin_amdgcn_sched_barrier(0);
         }
-        __syncthreads();
-    } else {
-        // =========================== output waves ==========================================
-        // o_acc[hg][t]: head group hg (16 heads), column tile t of this wave's 128-column slice
-        float4_t o_acc[4][8];
-#pragma unroll
-        for (int hg = 0; hg < 4; ++hg)
-#pragma unroll
-            for (int t = 0; t < 8; ++t) o_acc[hg][t] = float4_t{0.f, 0.f, 0.f, 0.f};
+    };
 
-        auto output_step = [&](const int j, const int set, const int tile_j) {
-            int th = tid;
-            asm volatile("" : "+v"(th));
-            const int lane = th & 63;
-            const int lq = lane >> 4;
-            const int ln = lane & 15;
-            if (j >= 2) {
-                const int tile = (tile_j == 2) ? 0 : tile_j + 1;   // (j + 1) % 3
-                const int pb = set;                                  // (j - 2) & 1
-                // ---- O^T += V^T P^T on this wave's 128-column slice, all four head groups.
-                //      k slot 8*lq + e of the MFMA is key (e >> 2) * 16 + lq * 4 + (e & 3) of the chunk.
-                //      The V^T operands come from the transposing LDS read (ds_read_b64_tr_b16): in a
-                //      16-lane group, lane s points at 4 columns (4*(s%4)..) of key row s/4 and receives
-                //      column s of the group's 16 for its 4 key rows.  Column tile ct = columns ct*16..+15
-                //      of the slice; the 16-byte unit of a row is swizzled with row & 7 = 4*(lq&1) + ln/4.
-                typedef short v4s_t __attribute__((ext_vector_type(4)));
-                const int tr_row = lq * 4 + (ln >> 2);
-                const int tr_k = 4 * (lq & 1) + (ln >> 2);
-                const uint8_t *tr_base = &sh.k[tile][tr_row * kMlaRowBytes + w4 * 256 + 8 * (ln & 1)];
-                int tr_off[4];   // unit (2*(ct&3) + (ln&3)/2) ^ tr_k inside its aligned group of eight
+    // ---- softmax of chunk j on s_acc, in place: register r of a lane is key 8*(r/4) + 4*lh + r%4 of the chunk
+    float m_ref = -INFINITY, l_run = 0.f, l_norm = 0.f;   // per lane: its 16 keys of every chunk; halves summed at the end
+    float psum = 0.f, nsum = 0.f;
+    u32x4_t pk[2];
+    // the scale vectors of slice g: registers 4g .. 4g+3 are keys 8g + 4*lh + 0..3
+    auto load_ksl = [&](int tile, int g) { return *reinterpret_cast<const float4 *>(&sh.sc[tile].ksl[4 * lh + 8 * g]); };
+    auto load_vs = [&](int tile, int g) { return *reinterpret_cast<const float4 *>(&sh.sc[tile].vs[4 * lh + 8 * g]); };
+    auto load_vsi = [&](int tile, int g) { return *reinterpret_cast<const float4 *>(&sh.sc[tile].vsi[4 * lh + 8 * g]); };
+    auto load_vsi_hi = [&](int tile, int g) { return *reinterpret_cast<const uint2 *>(&sh.sc[tile].vsi_hi[4 * lh + 8 * g]); };
+    auto load_vsi_lo = [&](int tile, int g) { return *reinterpret_cast<const uint2 *>(&sh.sc[tile].vsi_lo[4 * lh + 8 * g]); };
+    // scores in log2 units, in place, and their maximum (registers 4g .. 4g+3)
+    float xmax = -INFINITY;
+    auto softmax_scale4 = [&](int g, const float4 &kq) {
+        const float kv[4] = {kq.x, kq.y, kq.z, kq.w};
 #pragma unroll
-                for (int c4 = 0; c4 < 4; ++c4) tr_off[c4] = ((2 * c4 + ((ln & 3) >> 1)) ^ tr_k) << 4;
-                u32x4_t pkg[4];
-                const uint32_t bumps = *reinterpret_cast<const uint32_t *>(sh.bump[pb]);
-#pragma unroll
-                for (int hg = 0; hg < 4; ++hg) {
-                    pkg[hg] = sh.pk[pb][hg][lane];
-                    if ((bumps >> (8 * hg)) & 0xffu) {
-                        const float ag = sh.alpha[pb][hg][ln];
-#pragma unroll
-                        for (int t = 0; t < 8; ++t) {
-                            o_acc[hg][t][0] *= ag;
-                            o_acc[hg][t][1] *= ag;
-                            o_acc[hg][t][2] *= ag;
-                            o_acc[hg][t][3] *= ag;
-                        }
-                    }
-                }
-#pragma unroll
-                for (int ct = 0; ct < 8; ++ct) {
-                    u32x4_t va;
-#pragma unroll
-                    for (int hv = 0; hv < 2; ++hv) {
-                        const v4s_t r4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                            (__attribute__((address_space(3))) v4s_t *)(tr_base + hv * 16 * kMlaRowBytes + (ct >> 2) * 128 + tr_off[ct & 3]));
-                        const uint2 r2 = __builtin_bit_cast(uint2, r4);
-                        va[2 * hv] = r2.x;
-                        va[2 * hv + 1] = r2.y;
-                    }
-#pragma unroll
-                    for (int hg = 0; hg < 4; ++hg) o_acc[hg][ct] = mfma16<T>(va, pkg[hg], o_acc[hg][ct]);
-                }
+        for (int e = 0; e < 4; ++e) {
+            const int r = 4 * g + e;
+            float v = s_acc[r] * kv[e];
+            if constexpr (SOFTCAP) {
+                const float e2 = __expf(2.f * v);
+                v = p.softcap_post * (1.f - 2.f / (e2 + 1.f));
             }
-            __syncthreads();
-        };
-        int tile_j = 0;
-        for (int j = 0; j <= n + 1; j += 2) {
-            output_step(j, 0, tile_j);
-            tile_j = (tile_j == 2) ? 0 : tile_j + 1;
-            if (j + 1 <= n + 1) {
-                output_step(j + 1, 1, tile_j);
-                tile_j = (tile_j == 2) ? 0 : tile_j + 1;
-            }
+            s_acc[r] = v;
+            xmax = fmaxf(xmax, v);
         }
-
-        // ---- write the column slice: register i of tile t of group hg is column
-        //      w4*128 + t*16 + lq*4 + i of head hg*16 + ln
-        __syncthreads();   // sums of all heads are in LDS
-        const int lane = tid & 63;
-        const int lq = lane >> 4;
-        const int ln = lane & 15;
+    };
+    // The common chunk keeps the standing reference.  Anything else (the first chunk: the reference is -inf; a maximum
+    // beyond the lazy bound; a chunk with masked keys) goes through here: masks, a moved reference, the rescale
+    // factors for the column owners.  Returns the value the exponentials subtract.
+    auto softmax_check = [&](int j) -> float {
+        const int pb = j & 1;
+        const int key0 = (c_begin + j) * kChunk;
+        const bool edge = key0 < mask_lo || key0 + kChunk > mask_hi;   // wave-uniform
+        xmax = halves_max(xmax);
+        const bool slow = edge || __any(!(xmax <= m_ref + MlaLazy<T>::kLog2));
+        int moved = 0;
+        if (__builtin_expect(slow, 0)) {
+            float mloc = -INFINITY;
 #pragma unroll
-        for (int hg = 0; hg < 4; ++hg) {
-            const int row = hg * 16 + ln;   // row of the unit (0..63)
-            const int hd = half * kMlaHeadsPerUnit + row;
-            const float lg = sh.l[hg][ln];
-            const float inv = (lg > 0.f) ? 1.f / lg : 0.f;
-            if (write_final) {
-                uint16_t *dst = reinterpret_cast<uint16_t *>(p.out) + (int64_t)b * p.o_stride_b + (int64_t)qi * p.o_stride_s +
-                                (int64_t)hd * p.o_stride_h + w4 * 128;
+            for (int r = 0; r < 16; ++r) {
+                const int key = key0 + 8 * (r >> 2) + 4 * lh + (r & 3);
+                s_acc[r] = (key >= mask_lo && key < mask_hi) ? s_acc[r] : -INFINITY;
+                mloc = fmaxf(mloc, s_acc[r]);
+            }
+            mloc = halves_max(mloc);
+            const bool bump = mloc > m_ref + MlaLazy<T>::kLog2;   // a reference of -inf moves to any finite maximum
+            const float m_new = bump ? mloc : m_ref;
+            const float alpha = bump ? fast_exp2(m_ref - ((m_new == -INFINITY) ? 0.f : m_new)) : 1.f;
+            moved = __any(bump && m_ref != -INFINITY) ? 1 : 0;      // somebody's accumulators hold something to rescale
+            if (moved && lh == 0) sh.alpha[pb][row_u] = alpha;
+            l_run *= alpha;
+            l_norm *= alpha;
+            m_ref = m_new;
+        }
+        if (lane == 0) sh.moved[pb][wave] = moved;
+        xmax = -INFINITY;
+        return (m_ref == -INFINITY) ? 0.f : m_ref;
+    };
+    // exponentials (registers 4g .. 4g+3)
+    auto softmax_exp4 = [&](int g, float m_use) {
 #pragma unroll
-                for (int t = 0; t < 8; ++t) {
-                    const uint2 o2 = make_uint2(pack2<T>(o_acc[hg][t][0] * inv, o_acc[hg][t][1] * inv),
-                                                pack2<T>(o_acc[hg][t][2] * inv, o_acc[hg][t][3] * inv));
-                    *reinterpret_cast<uint2 *>(dst + t * 16 + lq * 4) = o2;
-                }
+        for (int e = 0; e < 4; ++e) s_acc[4 * g + e] = fast_exp2(s_acc[4 * g + e] - m_use);
+    };
+    // sums, V-side scale, rounding to the 16-bit type (registers 4g .. 4g+3); the weights really applied are summed
+    // with the inverse scales: exactly for fp16, with a two-term bf16 inverse (2^-17 relative) on the dot-product path
+    auto softmax_pack4 = [&](int g, const float4 &vq, const float4 &vi, const uint2 &ih, const uint2 &il) {
+        const float vv[4] = {vq.x, vq.y, vq.z, vq.w};
+#pragma unroll
+        for (int e = 0; e < 4; e += 2) {
+            const int r = 4 * g + e;
+            psum += s_acc[r] + s_acc[r + 1];
+            const uint32_t d = pack2<T>(s_acc[r] * vv[e], s_acc[r + 1] * vv[e + 1]);   // V side of the dequantisation folded into P
+            pk[r >> 3][(r & 7) >> 1] = d;
+            if constexpr (__is_same(T, BF16)) {
+                const uint32_t h2 = e ? ih.y : ih.x, l2 = e ? il.y : il.x;
+                nsum = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, d), __builtin_bit_cast(bf16x2_t, h2), nsum, false);
+                nsum = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, d), __builtin_bit_cast(bf16x2_t, l2), nsum, false);
             } else {
-                const int64_t srow = slot * p.rows + row;
-                float *dst = p.o_partial + srow * kMlaDv + w4 * 128;
-#pragma unroll
-                for (int t = 0; t < 8; ++t)
-                    *reinterpret_cast<float4 *>(dst + t * 16 + lq * 4) =
-                        make_float4(o_acc[hg][t][0] * inv, o_acc[hg][t][1] * inv, o_acc[hg][t][2] * inv, o_acc[hg][t][3] * inv);
+                const float iv[4] = {vi.x, vi.y, vi.z, vi.w};
+                nsum = __builtin_fmaf(to_float<T>((uint16_t)(d & 0xffffu)), iv[e], nsum);
+                nsum = __builtin_fmaf(to_float<T>((uint16_t)(d >> 16)), iv[e + 1], nsum);
             }
+        }
+    };
+    auto softmax_store = [&](int j) {
+        const int pb = j & 1;
+        l_run += psum;
+        l_norm += nsum;
+        psum = nsum = 0.f;
+        sh.pk[pb][wave][0][lane] = pk[0];
+        sh.pk[pb][wave][1][lane] = pk[1];
+    };
+
+    // ---- O^T += V^T P^T on this wave's 128 columns, all four head groups.  o_acc[cc][hg]: column tile cc (32 columns)
+    //      x head group hg; register r of a lane is column 128*wave + 32*cc + 8*(r/4) + 4*lh + r%4 of head 32*hg + ln.
+    //      k slot 8*lh + i of k-step s2 is key 16*s2 + 8*(i/4) + 4*lh + i%4 (the order the score registers come in).
+    //      The V^T operand comes from two transposing reads: in a 16-lane group, lane s points at 4 columns
+    //      (4*(s%4)..) of key row s/4 and receives column s of the group's 16 for its 4 key rows.
+    // accumulator tile (cc, hg) = a[16 * (4*cc + hg) .. +15]
+    static_for<0, 256>([&](auto r) { acc_zero<decltype(r)::value>(); });
+    int tr_off[2][2];   // [second four keys][odd column tile]
+    {
+        const int g16 = lane >> 4, s16 = lane & 15;
+        const int rbase = 4 * (g16 >> 1) + (s16 >> 2);           // key row of this lane inside an 8-row block
+        const int ub = 2 * (g16 & 1) + ((s16 & 3) >> 1);         // 16-byte unit inside the 64 bytes of a column tile
+#pragma unroll
+        for (int jj = 0; jj < 2; ++jj) {
+            const int row = 8 * jj + rbase;
+            const int sw = mla_swz(row);                          // rows 16 apart share it
+#pragma unroll
+            for (int c1 = 0; c1 < 2; ++c1)
+                tr_off[jj][c1] = row * kMlaRowBytes + (((4 * c1 + ub) ^ sw) << 4) + wave * 256 + 8 * (s16 & 1);
         }
     }
+    // accumulators of head groups whose reference moved in chunk j (rare)
+    auto rescale_moved = [&](int j) {
+        const int pb = j & 1;
+        const int4 mv = *reinterpret_cast<const int4 *>(sh.moved[pb]);
+        if (__builtin_expect((mv.x | mv.y | mv.z | mv.w) != 0, 0)) {
+            mfma_settle();
+            const int mvs[4] = {mv.x, mv.y, mv.z, mv.w};
+            static_for<0, 4>([&](auto hg_) {
+                constexpr int hg = decltype(hg_)::value;
+                if (mvs[hg]) {
+                    const float ag = sh.alpha[pb][hg * 32 + ln];
+                    static_for<0, 4>([&](auto cc_) {
+                        constexpr int cc = decltype(cc_)::value;
+                        static_for<0, 16>([&](auto r_) { acc_scale<16 * (4 * cc + hg) + decltype(r_)::value>(ag); });
+                    });
+                }
+            });
+            mfma_settle();
+        }
+    };
+    typedef short v4s_t __attribute__((ext_vector_type(4)));
+    auto read_va = [&](const uint8_t *tile_base, int cc) -> u32x4_t {
+        u32x4_t va;
+#pragma unroll
+        for (int jj = 0; jj < 2; ++jj) {
+            const v4s_t r4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                (__attribute__((address_space(3))) v4s_t *)(tile_base + tr_off[jj][cc & 1] + (cc >> 1) * 128));
+            const uint2 r2 = __builtin_bit_cast(uint2, r4);
+            va[2 * jj] = r2.x;
+            va[2 * jj + 1] = r2.y;
+        }
+        return va;
+    };
+    // ---- the second half of a step: the 32 output products of chunk j_out (OUT) beside the softmax of chunk j_sm
+    //      (SM), product by product.  Operands are requested from LDS a few products before they are used: the four
+    //      P^T operands of a 16-key half stay for its 16 products (in the half's last quarter the products run
+    //      head group by head group, and each operand is replaced by the next half's as soon as it is done with); two
+    //      pairs of V^T operands alternate, the idle pair being filled for the next quarter; the scale vectors of a
+    //      softmax slice arrive one slice ahead.  The one rare branch (softmax_check) sits after the first quarter.
+    auto phase_b = [&](auto out_, auto sm_, int j_out, int tile_out, int j_sm, int tile_sm) {
+        constexpr bool OUT = decltype(out_)::value, SM = decltype(sm_)::value;
+        const int pb = j_out & 1;
+        const uint8_t *tb0 = &sh.k[tile_out][0];
+        const uint8_t *tb1 = tb0 + 16 * kMlaRowBytes;
+        u32x4_t pkg[4], va[2], vb[2];
+        float4 sc0, sc1, sc2;
+        uint2 sh2, sl2;
+        if constexpr (OUT) {
+            rescale_moved(j_out);
+#pragma unroll
+            for (int hg = 0; hg < 4; ++hg) pkg[hg] = sh.pk[pb][hg][0][lane];
+            va[0] = read_va(tb0, 0);
+            va[1] = read_va(tb0, 1);
+        }
+        if constexpr (SM) sc0 = load_ksl(tile_sm, 0);
+        float m_use = 0.f;
+        // quarter 0: half 0, column tiles 0 and 1; scaled scores and their maximum
+        static_for<0, 8>([&](auto slot_) {
+            constexpr int slot = decltype(slot_)::value;
+            constexpr int c = slot >> 2, hg = slot & 3;
+            if constexpr (OUT) {
+                acc_mfma<T, 16 * (4 * c + hg)>(va[c], pkg[hg]);
+                if constexpr (slot == 0) vb[0] = read_va(tb0, 2);
+                if constexpr (slot == 2) vb[1] = read_va(tb0, 3);
+            }
+            if constexpr (SM && (slot & 1)) {
+                constexpr int g = slot >> 1;
+                const float4 cur = sc0;
+                if constexpr (g < 3) sc0 = load_ksl(tile_sm, g + 1);
+                softmax_scale4(g, cur);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        });
+        if constexpr (SM) {
+            m_use = softmax_check(j_sm);
+            sc1 = load_vs(tile_sm, 0);
+            if constexpr (__is_same(T, BF16)) {
+                sh2 = load_vsi_hi(tile_sm, 0);
+                sl2 = load_vsi_lo(tile_sm, 0);
+            } else {
+                sc2 = load_vsi(tile_sm, 0);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        // quarter 1: half 0, column tiles 2 and 3, head group by head group; exponentials
+        static_for<0, 8>([&](auto slot_) {
+            constexpr int slot = decltype(slot_)::value;
+            constexpr int hg = slot >> 1, c = slot & 1;
+            if constexpr (OUT) {
+                acc_mfma<T, 16 * (4 * (2 + c) + hg)>(vb[c], pkg[hg]);
+                if constexpr (c == 1) pkg[hg] = sh.pk[pb][hg][1][lane];
+                if constexpr (slot == 2) va[0] = read_va(tb1, 0);
+                if constexpr (slot == 4) va[1] = read_va(tb1, 1);
+            }
+            if constexpr (SM && (slot & 1)) softmax_exp4(slot >> 1, m_use);
+            __builtin_amdgcn_sched_barrier(0);
+        });
+        // quarters 2 and 3: half 1; sums, V-side scale, rounding
+        static_for<0, 16>([&](auto slot_) {
+            constexpr int slot = decltype(slot_)::value;
+            constexpr int cc = slot >> 2, hg = slot & 3;
+            if constexpr (OUT) {
+                if constexpr (cc < 2)
+                    acc_mfma<T, 16 * (4 * cc + hg)>(va[cc], pkg[hg]);
+                else
+                    acc_mfma<T, 16 * (4 * cc + hg)>(vb[cc - 2], pkg[hg]);
+                if constexpr (slot == 0) vb[0] = read_va(tb1, 2);
+                if constexpr (slot == 2) vb[1] = read_va(tb1, 3);
+            }
+            if constexpr (SM && (slot & 3) == 3) {
+                constexpr int g = slot >> 2;
+                const float4 cv = sc1, ci = sc2;
+                const uint2 ch = sh2, cl = sl2;
+                if constexpr (g < 3) {
+                    sc1 = load_vs(tile_sm, g + 1);
+                    if constexpr (__is_same(T, BF16)) {
+                        sh2 = load_vsi_hi(tile_sm, g + 1);
+                        sl2 = load_vsi_lo(tile_sm, g + 1);
+                    } else {
+                        sc2 = load_vsi(tile_sm, g + 1);
+                    }
+                }
+                softmax_pack4(g, cv, ci, ch, cl);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        });
+        if constexpr (SM) softmax_store(j_sm);
+    };
+    using Yes = std::true_type;
+    using No = std::false_type;
+
+    // ---- the pipeline.  Chunk j lives in tile j % 3.
+    //      step i: scores of chunk i beside the widening of chunk i+1 (the loads of chunk i+2 leave piece by piece),
+    //              softmax of chunk i beside the output products of chunk i-1, one barrier.
+    int blk_next;
+    {
+        fetch_setup(0, blk_first);
+#pragma unroll
+        for (int i = 0; i < kMlaRounds; ++i) fetch_piece(i);
+        fetch_scales();
+        blk_next = blk_second;
+#pragma unroll
+        for (int i = 0; i < kMlaRounds; ++i)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) widen_quarter(0, i, q);
+        stash_scales(0);
+        fetch_setup(1, blk_next);
+#pragma unroll
+        for (int i = 0; i < kMlaRounds; ++i) fetch_piece(i);
+        fetch_scales();
+        blk_next = fetch_blk(2);
+    }
+    __syncthreads();
+    int t_cur = 0;   // tile of chunk i
+    for (int i = 0; i < nch; ++i) {
+        const int t_nxt = (t_cur == 2) ? 0 : t_cur + 1;
+        const int t_prv = (t_cur == 0) ? 2 : t_cur - 1;
+        stash_scales(t_nxt);                // chunk i+1 (past the end: the last chunk again, into a tile nobody reads)
+        fetch_setup(i + 2, blk_next);
+        fetch_scales();
+        scores(t_cur, t_nxt);
+        blk_next = fetch_blk(i + 3);
+        mfma_settle();
+        __builtin_amdgcn_sched_barrier(0);
+        if (i > 0)
+            phase_b(Yes{}, Yes{}, i - 1, t_prv, i, t_cur);
+        else
+            phase_b(No{}, Yes{}, 0, 0, i, t_cur);
+        __syncthreads();
+        t_cur = t_nxt;
+    }
+    phase_b(Yes{}, No{}, nch - 1, (t_cur == 0) ? 2 : t_cur - 1, 0, 0);
+    mfma_settle();
+
+    // ---- sums of the two half-waves, LSE, normaliser to LDS for the column owners
+    l_run = halves_sum(l_run);
+    l_norm = halves_sum(l_norm);
+    if (lh == 0) {
+        sh.l[row_u] = (l_run > 0.f) ? l_norm : 0.f;
+        if (head < p.nheads) {
+            if (write_final)
+                p.lse[((int64_t)b * p.nheads + head) * p.seqlen_q + qi] = (l_run > 0.f) ? (m_ref + fast_log2(l_run)) * kLn2 : INFINITY;
+            else
+                p.lse_partial[slot * p.rows + row_u] = (l_run > 0.f) ? m_ref + fast_log2(l_run) : -INFINITY;
+        }
+    }
+    __syncthreads();
+    // ---- write this wave's 128-column slice of every head
+    static_for<0, 4>([&](auto hg_) {
+        constexpr int hg = decltype(hg_)::value;
+        const int row = hg * 32 + ln;
+        const int hd = hgrp * kMlaUnitHeads + row;
+        const float lg = sh.l[row];
+        const float inv = (lg > 0.f) ? 1.f / lg : 0.f;
+        const bool live = hd < p.nheads;
+        uint16_t *dst16 = reinterpret_cast<uint16_t *>(p.out) + (int64_t)b * p.o_stride_b + (int64_t)qi * p.o_stride_s +
+                          (int64_t)hd * p.o_stride_h + wave * 128 + 4 * lh;
+        float *dst32 = p.o_partial + (slot * p.rows + row) * kMlaDv + wave * 128 + 4 * lh;
+        static_for<0, 16>([&](auto t_) {
+            constexpr int cc = decltype(t_)::value >> 2, g = decltype(t_)::value & 3;
+            constexpr int base = 16 * (4 * cc + hg) + 4 * g;
+            const float o0 = acc_read<base>() * inv, o1 = acc_read<base + 1>() * inv;
+            const float o2 = acc_read<base + 2>() * inv, o3 = acc_read<base + 3>() * inv;
+            if (live) {
+                if (write_final)
+                    *reinterpret_cast<uint2 *>(dst16 + cc * 32 + g * 8) = make_uint2(pack2<T>(o0, o1), pack2<T>(o2, o3));
+                else
+                    *reinterpret_cast<float4 *>(dst32 + cc * 32 + g * 8) = make_float4(o0, o1, o2, o3);
+            }
+        });
+    });
     __syncthreads();   // the LDS tiles and sums are reused by the next piece
 }
 
@@ -428,9 +645,9 @@ __global__ void __launch_bounds__(kMlaThreads) decode_mla_i8_kernel(const Decode
     });
 }
 
-// p.nheads_k counts units per batch row here (seqlen_q * 64-head groups), p.group = p.rows = 64.
+// p.nheads_k counts units per batch row here (seqlen_q * 128-head groups), p.group = p.rows = 128.
 hipError_t launch_decode_mla_i8(const DecodeParams &p, int dtype, hipStream_t stream) {
-    if (p.units_per_token <= 0 || p.rows != kMlaHeadsPerUnit || p.group != kMlaHeadsPerUnit || !p.balanced)
+    if (p.units_per_token <= 0 || p.rows != kMlaUnitHeads || p.group != kMlaUnitHeads || !p.balanced)
         return hipErrorInvalidValue;
     dim3 grid(p.num_wgs), block(kMlaThreads);
     const bool softcap = p.softcap_post != 0.f;

@@ -578,7 +578,8 @@ __global__ void __launch_bounds__(256) splitkv_combine_balanced_kernel(const Dec
         return;
     }
     // many pieces: the whole workgroup on one row at a time
-    for (int row = row0 + blockIdx.x; row < p.rows; row += gridDim.x) combine_row_block<T, D>(p, b, kvh, row, pcs);
+    for (int row = row0 + blockIdx.x; row < p.rows; row += gridDim.x)
+        if (row_id(p, kvh, row).head < p.nheads) combine_row_block<T, D>(p, b, kvh, row, pcs);   // block-uniform
 }
 
 template <typename T, int D, int RT>

@@ -127,7 +127,6 @@ int fa_rocm_kvcache_validate(const fa_kvcache_args *a) {
                 return fail(FA_ERR_UNSUPPORTED, "int8 KV cache: v must be the view k[..., :512] of the new latent rows");
             if (a->rotary_cos) return fail(FA_ERR_UNSUPPORTED, "rotary embedding is not supported with an int8 KV cache");
         }
-        if (a->nheads % 64 != 0) return fail(FA_ERR_SHAPE, "int8 KV cache needs a multiple of 64 query heads");
         if (a->v_cache != a->k_cache || a->v_stride_block != a->k_stride_block || a->v_stride_row != a->k_stride_row)
             return fail(FA_ERR_UNSUPPORTED, "int8 KV cache: v_cache must be the view k_cache[..., :512] of the latent cache");
         if (a->k_stride_row % 16 || a->k_stride_block % 16)
@@ -167,8 +166,8 @@ int fa_rocm_plan_kvcache(const fa_kvcache_args *a, int num_cus, fa_split_plan *p
     if (a->nheads <= 0 || a->nheads_k <= 0 || a->nheads % a->nheads_k != 0)
         return fail(FA_ERR_SHAPE, "Number of heads in key/value must divide number of heads in query");
     const int group = a->nheads / a->nheads_k;
-    // the int8 latent kernel works on units of 64 query heads and always uses the balanced partition
-    const size_t rows = is_mla_i8(a) ? 64 : (size_t)a->seqlen_q * group;
+    // the int8 latent kernel works on units of 128 query heads and always uses the balanced partition
+    const size_t rows = is_mla_i8(a) ? 128 : (size_t)a->seqlen_q * group;
     const size_t slot_bytes = rows * ((size_t)a->headdim_v + 1) * sizeof(float);
     if (!is_mla_i8(a) && rows > (size_t)decode_max_rows(a)) {
         // Query block too tall for the decode kernels: the tiled forward.  When its tiles alone
@@ -560,10 +559,10 @@ static int fwd_kvcache_impl(const fa_kvcache_args *a, void *stream_, void *const
 
     hipError_t e;
     if (is_mla_i8(a)) {
-        p.units_per_token = a->nheads / 64;               // 64-head groups
+        p.units_per_token = (a->nheads + 127) / 128;      // 128-head groups (the last one may be partly empty)
         p.nheads_k = a->seqlen_q * p.units_per_token;     // units per batch row
-        p.group = 64;
-        p.rows = 64;
+        p.group = 128;
+        p.rows = 128;
         e = fa::launch_decode_mla_i8(p, a->io_dtype, stream);
     }
     else {
