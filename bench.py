@@ -1,14 +1,17 @@
 #!/usr/bin/env python3
 """Benchmark of the paged KV-cache attention path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2|c2_8k|c3a|c3b|c4|c5|mixed] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config all|c2|c2_8k|c3a|c3b|c4|c5|mixed] [--no-cpu]
 
 A step is one call of the hot path (append + rotary + attention + split combine for the decode
 configs, one varlen forward for c5) on synthetic inputs that are resident in HBM before the
 timed region.  Two input sets are alternated so that no step finds its K/V in the 256 MB
-last-level cache.  Prints ONE JSON line: whole-call throughput (`value`), the roofline record of
+last-level cache.  Prints ONE JSON line: whole-call throughput (`value`, K steps between two device
+synchronisations), the median of the per-step durations taken with HIP events, the roofline record of
 the dominant kernel (its duration measured with HIP events the library records around it on the
-launch stream) and the CPU golden path timed on the host cores of this box.
+launch stream) and the CPU golden path timed on the host cores of this box.  The default (`all`) is
+the headline config c2 plus a `configs` object with the same measurements, on the same K and W, for
+every other configuration of the baseline (c2_8k, c3a, c3b, c4, c5), each with a short CPU sample.
 """
 from __future__ import annotations
 
@@ -26,10 +29,35 @@ for _p in (os.path.join(ROOT, "flash-attention-npu_amd"), os.path.join(ROOT, "or
         sys.path.insert(0, _p)
 
 HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E
-# HBM bytes per launch of the attention kernel from the FETCH_SIZE / WRITE_SIZE counter passes
-# (calibrated against a 1 GiB device copy); the workloads are seeded, so these are constants.
-MEASURED_TRAFFIC_BYTES = {"c2": 1241.6e6, "c3a": 2156.7e6, "c4": 399.7e6}
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
+
+# HBM bytes per launch of the dominant kernel are not something a timing run can see: they come from the
+# FETCH_SIZE / WRITE_SIZE counter passes whose summaries are tracked under profiles/ (a line
+# "traffic_bytes_per_launch: N" in the summary of that kernel and workload).  The workloads are seeded, so the
+# figure belongs to the kernel as it was when the summary was made; the record names the file it was read from.
+PROFILE_OF = {"c2": "decode_wave_kernel_c2.txt", "c3a": "decode_wave_kernel_c3a.txt", "c3b": "decode_wave_kernel_c3b.txt",
+              "c4": "decode_mla_i8_kernel_c4.txt", "c5": "prefill_kernel_c5.txt"}
+
+
+def traffic_from_profile(name: str):
+    """(bytes, file) of the counter-measured HBM traffic per launch for config `name`, or (None, None)."""
+    fn = PROFILE_OF.get(name)
+    path = os.path.join(ROOT, "profiles", fn) if fn else None
+    if not path or not os.path.exists(path):
+        return None, None
+    for line in open(path):
+        if line.startswith("traffic_bytes_per_launch:"):
+            try:
+                return float(line.split(":", 1)[1].split()[0]), "profiles/" + fn
+            except ValueError:
+                return None, None
+    return None, None
+
+
+def median(xs):
+    xs = sorted(xs)
+    n = len(xs)
+    return xs[n // 2] if n % 2 else 0.5 * (xs[n // 2 - 1] + xs[n // 2])
 
 
 # ----------------------------------------------------------------------------- HIP events
@@ -189,7 +217,7 @@ def bind_decode(w, num_splits=0):
                             w["window"][0], w["window"][1], 0.0, False, num_splits, w.get("k_scale"), None)
 
 
-def cpu_decode_baseline(w, budget_s: float = 20.0):
+def cpu_decode_baseline(w, budget_s: float = 20.0, min_s: float = 10.0):
     """The oracle's blocked golden (restated reference test golden) on host cores."""
     import torch
     import fa_oracle as O
@@ -200,7 +228,6 @@ def cpu_decode_baseline(w, budget_s: float = 20.0):
     # bounded sample: whole passes over the batch rows for at least min_s seconds, cut off inside a
     # pass once the budget is used up
     B = w["B"]
-    min_s = 10.0
     t0 = time.perf_counter()
     secs, bytes_done, rows_done, passes = 0.0, 0.0, 0, 0
     while time.perf_counter() - t0 < min_s:
@@ -236,7 +263,7 @@ def cpu_decode_baseline(w, budget_s: float = 20.0):
 
 
 # ----------------------------------------------------------------------------- main
-def run_decode(args, name):
+def run_decode(args, name, cpu_budget=(20.0, 10.0)):
     import torch
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
@@ -269,9 +296,12 @@ def run_decode(args, name):
     k_ms = [ev.elapsed_ms(4 * i + 1, 4 * i + 2) for i in range(args.steps)]
     a_ms = [ev.elapsed_ms(4 * i + 0, 4 * i + 1) for i in range(args.steps)]
     c_ms = [ev.elapsed_ms(4 * i + 2, 4 * i + 3) for i in range(args.steps)]
+    t_ms = [ev.elapsed_ms(4 * i + 0, 4 * i + 3) for i in range(args.steps)]
     ev.close()
-    kern_ms = sum(k_ms) / len(k_ms)
+    call_ms = [ev_ms for ev_ms in t_ms]
+    kern_ms = median(k_ms)
     achieved = attn_bytes / (kern_ms * 1e-3) / 1e9
+    traffic, traffic_file = traffic_from_profile(name) if args.kv_layout == "nhd" and args.num_splits == 0 else (None, None)
 
     from flash_attn_npu import _lib
     lib = _lib.load()
@@ -293,13 +323,15 @@ def run_decode(args, name):
                    "split_mode": "balanced" if plan.mode == 1 else "grid", "workgroups": plan.num_wgs, "workers": plan.num_workers,
                    "kv_splits": plan.nsplits, "split_keys": plan.split_keys, "cold_cache": "two pools alternated", "kv_layout": args.kv_layout},
         "us_per_call": ms_per_step * 1e3,
+        "us_per_call_median": median(call_ms) * 1e3,     # per-step HIP events on the launch stream, whole call
         "pct_of_hbm_peak": 100.0 * total_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,
         "algorithmic_bytes": total_bytes,
         "roofline": {"bound": "hbm", "kernel": kernel_name, "achieved": achieved, "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(name) if args.kv_layout == "nhd" and args.num_splits == 0 else None,
-                     "kernel_us": kern_ms * 1e3, "append_us": sum(a_ms) / len(a_ms) * 1e3,
-                     "combine_us": sum(c_ms) / len(c_ms) * 1e3, "algorithmic_bytes_per_launch": attn_bytes},
+                     "traffic": traffic, "traffic_source": traffic_file,
+                     "kernel_us": kern_ms * 1e3, "kernel_us_stat": "median of per-step HIP events",
+                     "append_us": median(a_ms) * 1e3, "combine_us": median(c_ms) * 1e3,
+                     "algorithmic_bytes_per_launch": attn_bytes},
     }
     if name == "c4":
         # arithmetic intensity of this config is above the ridge: report the matrix-core side too
@@ -309,7 +341,9 @@ def run_decode(args, name):
                                 "unit": "TFLOP/s", "frac": flops / (kern_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
                                 "algorithmic_flops": flops}
     if not args.no_cpu:
-        out["cpu_baseline"] = cpu_decode_baseline(w)
+        out["cpu_baseline"] = cpu_decode_baseline(w, budget_s=cpu_budget[0], min_s=cpu_budget[1])
+    del calls, sets, w
+    torch.cuda.empty_cache()
     return out
 
 
@@ -335,7 +369,7 @@ def prefill_workload(device, seed: int = 0):
                 max_len=int(lens.max()), hq=32, hk=8, d=128)
 
 
-def run_prefill(args):
+def run_prefill(args, cpu_budget_s: float = 20.0):
     import torch
     from flash_attn_npu import flash_attn_npu as ops
     dev = torch.device("cuda:0")
@@ -365,9 +399,10 @@ def run_prefill(args):
         step()
         ev.record(2 * i + 1, stream)
     torch.cuda.synchronize()
-    kern_ms = sum(ev.elapsed_ms(2 * i, 2 * i + 1) for i in range(args.steps)) / args.steps
+    kern_ms = median([ev.elapsed_ms(2 * i, 2 * i + 1) for i in range(args.steps)])
     ev.close()
     achieved = flops / (kern_ms * 1e-3) / 1e12
+    traffic, traffic_file = traffic_from_profile("c5")
     res = {
         "metric": "varlen_prefill_fwd_tflops", "value": flops / (ms_per_step * 1e-3) / 1e12, "unit": "TFLOP/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
@@ -375,11 +410,12 @@ def run_prefill(args):
         "config": {"workload": "c5: varlen prefill forward bf16, 16 sequences (lengths U[512,4096] rescaled to 32768 "
                                "tokens), 32q/8kv heads, d=128, causal", "seq_lens": [int(x) for x in w["lens"]],
                    "flop_count": "sum 4*S^2*d*Hq / 2"},
-        "us_per_call": ms_per_step * 1e3, "algorithmic_flops": flops,
+        "us_per_call": ms_per_step * 1e3, "us_per_call_median": kern_ms * 1e3, "algorithmic_flops": flops,
         "pct_of_mfma_peak": 100.0 * flops / (ms_per_step * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
         "roofline": {"bound": "mfma", "kernel": "prefill_kernel", "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS,
-                     "unit": "TFLOP/s", "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
-                     "kernel_us": kern_ms * 1e3},
+                     "unit": "TFLOP/s", "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": traffic,
+                     "traffic_source": traffic_file, "kernel_us": kern_ms * 1e3,
+                     "kernel_us_stat": "median of per-step HIP events"},
     }
     if not args.no_cpu:
         import fa_oracle as O
@@ -393,11 +429,13 @@ def run_prefill(args):
             secs += time.perf_counter() - t1
             done_flops += 4.0 * (e - a) * (e - a) * w["d"] * w["hq"] / 2.0
             n += 1
-            if secs > 20.0:
+            if secs > cpu_budget_s:
                 break
         res["cpu_baseline"] = dict(value=done_flops / secs / 1e12, unit="TFLOP/s", cores=torch.get_num_threads(), kind="port",
                                    sample=f"oracle blocked golden on the first {n} of 16 sequences, {secs:.2f} s on "
                                           f"{os.cpu_count()} host cpus, torch threads {torch.get_num_threads()}")
+    del w, out
+    torch.cuda.empty_cache()
     return res
 
 
@@ -480,12 +518,21 @@ def run_copy(args):
             "config": {"workload": "copy: 1 GiB torch copy_ (read 1 GiB + write 1 GiB per step)"}}
 
 
+def sub_record(r):
+    """What a sub-record of the default line keeps of a config's own line."""
+    keep = ("metric", "value", "unit", "ms_per_step", "us_per_call", "us_per_call_median", "dtype", "roofline",
+            "roofline_mfma", "cpu_baseline", "algorithmic_bytes", "algorithmic_flops")
+    d = {k: r[k] for k in keep if k in r}
+    d["workload"] = r["config"]["workload"]
+    return d
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--config", default="c2")
+    ap.add_argument("--config", default="all", help="all = c2 headline plus sub-records of every other baseline config")
     ap.add_argument("--num-splits", type=int, default=0, help="0 = balanced partition (default), n >= 1 = fixed splits")
     ap.add_argument("--kv-layout", default="nhd", choices=["nhd", "hnd"], help="memory layout of the paged caches")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU golden timing")
@@ -498,7 +545,15 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py needs a ROCm GPU", file=sys.stderr)
         sys.exit(2)
-    if args.config in ("c2", "c2_8k", "c3a", "c3b", "c4") or args.config.startswith("c2_u"):
+    if args.config == "all":
+        out = run_decode(args, "c2")
+        subs = {}
+        for name in ("c2_8k", "c3a", "c3b", "c4"):
+            r = run_decode(args, name, cpu_budget=(4.0, 2.5))
+            subs[name] = sub_record(r)
+        subs["c5"] = sub_record(run_prefill(args, cpu_budget_s=3.0))
+        out["configs"] = subs
+    elif args.config in ("c2", "c2_8k", "c3a", "c3b", "c4") or args.config.startswith("c2_u"):
         out = run_decode(args, args.config)
     elif args.config == "c5":
         out = run_prefill(args)
