@@ -89,3 +89,13 @@ def check_vs_golden(out, golden, lse, golden_lse, what=""):
     fin = ~torch.isinf(golden_lse)
     assert torch.equal(torch.isinf(l), torch.isinf(golden_lse)), f"{what}: +inf LSE rows differ"
     torch.testing.assert_close(l[fin], golden_lse[fin], rtol=REF_RTOL, atol=REF_ATOL, msg=lambda m: f"{what} lse: {m}")
+
+
+def check_compare_rule(out, ref_fp32, what="", rel=5e-3, floor=5e-3, share=0.995):
+    """The element-wise rule of the reference's fourth-generation tests (tests/npu_precision_utils.py:130-164, used at
+    tests/test_flash_attn_npu_v4.py:614-619): at least 99.5 % of the elements lie within max(5e-3 * |golden|, 5e-3)."""
+    o = out.detach().float().cpu().flatten()
+    g = ref_fp32.detach().float().cpu().flatten()
+    limit = torch.maximum(g.abs() * rel, torch.tensor(floor))
+    ok = ((o - g).abs() <= limit).float().mean().item()
+    assert ok >= share, f"{what}: only {100 * ok:.3f} % of the elements within max({rel}*|g|, {floor})"

@@ -4,7 +4,7 @@ import pytest
 import torch
 
 import fa_oracle as O
-from helpers import check_out, check_vs_golden, make_paged_case, to_dev
+from helpers import check_compare_rule, check_out, check_vs_golden, make_paged_case, to_dev
 
 pytestmark = pytest.mark.gpu
 
@@ -22,6 +22,13 @@ def varlen_case(seqs_q, seqs_k, hq, hk, d, dtype=torch.bfloat16, seed=0, dist="n
     cu_k = torch.tensor([0] + list(torch.tensor(seqs_k).cumsum(0)), dtype=torch.int32)
     return dict(q=rnd(tq, hq, d).to(dtype), k=rnd(tk, hk, d).to(dtype), v=rnd(tk, hk, d).to(dtype),
                 cu_q=cu_q, cu_k=cu_k, max_q=max(seqs_q), max_k=max(seqs_k))
+
+
+def check_paged(out, ref, lse, ref_lse, what=""):
+    """The bars of the paged-varlen tests: the fp32 bars plus the element-wise rule of the reference's own paged-varlen
+    tests (its fourth API generation)."""
+    check_out(out, ref, lse, ref_lse, what)
+    check_compare_rule(out, ref, what)
 
 
 def run_varlen(c, **kw):
@@ -102,7 +109,7 @@ def test_varlen_paged_kv():
     kl = torch.cat([O.gather_paged(case["k_cache"], case["block_table"][b], lens_k[b]) for b in range(3)])
     vl = torch.cat([O.gather_paged(case["v_cache"], case["block_table"][b], lens_k[b]) for b in range(3)])
     ref, ref_lse = O.flash_attn_varlen(q, kl, vl, cu_q, cu_k, max(lens_q), max(lens_k), causal=True, mode="fp32")
-    check_out(out, ref, lse, ref_lse, "paged varlen")
+    check_paged(out, ref, lse, ref_lse, "paged varlen")
 
 
 @pytest.mark.parametrize("sq,hq,hk", [(128, 8, 2), (1024, 4, 4), (33, 8, 1), (17, 16, 2)])
@@ -305,7 +312,7 @@ def test_varlen_paged_ragged_blocks_split_keys(hq, hk, d, causal, window, num_sp
                                 0.0, d ** -0.5, False, causal, window[0], window[1], 0.0, False, None, num_splits=num_splits)
     torch.cuda.synchronize()
     ref, ref_lse = O.flash_attn_varlen(q, kl, vl, cu_q, cu_k, max(lens_q), max(lens_k), causal=causal, window_size=window, mode="fp32")
-    check_out(out, ref, lse, ref_lse, "ragged split")
+    check_paged(out, ref, lse, ref_lse, "ragged split")
 
 
 @pytest.mark.parametrize("causal,window,softcap", [(True, (-1, -1), 0.0), (False, (-1, -1), 0.0), (True, (1500, 0), 0.0),
@@ -333,13 +340,13 @@ def test_varlen_paged_short_blocks_on_the_decode_kernels(causal, window, softcap
     out, lse = call()
     ref, ref_lse = O.flash_attn_varlen(q, kl, vl, cu_q, cu_k, max(lens_q), max(lens_k), causal=causal, window_size=window,
                                        softcap=softcap, mode="fp32")
-    check_out(out, ref, lse, ref_lse, "short blocks")
+    check_paged(out, ref, lse, ref_lse, "short blocks")
     os.environ["FA_ROCM_NO_SHORT_BLOCKS"] = "1"
     try:
         out2, lse2 = call()
     finally:
         del os.environ["FA_ROCM_NO_SHORT_BLOCKS"]
-    check_out(out2, ref, lse2, ref_lse, "short blocks, tiled kernel only")
+    check_paged(out2, ref, lse2, ref_lse, "short blocks, tiled kernel only")
     short = torch.tensor([1 <= n <= 4 for n in lens_q for _ in range(n)])
     assert torch.equal(out[~short].cpu(), out2[~short].cpu()), "rows of the tiled kernel changed with the routing"
     assert not torch.equal(out[short].cpu(), out2[short].cpu()), "the short blocks did not take the other path"
@@ -359,7 +366,7 @@ def test_varlen_paged_all_blocks_short(causal, window, lens_q, hq, hk):
                                 0.0, d ** -0.5, False, causal, window[0], window[1], 0.0, False, None)
     torch.cuda.synchronize()
     ref, ref_lse = O.flash_attn_varlen(q, kl, vl, cu_q, cu_k, max(lens_q), max(lens_k), causal=causal, window_size=window, mode="fp32")
-    check_out(out, ref, lse, ref_lse, "all blocks short")
+    check_paged(out, ref, lse, ref_lse, "all blocks short")
 
 
 def test_varlen_paged_small_mixed_batch():
@@ -374,4 +381,4 @@ def test_varlen_paged_small_mixed_batch():
                                 0.0, d ** -0.5, False, True, -1, -1, 0.0, False, None)
     torch.cuda.synchronize()
     ref, ref_lse = O.flash_attn_varlen(q, kl, vl, cu_q, cu_k, max(lens_q), max(lens_k), causal=True, mode="fp32")
-    check_out(out, ref, lse, ref_lse, "small mixed batch")
+    check_paged(out, ref, lse, ref_lse, "small mixed batch")

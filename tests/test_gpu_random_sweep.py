@@ -38,6 +38,28 @@ def draw_kvcache(seed):
                 num_splits=num_splits, dtype=dtype, rot=rot, interleaved=interleaved)
 
 
+def draw_odd_groups(seed):
+    """GQA groups that are not powers of two and query blocks whose row count (tokens x group) lands on either side of
+    the kernels' 16- and 32-row switches: 18, 30, 33, 50, 70 and their neighbours."""
+    r = random.Random(seed)
+    group = r.choice([3, 6, 7, 9, 12, 20])
+    rows_target = r.choice([9, 15, 16, 18, 30, 32, 33, 50, 70])
+    sq = max(1, round(rows_target / group))
+    hk = r.choice([1, 2, 4])
+    d = r.choice([64, 128, 128, 256])
+    page = r.choice([32, 128, 256])
+    B = r.randint(1, 4)
+    lens = [r.choice([0, 1, 33, r.randint(1, 300), r.randint(300, 3000)]) for _ in range(B)]
+    snew = r.choice([0, 0, 1, sq])
+    causal = r.random() < 0.6
+    window = r.choice([(-1, -1), (-1, -1), (r.randint(0, 300), 0), (r.randint(0, 300), r.randint(0, 64))])
+    dtype = r.choice([torch.bfloat16, torch.bfloat16, torch.float16])
+    rot = r.choice([0, 0, 32, d]) if snew else 0
+    return dict(B=B, hq=hk * group, hk=hk, d=d, page=page, lens=lens, sq=sq, snew=snew, causal=causal, window=window,
+                softcap=r.choice([0.0, 0.0, 30.0]), num_splits=r.choice([0, 0, 1, 3]), dtype=dtype, rot=rot,
+                interleaved=r.random() < 0.5)
+
+
 def draw_tall(seed):
     """Query blocks up to 257 tokens x 16 heads per kv head and batches up to 24 rows: the blocks that leave the
     decode kernels for the tiled one, its packed heads and its key-range split.  Sized so the oracle takes ~0.1 s."""
@@ -64,10 +86,10 @@ def draw_tall(seed):
                 softcap=softcap, num_splits=num_splits, dtype=dtype, rot=rot, interleaved=r.random() < 0.5)
 
 
-@pytest.mark.parametrize("seed", [*range(60), 324, *range(2000, 2060)])     # 324: an fp16 rotary result on an exact tie
+@pytest.mark.parametrize("seed", [*range(60), 324, *range(2000, 2060), *range(4000, 4048)])     # 324: an fp16 rotary result on an exact tie
 def test_random_kvcache(seed):
     from flash_attn_npu import flash_attn_with_kvcache
-    c = draw_kvcache(1000 + seed) if seed < 2000 else draw_tall(seed - 2000)
+    c = draw_kvcache(1000 + seed) if seed < 2000 else (draw_tall(seed - 2000) if seed < 4000 else draw_odd_groups(seed))
     print("random kvcache", seed, c, flush=True)
     case = make_paged_case(c["B"], c["hq"], c["hk"], c["d"], c["page"], c["lens"], seqlen_q=c["sq"], seqlen_new=c["snew"],
                            dtype=c["dtype"], seed=seed, extra_table_cols=seed % 2)
