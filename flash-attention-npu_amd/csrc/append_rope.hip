@@ -16,9 +16,10 @@ namespace fa {
 // grid: (Hk, Snew, B); block: 64 threads striding over the element pairs of one head row
 template <typename T>
 __global__ void __launch_bounds__(64) append_kv_kernel(const AppendParams p) {
-    const int h = blockIdx.x;
-    const int t = blockIdx.y;
-    const int b = blockIdx.z;
+    // one-dimensional grid (the y and z extents stop at 65535): block = (b * seqlen_new + t) * nheads_k + h
+    const int h = blockIdx.x % p.nheads_k;
+    const int t = (blockIdx.x / p.nheads_k) % p.seqlen_new;
+    const int b = blockIdx.x / (p.nheads_k * p.seqlen_new);
     const int pos = p.cache_seqlens[b] + t;
     if (pos < 0) return;
     const int page = pos / p.page_size;
@@ -76,8 +77,8 @@ __global__ void __launch_bounds__(64) append_kv_kernel(const AppendParams p) {
 // and scales can be compared bit-for-bit with a host computation.
 template <typename T>
 __global__ void __launch_bounds__(64) append_quant_i8_kernel(const AppendParams p) {
-    const int t = blockIdx.x;
-    const int b = blockIdx.y;
+    const int t = blockIdx.x % p.seqlen_new;     // one-dimensional grid: block = b * seqlen_new + t
+    const int b = blockIdx.x / p.seqlen_new;
     const int lane = threadIdx.x;
     const int pos = p.cache_seqlens[b] + t;
     if (pos < 0) return;
@@ -109,7 +110,8 @@ __global__ void __launch_bounds__(64) append_quant_i8_kernel(const AppendParams 
 }
 
 hipError_t launch_append_quant_i8(const AppendParams &p, int dtype, hipStream_t stream) {
-    dim3 grid(p.seqlen_new, p.batch);
+    if ((int64_t)p.seqlen_new * p.batch > INT32_MAX) return hipErrorInvalidValue;
+    dim3 grid((unsigned)(p.seqlen_new * p.batch));
     if (dtype == 0)
         hipLaunchKernelGGL(append_quant_i8_kernel<BF16>, grid, dim3(64), 0, stream, p);
     else
@@ -121,9 +123,9 @@ hipError_t launch_append_quant_i8(const AppendParams &p, int dtype, hipStream_t 
 // same arithmetic as the append (flash_attn_npu_interface.py:1469-1474).  grid: (Hq, Sq, B)
 template <typename T>
 __global__ void __launch_bounds__(64) rotate_q_kernel(const RotateQParams p) {
-    const int h = blockIdx.x;
-    const int i = blockIdx.y;
-    const int b = blockIdx.z;
+    const int h = blockIdx.x % p.nheads;         // one-dimensional grid: block = (b * seqlen_q + i) * nheads + h
+    const int i = (blockIdx.x / p.nheads) % p.seqlen_q;
+    const int b = blockIdx.x / (p.nheads * p.seqlen_q);
     const int pos = p.cache_seqlens[b] + (p.rotary_per_token ? i : 0);
     const int rpos = min(max(pos, 0), p.seqlen_ro - 1);
     const uint16_t *src = reinterpret_cast<const uint16_t *>(p.q) + (int64_t)b * p.q_stride_b + (int64_t)i * p.q_stride_s +
@@ -158,7 +160,8 @@ __global__ void __launch_bounds__(64) rotate_q_kernel(const RotateQParams p) {
 }
 
 hipError_t launch_rotate_q(const RotateQParams &p, int dtype, hipStream_t stream) {
-    dim3 grid(p.nheads, p.seqlen_q, p.batch);
+    if ((int64_t)p.nheads * p.seqlen_q * p.batch > INT32_MAX) return hipErrorInvalidValue;
+    dim3 grid((unsigned)(p.nheads * p.seqlen_q * p.batch));
     if (dtype == 0)
         hipLaunchKernelGGL(rotate_q_kernel<BF16>, grid, dim3(64), 0, stream, p);
     else
@@ -167,7 +170,8 @@ hipError_t launch_rotate_q(const RotateQParams &p, int dtype, hipStream_t stream
 }
 
 hipError_t launch_append_kv(const AppendParams &p, int dtype, hipStream_t stream) {
-    dim3 grid(p.nheads_k, p.seqlen_new, p.batch);
+    if ((int64_t)p.nheads_k * p.seqlen_new * p.batch > INT32_MAX) return hipErrorInvalidValue;
+    dim3 grid((unsigned)(p.nheads_k * p.seqlen_new * p.batch));
     if (dtype == 0)
         hipLaunchKernelGGL(append_kv_kernel<BF16>, grid, dim3(64), 0, stream, p);
     else

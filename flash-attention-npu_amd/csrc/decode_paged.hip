@@ -624,8 +624,6 @@ hipError_t launch_decode_paged(const DecodeParams &p, int dtype, int headdim, hi
     return dtype == 0 ? launch_decode_t<BF16>(p, headdim, stream) : launch_decode_t<FP16>(p, headdim, stream);
 }
 
-int decode_wgs_per_cu(int headdim, int rows) { return (headdim <= 128 && rows <= 32) ? 2 : 1; }
-
 template <typename T, int D> static void launch_combine_d(const DecodeParams &p, hipStream_t stream) {
     if (p.balanced) {
         // one workgroup per unit when there are many units, up to one per query row when there are few (units

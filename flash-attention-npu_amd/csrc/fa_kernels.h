@@ -151,13 +151,29 @@ struct PrefillParams {
     float *lse_partial;
 };
 
+// ---- planning rules shared by the host API and the launchers (host integer code; 64-bit inside so that no
+// combination of 32-bit dimensions overflows) ----
+constexpr int kPrefillTileRows = 128;   // query rows of one tile of the tiled forward
+
 // GQA group packed into the tile rows of the tiled forward for query blocks of max_seqlen_q rows
-// (1 = one q head per tile).
-int prefill_pack(int group, int max_seqlen_q);
-// 1 when the blocks of a token-major launch that does not pack (prefill_pack == 1) pack on their own where they are short.
-int prefill_pack_short(int group, int max_seqlen_q, int total_q, int batch);
+// (1 = one q head per tile): the heads of a group share a tile when that saves at least a quarter of the tiles.
+inline int prefill_pack(int group, int max_seqlen_q) {
+    if (group <= 1 || max_seqlen_q <= 0) return 1;
+    const int64_t tiles_plain = (int64_t)group * (((int64_t)max_seqlen_q + kPrefillTileRows - 1) / kPrefillTileRows);
+    const int64_t tiles_packed = ((int64_t)max_seqlen_q * group + kPrefillTileRows - 1) / kPrefillTileRows;
+    return tiles_packed * 4 <= tiles_plain * 3 ? group : 1;
+}
+// 1 when the blocks of a token-major launch that does not pack (prefill_pack == 1) pack on their own where they are
+// short: blocks that differ in length and whose average would pack (mixed prefill / decode batches).
+inline int prefill_pack_short(int group, int max_seqlen_q, int total_q, int batch) {
+    if (group <= 1 || batch <= 0 || total_q <= 0 || prefill_pack(group, max_seqlen_q) > 1) return 0;
+    return prefill_pack(group, (int)(((int64_t)total_q + batch - 1) / batch)) > 1 ? 1 : 0;
+}
 // Tiles (workgroups) of the tiled forward per batch row.
-int prefill_tiles(int nheads, int nheads_k, int max_seqlen_q);
+inline int64_t prefill_tiles(int nheads, int nheads_k, int max_seqlen_q) {
+    const int pack = prefill_pack(nheads / nheads_k, max_seqlen_q);
+    return (int64_t)(pack > 1 ? nheads_k : nheads) * (((int64_t)max_seqlen_q * pack + kPrefillTileRows - 1) / kPrefillTileRows);
+}
 
 // dtype: 0 = bf16, 1 = fp16 (enum fa_dtype).  All return hipError_t of the launch.
 hipError_t launch_append_kv(const AppendParams &p, int dtype, hipStream_t stream);
@@ -175,7 +191,7 @@ hipError_t launch_gather_short_blocks(const ShortBlocksParams &p, hipStream_t st
 hipError_t launch_scatter_short_blocks(const ShortBlocksParams &p, hipStream_t stream);
 
 // Resident decode workgroups per compute unit for a head dimension / query-block height.
-int decode_wgs_per_cu(int headdim, int rows);
+inline int decode_wgs_per_cu(int headdim, int rows) { return (headdim <= 128 && rows <= 32) ? 2 : 1; }
 
 // Largest query block (seqlen_q * group) that runs on the decode kernels: one or two 16-row MFMA
 // tiles.  Taller blocks run on the tiled kernel with the GQA heads packed into its 128-row tiles, which

@@ -15,6 +15,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 
 #include "../../include/fa_rocm.h"
 #include "fa_kernels.h"
@@ -50,7 +51,109 @@ int device_cus() {
 
 bool is_mla_i8(const fa_kvcache_args *a) { return a->kv_dtype == FA_INT8; }
 
-// Upper bound of the live key range any row can have, from shapes alone.
+// Experiment knobs and the validation switch, from the environment.  They are read ONCE, on the first call that
+// needs them (or again when fa_rocm_reload_env() is called): nothing on the call path touches the environment.
+struct EnvKnobs {
+    int decode_max_rows = 0;       // FA_ROCM_DECODE_MAX_ROWS: 16 or 32, else the built-in rule
+    int decode_wgs = 0;            // FA_ROCM_DECODE_WGS: workgroups of the balanced partition
+    bool block_workers = false;    // FA_ROCM_DECODE_BLOCK_WORKERS
+    int min_share = 0;             // FA_ROCM_MIN_SHARE
+    int piece_cost = -1;           // FA_ROCM_PIECE_COST
+    bool no_head_interleave = false, separate_append = false, no_short_blocks = false;
+    bool validate = false;         // FA_ROCM_VALIDATE: check tables, capacities and positions on the device (slow)
+};
+EnvKnobs g_env;
+std::once_flag g_env_once;
+
+void load_env() {
+    EnvKnobs e;
+    auto num = [](const char *name, int dflt) {
+        const char *v = std::getenv(name);
+        return v ? std::atoi(v) : dflt;
+    };
+    auto flag = [](const char *name) {
+        const char *v = std::getenv(name);
+        return v != nullptr && std::strcmp(v, "0") != 0;
+    };
+    e.decode_max_rows = num("FA_ROCM_DECODE_MAX_ROWS", 0);
+    e.decode_wgs = num("FA_ROCM_DECODE_WGS", 0);
+    e.block_workers = flag("FA_ROCM_DECODE_BLOCK_WORKERS");
+    e.min_share = num("FA_ROCM_MIN_SHARE", 0);
+    e.piece_cost = std::getenv("FA_ROCM_PIECE_COST") ? std::max(0, num("FA_ROCM_PIECE_COST", 0)) : -1;
+    e.no_head_interleave = flag("FA_ROCM_NO_HEAD_INTERLEAVE");
+    e.separate_append = flag("FA_ROCM_SEPARATE_APPEND");
+    e.no_short_blocks = flag("FA_ROCM_NO_SHORT_BLOCKS");
+    e.validate = flag("FA_ROCM_VALIDATE");
+    g_env = e;
+}
+const EnvKnobs &env() {
+    std::call_once(g_env_once, load_env);
+    return g_env;
+}
+
+// ---- FA_ROCM_VALIDATE: the checks that need the device's own data (lengths and page ids live there) ----
+// One thread per batch row; the first violation found is recorded as {kind, row, value, limit}.
+enum { kBadNone = 0, kBadLength = 1, kBadCapacity = 2, kBadPage = 3, kBadRotary = 4 };
+static __device__ int g_check_result[4];
+
+__global__ void check_paged_rows_kernel(const int32_t *__restrict__ lens, const int32_t *__restrict__ block_table, int64_t bt_stride_b,
+                                        int batch, int add, int page_size, int max_blocks, int num_blocks, int seqlen_ro, int *result) {
+    const int b = blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= batch) return;
+    auto report = [&](int kind, int value, int limit) {
+        if (atomicCAS(&result[0], kBadNone, kind) == kBadNone) {
+            result[1] = b;
+            result[2] = value;
+            result[3] = limit;
+        }
+    };
+    const int len = lens[b];
+    if (len < 0) return report(kBadLength, len, 0);
+    const int64_t total = (int64_t)len + add;
+    const int64_t capacity = (int64_t)max_blocks * page_size;
+    if (total > capacity) return report(kBadCapacity, (int)(total < INT32_MAX ? total : INT32_MAX), (int)(capacity < INT32_MAX ? capacity : INT32_MAX));
+    if (seqlen_ro > 0 && total > seqlen_ro) return report(kBadRotary, (int)total, seqlen_ro);
+    const int used = (int)((total + page_size - 1) / page_size);
+    for (int i = 0; i < used; ++i) {
+        const int id = block_table[b * bt_stride_b + i];
+        if (id < 0 || id >= num_blocks) return report(kBadPage, id, num_blocks);
+    }
+}
+
+// Runs the check and WAITS for it (the only place where the library synchronises with the host): a debugging mode,
+// unusable while `stream` is being captured.  `what` names the length array in the message.
+int check_paged_rows(const char *what, const int32_t *lens, const int32_t *block_table, int64_t bt_stride_b, int batch, int add,
+                     int page_size, int max_blocks, int num_blocks, int seqlen_ro, hipStream_t stream) {
+    if (batch <= 0) return FA_OK;
+    int *result = nullptr;
+    if (hipGetSymbolAddress((void **)&result, HIP_SYMBOL(g_check_result)) != hipSuccess || !result)
+        return fail(FA_ERR_LAUNCH, "FA_ROCM_VALIDATE: the result words of the check kernel have no device address");
+    int host[4] = {0, 0, 0, 0};
+    hipError_t e = hipMemcpyAsync(result, host, sizeof(host), hipMemcpyHostToDevice, stream);
+    if (e == hipSuccess) {
+        hipLaunchKernelGGL(check_paged_rows_kernel, dim3((batch + 255) / 256), dim3(256), 0, stream, lens, block_table, bt_stride_b, batch, add,
+                           page_size, max_blocks, num_blocks, seqlen_ro, result);
+        e = hipGetLastError();
+    }
+    if (e == hipSuccess) e = hipMemcpyAsync(host, result, sizeof(host), hipMemcpyDeviceToHost, stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(stream);
+    if (e != hipSuccess) return fail(FA_ERR_LAUNCH, "FA_ROCM_VALIDATE: %s", hipGetErrorString(e));
+    switch (host[0]) {
+        case kBadLength:
+            return fail(FA_ERR_SHAPE, "%s[%d] = %d is negative", what, host[1], host[2]);
+        case kBadCapacity:
+            return fail(FA_ERR_SHAPE, "batch row %d holds %d keys (%s + new tokens) but its block_table row addresses only %d", host[1], host[2],
+                        what, host[3]);
+        case kBadRotary:
+            return fail(FA_ERR_SHAPE, "batch row %d needs %d rotary positions but rotary_cos / rotary_sin have seqlen_ro = %d rows", host[1], host[2],
+                        host[3]);
+        case kBadPage:
+            return fail(FA_ERR_SHAPE, "block_table row %d names page %d; the cache has num_blocks = %d", host[1], host[2], host[3]);
+        default:
+            return FA_OK;
+    }
+}
+
 // bytes of the rotated copy of q that a tall query block with rotary embedding keeps at the start of
 // the workspace (a multiple of 256 so that the partials behind it stay aligned)
 size_t tall_q_bytes(const fa_kvcache_args *a) {
@@ -62,10 +165,8 @@ size_t tall_q_bytes(const fa_kvcache_args *a) {
 // Tallest query block (rows = seqlen_q * group) that runs on the decode kernels.
 int decode_max_rows(const fa_kvcache_args *a) {
     // tuning aid: FA_ROCM_DECODE_MAX_ROWS (16 or 32) overrides the rule
-    if (const char *env = std::getenv("FA_ROCM_DECODE_MAX_ROWS")) {
-        const int v = std::atoi(env);
-        if (v == 16 || v == 32) return v;
-    }
+    const int v = env().decode_max_rows;
+    if (v == 16 || v == 32) return v;
     (void)a;
     return fa::kDecodeMaxRows;
 }
@@ -96,6 +197,11 @@ size_t fa_rocm_sizeof_varlen_args(void) { return sizeof(fa_varlen_args); }
 size_t fa_rocm_sizeof_split_plan(void) { return sizeof(fa_split_plan); }
 
 int fa_rocm_num_cus(void) { return device_cus(); }
+
+void fa_rocm_reload_env(void) {
+    (void)env();
+    load_env();
+}
 
 int fa_rocm_kvcache_validate(const fa_kvcache_args *a) {
     if (!a) return fail(FA_ERR_NULL, "args is NULL");
@@ -137,6 +243,11 @@ int fa_rocm_kvcache_validate(const fa_kvcache_args *a) {
         if (a->headdim_qk != 64 && a->headdim_qk != 128 && a->headdim_qk != 256)
             return fail(FA_ERR_SHAPE, "head dimension must be 64, 128 or 256");
     }
+    // the combine and the explicit-split kernels put the batch and the units of a row (kv heads; for the latent cache
+    // query tokens x 128-head groups) in the grid's y / z extents
+    if (a->batch > 65535) return fail(FA_ERR_SHAPE, "batch size must be at most 65535");
+    if ((int64_t)a->nheads_k > 65535 || (is_mla_i8(a) && (int64_t)a->seqlen_q * (((int64_t)a->nheads + 127) / 128) > 65535))
+        return fail(FA_ERR_SHAPE, "too many units per batch row (kv heads, or query tokens x head groups): at most 65535");
     if ((a->k_new == nullptr) != (a->v_new == nullptr)) return fail(FA_ERR_NULL, "k and v must be passed together");
     if (a->k_new && a->seqlen_new <= 0) return fail(FA_ERR_SHAPE, "seqlen_new must be positive when k is given");
     if (!a->k_new && a->seqlen_new != 0) return fail(FA_ERR_SHAPE, "seqlen_new must be 0 without k");
@@ -162,9 +273,22 @@ int fa_rocm_plan_kvcache(const fa_kvcache_args *a, int num_cus, fa_split_plan *p
     if (!a || !plan) return fail(FA_ERR_NULL, "args or plan is NULL");
     if (num_cus <= 0) num_cus = 256;
     std::memset(plan, 0, sizeof(*plan));
-    if (a->batch <= 0 || a->seqlen_q <= 0) return fail(FA_ERR_SHAPE, "batch size and seqlen_q must be positive");
-    if (a->nheads <= 0 || a->nheads_k <= 0 || a->nheads % a->nheads_k != 0)
-        return fail(FA_ERR_SHAPE, "Number of heads in key/value must divide number of heads in query");
+    {
+        // The plan is defined for exactly the shapes the call accepts.  A caller that only plans may leave the tensor
+        // pointers NULL: they are stood in for here, so that the dimension checks of the validator decide alone.
+        fa_kvcache_args c = *a;
+        void *const some = &c;
+        if (!c.q) c.q = some;
+        if (!c.out) c.out = some;
+        if (!c.softmax_lse) c.softmax_lse = static_cast<float *>(some);
+        if (!c.k_cache && !c.v_cache) c.k_cache = c.v_cache = some;
+        if (!c.block_table) c.block_table = static_cast<const int32_t *>(some);
+        if (!c.cache_seqlens) c.cache_seqlens = static_cast<const int32_t *>(some);
+        if (is_mla_i8(&c) && !c.k_scale_cache) c.k_scale_cache = static_cast<float *>(some);
+        if (c.seqlen_new > 0 && !c.k_new && !c.v_new) c.k_new = c.v_new = some;
+        const int rc = fa_rocm_kvcache_validate(&c);
+        if (rc != FA_OK) return rc;
+    }
     const int group = a->nheads / a->nheads_k;
     // the int8 latent kernel works on units of 128 query heads and always uses the balanced partition
     const size_t rows = is_mla_i8(a) ? 128 : (size_t)a->seqlen_q * group;
@@ -203,20 +327,14 @@ int fa_rocm_plan_kvcache(const fa_kvcache_args *a, int num_cus, fa_split_plan *p
         // not cut below 4 chunks per workgroup (1 sequence x 8 K tokens: 46 -> 37 us)
         plan->min_share = is_mla_i8(a) ? 4 : 1;
         // tuning aid: FA_ROCM_DECODE_WGS overrides the workgroup count of the balanced partition
-        if (const char *env = std::getenv("FA_ROCM_DECODE_WGS")) {
-            const int v = std::atoi(env);
-            if (v > 0) plan->num_wgs = v;
-        }
+        if (env().decode_wgs > 0) plan->num_wgs = env().decode_wgs;
         // Query blocks of one 16-row tile: every wave is a worker with its own contiguous share (no
         // workgroup barrier anywhere in the stream); taller blocks and the latent kernel: the
         // workgroup is the worker.
-        const bool wave_workers = !is_mla_i8(a) && rows <= 16 && !std::getenv("FA_ROCM_DECODE_BLOCK_WORKERS");
+        const bool wave_workers = !is_mla_i8(a) && rows <= 16 && !env().block_workers;
         plan->num_workers = wave_workers ? plan->num_wgs * 4 : plan->num_wgs;
         if (wave_workers) plan->min_share = 2;   // short shares: the pipeline fill dominates tiny contexts otherwise
-        if (const char *env = std::getenv("FA_ROCM_MIN_SHARE")) {
-            const int v = std::atoi(env);
-            if (v > 0) plan->min_share = v;
-        }
+        if (env().min_share > 0) plan->min_share = env().min_share;
         // every worker writes at most two partials (the units cut at the two ends of its share)
         plan->workspace_bytes = (size_t)plan->num_workers * 2 * slot_bytes;
         return FA_OK;
@@ -283,8 +401,8 @@ static void fill_append(const fa_kvcache_args *a, fa::AppendParams &p) {
     p.vn_stride_h = a->vn_stride_h;
     p.bt_stride_b = a->bt_stride_b;
     // the scale tensors are inputs of attention and outputs of the quantising append
-    p.k_scale = const_cast<float *>(static_cast<const float *>(a->k_scale_cache));
-    p.v_scale = const_cast<float *>(static_cast<const float *>(a->v_scale_cache));
+    p.k_scale = a->k_scale_cache;
+    p.v_scale = a->v_scale_cache;
     p.ks_stride_block = a->ks_stride_block;
     p.ks_stride_row = a->ks_stride_row;
 }
@@ -314,6 +432,11 @@ static int fwd_kvcache_impl(const fa_kvcache_args *a, void *stream_, void *const
     int rc = fa_rocm_kvcache_validate(a);
     if (rc != FA_OK) return rc;
     hipStream_t stream = static_cast<hipStream_t>(stream_);
+    if (env().validate && q_live == nullptr) {
+        rc = check_paged_rows("cache_seqlens", a->cache_seqlens, a->block_table, a->bt_stride_b, a->batch, a->seqlen_new, a->page_size,
+                              a->max_blocks_per_seq, a->num_blocks, a->rotary_cos ? a->seqlen_ro : 0, stream);
+        if (rc != FA_OK) return rc;
+    }
     auto mark = [&](int i) {
         if (events) (void)hipEventRecord(static_cast<hipEvent_t>(events[i]), stream);
     };
@@ -526,9 +649,9 @@ static int fwd_kvcache_impl(const fa_kvcache_args *a, void *stream_, void *const
     // the critical path (c4 kernel 150 -> 145 us).  Wave-level kernel: ~6 us against ~5 us per chunk;
     // charging 1-3 chunks measured within +-1 %, so it is not charged.
     p.piece_cost = is_mla_i8(a) ? 7 : 0;
-    if (const char *env = std::getenv("FA_ROCM_PIECE_COST")) p.piece_cost = std::max(0, std::atoi(env));
+    if (env().piece_cost >= 0) p.piece_cost = env().piece_cost;
     p.head_interleave = p.wave_workers && a->nheads_k > 1 && plan.num_workers % a->nheads_k == 0 &&
-                        !std::getenv("FA_ROCM_NO_HEAD_INTERLEAVE");
+                        !env().no_head_interleave;
     const bool needs_combine = need > 0;
     if (needs_combine) {
         const size_t slot_rows = need / (((size_t)a->headdim_v + 1) * sizeof(float));
@@ -541,7 +664,7 @@ static int fwd_kvcache_impl(const fa_kvcache_args *a, void *stream_, void *const
     // exclude the oldest new key.  Otherwise the rows are written by their own kernel first.
     const bool fuse_append = a->k_new && p.balanced && p.wave_workers && (a->causal || a->window_right < 0) &&
                              (a->window_left < 0 || (int64_t)a->seqlen_q + a->window_left >= a->seqlen_new) &&
-                             !std::getenv("FA_ROCM_SEPARATE_APPEND");
+                             !env().separate_append;
     if (fuse_append) {
         p.k_new = a->k_new;
         p.v_new = a->v_new;
@@ -743,7 +866,7 @@ bool routes_short_blocks(const fa_varlen_args *a) {
     if (!a->block_table || a->total_q <= 0) return false;
     if (a->nheads / a->nheads_k > fa::kDecodeMaxRows) return false;
     if (a->max_seqlen_q > short_block_slots(a) && !uneven_blocks(a)) return false;
-    return std::getenv("FA_ROCM_NO_SHORT_BLOCKS") == nullptr;
+    return !env().no_short_blocks;
 }
 
 VarlenWorkspace varlen_workspace(const fa_varlen_args *a, int num_cus) {
@@ -836,6 +959,11 @@ int fa_rocm_varlen_fwd(const fa_varlen_args *a, void *stream_) {
     if (w.total > 0 && (!a->workspace || a->workspace_bytes < w.total))
         return fail(FA_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", w.total, a->workspace ? a->workspace_bytes : (size_t)0);
     hipStream_t stream = static_cast<hipStream_t>(stream_);
+    if (env().validate && a->block_table) {
+        const int rv = check_paged_rows("seqused_k", a->seqused_k, a->block_table, a->bt_stride_b, a->batch, 0, a->page_size,
+                                        a->max_blocks_per_seq, a->num_blocks, 0, stream);
+        if (rv != FA_OK) return rv;
+    }
     fa::ShortBlocksParams sr;
     std::memset(&sr, 0, sizeof(sr));
     if (w.short_blocks) {

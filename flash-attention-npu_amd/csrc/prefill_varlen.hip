@@ -610,24 +610,7 @@ __global__ void __launch_bounds__(256) prefill_combine_kernel(const PrefillParam
     if (lane == 0) p.lse[(int64_t)head * p.lse_stride_h + tok] = (tot > 0.f) ? (mx + fast_log2(tot)) * kLn2 : INFINITY;
 }
 
-// pack the heads of a GQA group into the tile rows when that saves at least a quarter of the tiles
-int prefill_pack(int group, int max_seqlen_q) {
-    const int tiles_plain = group * ((max_seqlen_q + kBM - 1) / kBM);
-    const int tiles_packed = (max_seqlen_q * group + kBM - 1) / kBM;
-    return (group > 1 && tiles_packed * 4 <= tiles_plain * 3) ? group : 1;
-}
-
-// token-major q whose blocks differ in length and whose average block would pack: every block decides
-// for itself (mixed prefill / decode batches)
-int prefill_pack_short(int group, int max_seqlen_q, int total_q, int batch) {
-    if (group <= 1 || batch <= 0 || total_q <= 0 || prefill_pack(group, max_seqlen_q) > 1) return 0;
-    return prefill_pack(group, (total_q + batch - 1) / batch) > 1 ? 1 : 0;
-}
-
-int prefill_tiles(int nheads, int nheads_k, int max_seqlen_q) {
-    const int pack = prefill_pack(nheads / nheads_k, max_seqlen_q);
-    return (pack > 1 ? nheads_k : nheads) * ((max_seqlen_q * pack + kBM - 1) / kBM);
-}
+static_assert(kBM == kPrefillTileRows, "the planning rules in fa_kernels.h assume this tile height");
 
 template <typename T, int D> static hipError_t launch_prefill_d(const PrefillParams &p_in, hipStream_t stream) {
     PrefillParams p = p_in;

@@ -56,6 +56,7 @@ class SplitPlan(C.Structure):
 
 EXPORTS = {
     "fa_rocm_abi_version": (C.c_int, []),
+    "fa_rocm_reload_env": (None, []),
     "fa_rocm_last_error": (C.c_char_p, []),
     "fa_rocm_sizeof_kvcache_args": (_sz, []),
     "fa_rocm_sizeof_varlen_args": (_sz, []),

@@ -185,6 +185,10 @@ def bind_kvcache(q, kcache, vcache, k_, v_, seqlens_k_, rotary_cos_, rotary_sin_
     _require(leftpad_k_ is None, "NPU FlashAttention does not support leftpad_k")
     _require(softcap >= 0.0, "softcap must be non-negative (0.0 disables softcap)")
     _require(q.dim() == 4 and kcache.dim() == 4 and vcache.dim() == 4, "q, kcache and vcache must be 4-D")
+    # the rotation is part of the append (positions cache_seqlens .. + seqlen_new of q and k); without new tokens the
+    # tables would be silently unused
+    _require((k_ is not None or v_ is not None) or (rotary_cos_ is None and rotary_sin_ is None),
+             "rotary_cos / rotary_sin are only applied together with new k / v")
     _require_device(q, kcache, vcache, k_, v_, seqlens_k_, block_table_, rotary_cos_, rotary_sin_)
 
     B, sq, hq, d = q.shape
@@ -288,8 +292,13 @@ def varlen_fwd(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k_, leftpad_k_
     _require(p_dropout == 0.0, "NPU FlashAttention does not support dropout")
     _require(not return_softmax, "NPU FlashAttention does not support return_softmax")
     _require(softcap >= 0.0, "softcap must be non-negative (0.0 disables softcap)")
-    _require_device(q, k, v, cu_seqlens_q, cu_seqlens_k, seqused_k_, block_table_)
+    # flash_api.cpp:890 (the outputs are written in full either way, nothing is left to clear)
+    _require(not zero_tensors, "NPU FlashAttention does not support zero_tensors.")
     paged = block_table_ is not None
+    # flash_api.cpp:886 rejects seqused_k always; here it is the length array of paged K/V and has no meaning for
+    # packed keys, whose lengths are the differences of cu_seqlens_k
+    _require(paged or seqused_k_ is None, "NPU FlashAttention does not support seqused_k.")
+    _require_device(q, k, v, cu_seqlens_q, cu_seqlens_k, seqused_k_, block_table_)
     total_q, hq, d = q.shape
     B = cu_seqlens_q.numel() - 1
     _require(B > 0, "batch size must be positive")

@@ -240,7 +240,7 @@ def _even_cu_seqlens(batch: int, seqlen: int, device) -> torch.Tensor:
     """cu_seqlens of `batch` sequences of `seqlen` tokens each, built once per (batch, seqlen, device)."""
     key = (batch, seqlen, str(device))
     if key not in _cu_cache:
-        _cu_cache[key] = torch.arange(0, (batch + 1) * seqlen, max(seqlen, 1), dtype=torch.int32, device=device)[: batch + 1]
+        _cu_cache[key] = torch.arange(batch + 1, dtype=torch.int32, device=device) * seqlen
     return _cu_cache[key]
 
 

@@ -4,9 +4,14 @@
  * Plain C: pointers, sizes, PODs.  No torch, no HIP types in the signatures (a
  * stream is passed as void* and must be a hipStream_t or NULL for the default
  * stream).  Every entry point enqueues work on the given stream and returns;
- * nothing here synchronises with the host, allocates device memory or keeps
- * mutable global state, so calls from several host threads on different
+ * nothing here synchronises with the host or allocates device memory, and the
+ * only process-wide state is read-only after the first call (the device's
+ * compute-unit count and the FA_ROCM_* environment settings, see
+ * fa_rocm_reload_env), so calls from several host threads on different
  * streams are safe.  The caller owns every buffer, including the workspace.
+ * Two exceptions, each described at its declaration: FA_ROCM_VALIDATE=1 makes
+ * the calls wait for a check kernel, and fa_rocm_fwd_kvcache_static keeps its
+ * partials in a device array of the library's own.
  *
  * Return value: 0 on success; a negative FA_ERR_* code otherwise, with a
  * human-readable message retrievable (per host thread) via fa_rocm_last_error().
@@ -52,9 +57,9 @@ typedef struct fa_kvcache_args {
     float *softmax_lse;          /* (B, Hq, Sq) fp32, natural log; +inf for rows with no key     */
     void *k_cache;               /* (num_blocks, page, Hk, Dqk) kv dtype; written when k_new set */
     void *v_cache;               /* (num_blocks, page, Hk, Dv)  kv dtype; may alias k_cache      */
-    const float *k_scale_cache;  /* (num_blocks, page, Hk) fp32 per-token scale; int8 cache only;
+    float *k_scale_cache;        /* (num_blocks, page, Hk) fp32 per-token scale; int8 cache only;
                                     written for the appended tokens when k_new is given         */
-    const float *v_scale_cache;  /* same for V; NULL = use k_scale_cache                         */
+    float *v_scale_cache;        /* same for V; NULL = use k_scale_cache                         */
     const void *k_new;           /* (B, Snew, Hk, Dqk) io dtype or NULL                          */
     const void *v_new;           /* (B, Snew, Hk, Dv)  io dtype or NULL                          */
     const void *rotary_cos;      /* (seqlen_ro, rotary_dim/2) io dtype or NULL                   */
@@ -149,6 +154,22 @@ size_t fa_rocm_sizeof_varlen_args(void);
 size_t fa_rocm_sizeof_split_plan(void);
 /* Compute units of the current HIP device (256 on MI355X); < 0 on error. */
 int fa_rocm_num_cus(void);
+
+/*
+ * The FA_ROCM_* environment variables are read once, by the first call that needs them; this reads them again
+ * (for tests and tuning scripts that change them inside a process; not safe beside calls running on other threads).
+ *   FA_ROCM_VALIDATE=1   debugging mode: before any work is queued, fa_rocm_fwd_kvcache* and fa_rocm_varlen_fwd (paged)
+ *                        run a check kernel over the data only the device holds and WAIT for it: negative lengths,
+ *                        cache_seqlens + seqlen_new beyond the pages of a block_table row (an append past the end),
+ *                        page ids outside [0, num_blocks), positions beyond seqlen_ro.  A violation returns
+ *                        FA_ERR_SHAPE naming the row; nothing is written.  Not usable under stream capture.
+ *                        Without it these cases are the caller's contract, as in the reference, whose host
+ *                        never reads the table either (csrc/ascend910/flash_attn_npu/flash_api.cpp:386-420).
+ *   FA_ROCM_DECODE_MAX_ROWS, FA_ROCM_DECODE_WGS, FA_ROCM_DECODE_BLOCK_WORKERS, FA_ROCM_MIN_SHARE, FA_ROCM_PIECE_COST,
+ *   FA_ROCM_NO_HEAD_INTERLEAVE, FA_ROCM_SEPARATE_APPEND, FA_ROCM_NO_SHORT_BLOCKS: experiment switches of the decode
+ *   partition and the kernel choice; results do not depend on them beyond rounding.
+ */
+void fa_rocm_reload_env(void);
 
 /*
  * Split-KV plan of a kvcache call, decided from shapes alone (per-row lengths stay on the device).

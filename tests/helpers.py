@@ -99,3 +99,26 @@ def check_compare_rule(out, ref_fp32, what="", rel=5e-3, floor=5e-3, share=0.995
     limit = torch.maximum(g.abs() * rel, torch.tensor(floor))
     ok = ((o - g).abs() <= limit).float().mean().item()
     assert ok >= share, f"{what}: only {100 * ok:.3f} % of the elements within max({rel}*|g|, {floor})"
+
+
+import contextlib
+
+
+@contextlib.contextmanager
+def library_env(**settings):
+    """Set FA_ROCM_* variables for the calls inside the block.  The library reads its environment once, so it is told
+    to read it again on the way in and on the way out."""
+    import os
+    from flash_attn_npu import _lib
+    old = {k: os.environ.get(k) for k in settings}
+    os.environ.update({k: str(v) for k, v in settings.items()})
+    _lib.load().fa_rocm_reload_env()
+    try:
+        yield
+    finally:
+        for k, v in old.items():
+            if v is None:
+                os.environ.pop(k, None)
+            else:
+                os.environ[k] = v
+        _lib.load().fa_rocm_reload_env()

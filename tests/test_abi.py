@@ -89,6 +89,42 @@ def test_validate_messages_follow_the_reference():
     assert lib.fa_rocm_kvcache_validate(None) != 0
 
 
+def test_grid_extent_limits_are_rejected_with_a_message():
+    # batch rows and the units of a row index the y / z extents of the explicit-split and combine grids (16 bits each)
+    lib = _lib.load()
+    a = good_args(); a.batch = 65535
+    assert lib.fa_rocm_kvcache_validate(C.byref(a)) == 0
+    a.batch = 65536
+    expect_error(a, "batch size must be at most 65535")
+    a = good_args(); a.nheads = a.nheads_k = 65536
+    expect_error(a, "too many units per batch row")
+    plan = _lib.SplitPlan()
+    a = good_args(); a.batch = 1 << 20
+    assert lib.fa_rocm_plan_kvcache(C.byref(a), 256, C.byref(plan)) == -3     # the planner accepts what the call accepts
+    a = good_args(); a.page_size = 0
+    assert lib.fa_rocm_plan_kvcache(C.byref(a), 256, C.byref(plan)) == -3
+    assert lib.fa_rocm_kvcache_workspace_bytes(C.byref(a), 256) == 0
+
+
+def test_environment_is_read_once_and_on_request(monkeypatch):
+    lib = _lib.load()
+    plan = _lib.SplitPlan()
+    a = good_args()
+    lib.fa_rocm_reload_env()
+    lib.fa_rocm_plan_kvcache(C.byref(a), 256, C.byref(plan))
+    assert plan.num_wgs == 512
+    monkeypatch.setenv("FA_ROCM_DECODE_WGS", "100")
+    lib.fa_rocm_plan_kvcache(C.byref(a), 256, C.byref(plan))
+    assert plan.num_wgs == 512, "the environment was read again on the call path"
+    lib.fa_rocm_reload_env()
+    lib.fa_rocm_plan_kvcache(C.byref(a), 256, C.byref(plan))
+    assert plan.num_wgs == 100
+    monkeypatch.delenv("FA_ROCM_DECODE_WGS")
+    lib.fa_rocm_reload_env()
+    lib.fa_rocm_plan_kvcache(C.byref(a), 256, C.byref(plan))
+    assert plan.num_wgs == 512
+
+
 def test_split_plan_invariants():
     lib = _lib.load()
     plan = _lib.SplitPlan()
@@ -142,6 +178,23 @@ def test_operator_layer_fails_loudly_without_gpu_tensors():
         flash_attn_varlen_func(x, x, x, cu, cu, 4, 4)
     with pytest.raises(RuntimeError, match="inference forward only"):
         flash_attn_varlen_func(x.requires_grad_(), x, x, cu, cu, 4, 4)
+    x = x.detach()
+    # arguments that would otherwise be ignored without a word (reference flash_api.cpp:886,890)
+    from flash_attn_npu.flash_attn_npu_interface import _varlen_forward_eager
+    with pytest.raises(RuntimeError, match="does not support zero_tensors"):
+        _varlen_forward_eager(x, x, x, cu, cu, 4, 4, 0.0, 0.1, False, zero_tensors=True)
+    with pytest.raises(RuntimeError, match="does not support seqused_k"):
+        _varlen_forward_eager(x, x, x, cu, cu, 4, 4, 0.0, 0.1, False, seqused_k=torch.tensor([4], dtype=torch.int32))
+    with pytest.raises(RuntimeError, match="only applied together with new k / v"):
+        flash_attn_with_kvcache(q, kc, kc, cache_seqlens=5, block_table=bt, rotary_cos=torch.zeros(8, 32, dtype=torch.bfloat16),
+                                rotary_sin=torch.zeros(8, 32, dtype=torch.bfloat16))
+
+
+def test_even_cu_seqlens_of_empty_sequences():
+    from flash_attn_npu.flash_attn_npu_interface import _even_cu_seqlens
+    assert _even_cu_seqlens(3, 0, "cpu").tolist() == [0, 0, 0, 0]
+    assert _even_cu_seqlens(3, 5, "cpu").tolist() == [0, 5, 10, 15]
+    assert _even_cu_seqlens(1, 7, "cpu").dtype == torch.int32
 
 
 def test_missing_library_is_an_error(monkeypatch):

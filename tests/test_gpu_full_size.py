@@ -9,7 +9,7 @@ import pytest
 import torch
 
 import fa_oracle as O
-from helpers import check_out
+from helpers import check_out, library_env
 
 pytestmark = pytest.mark.gpu
 
@@ -205,7 +205,7 @@ def test_c5_packed_prefill_full_size():
 
 
 @pytest.mark.parametrize("cost", [1, 5])
-def test_c2_partition_charging_unit_starts(cost, monkeypatch):
+def test_c2_partition_charging_unit_starts(cost):
     # the balanced partition with a fixed cost per unit start (the latent kernel's default; an
     # experiment knob for the others): other cuts of the same keys, same appended bytes, same result
     from bench import decode_workload
@@ -213,8 +213,8 @@ def test_c2_partition_charging_unit_starts(cost, monkeypatch):
     k0, v0 = w["k_cache"].clone(), w["v_cache"].clone()
     base = run_call(w)
     k1, v1 = w["k_cache"].clone(), w["v_cache"].clone()
-    monkeypatch.setenv("FA_ROCM_PIECE_COST", str(cost))
     print("full size c2: unit cost", cost, flush=True)
-    got = run_call(w, k_cache=k0, v_cache=v0)
+    with library_env(FA_ROCM_PIECE_COST=cost):
+        got = run_call(w, k_cache=k0, v_cache=v0)
     close_splits(base, got, f"unit cost {cost}")
     assert torch.equal(k0, k1) and torch.equal(v0, v1), "appended rows differ"

@@ -4,7 +4,7 @@ import pytest
 import torch
 
 import fa_oracle as O
-from helpers import check_compare_rule, check_out, check_vs_golden, make_paged_case, to_dev
+from helpers import check_compare_rule, check_out, check_vs_golden, library_env, make_paged_case, to_dev
 
 pytestmark = pytest.mark.gpu
 
@@ -341,11 +341,8 @@ def test_varlen_paged_short_blocks_on_the_decode_kernels(causal, window, softcap
     ref, ref_lse = O.flash_attn_varlen(q, kl, vl, cu_q, cu_k, max(lens_q), max(lens_k), causal=causal, window_size=window,
                                        softcap=softcap, mode="fp32")
     check_paged(out, ref, lse, ref_lse, "short blocks")
-    os.environ["FA_ROCM_NO_SHORT_BLOCKS"] = "1"
-    try:
+    with library_env(FA_ROCM_NO_SHORT_BLOCKS=1):
         out2, lse2 = call()
-    finally:
-        del os.environ["FA_ROCM_NO_SHORT_BLOCKS"]
     check_paged(out2, ref, lse2, ref_lse, "short blocks, tiled kernel only")
     short = torch.tensor([1 <= n <= 4 for n in lens_q for _ in range(n)])
     assert torch.equal(out[~short].cpu(), out2[~short].cpu()), "rows of the tiled kernel changed with the routing"

@@ -135,3 +135,84 @@ def test_latent_cache_beyond_2_31_bytes():
     check_out(out, ref, lse, ref_lse, "big latent cache")
     del kc, sc
     torch.cuda.empty_cache()
+
+
+def test_validate_mode_checks_what_only_the_device_knows():
+    """FA_ROCM_VALIDATE=1: page ids, capacities and rotary positions are checked by a kernel before anything is queued;
+    a violation is an error naming the row and the cache is left as it was.  A valid call gives the usual result."""
+    from flash_attn_npu import flash_attn_varlen_func, flash_attn_with_kvcache
+    from helpers import library_env, rotary_tables
+    lens = [100, 1, 0, 777, 64]
+    case = make_paged_case(len(lens), 32, 8, 128, 64, lens, seqlen_q=1, seqlen_new=1, seed=9)
+    dev = to_dev(case)
+
+    def call(d, **kw):
+        r = flash_attn_with_kvcache(d["q"], d["k_cache"], d["v_cache"], d["k"], d["v"], cache_seqlens=d["cache_seqlens"],
+                                    block_table=d["block_table"], causal=True, return_softmax_lse=True, **kw)
+        torch.cuda.synchronize()
+        return r
+
+    with library_env(FA_ROCM_VALIDATE=1):
+        print("validate mode: valid call", flush=True)
+        fresh = to_dev(case)
+        out, lse = call(fresh)
+        ref, ref_lse = O.flash_attn_with_kvcache(case["q"], case["k_cache"].clone(), case["v_cache"].clone(), case["k"], case["v"],
+                                                 cache_seqlens=case["cache_seqlens"], block_table=case["block_table"], causal=True, mode="fp32")
+        check_out(out, ref, lse, ref_lse, "validate mode")
+
+        before_k = dev["k_cache"].clone()
+        bad = dict(dev)
+        bad["block_table"] = dev["block_table"].clone()
+        bad["block_table"][3, 2] = dev["k_cache"].shape[0]           # one past the pool
+        print("validate mode: page id beyond the pool", flush=True)
+        with pytest.raises(RuntimeError, match=r"block_table row 3 names page \d+; the cache has num_blocks"):
+            call(bad)
+        bad["block_table"][3, 2] = -1
+        with pytest.raises(RuntimeError, match="block_table row 3 names page -1"):
+            call(bad)
+        # an id behind the used pages of a row is never read: not an error
+        ok = dict(dev)
+        ok["block_table"] = dev["block_table"].clone()
+        ok["k_cache"], ok["v_cache"] = dev["k_cache"].clone(), dev["v_cache"].clone()
+        ok["block_table"][1, 1:] = 1 << 30
+        call(ok)
+
+        bad = dict(dev)
+        bad["cache_seqlens"] = dev["cache_seqlens"].clone()
+        cap = dev["block_table"].shape[1] * 64
+        bad["cache_seqlens"][4] = cap                                # the appended token would fall behind the last page
+        print("validate mode: append beyond the pages", flush=True)
+        with pytest.raises(RuntimeError, match=rf"batch row 4 holds {cap + 1} keys .* addresses only {cap}"):
+            call(bad)
+        bad["cache_seqlens"][4] = -5
+        with pytest.raises(RuntimeError, match=r"cache_seqlens\[4\] = -5 is negative"):
+            call(bad)
+
+        cos, sin = rotary_tables(778, 128, dtype=torch.bfloat16)           # positions 0..777: row 3 appends at 777, the last one
+        cos, sin = cos.cuda(), sin.cuda()
+        ok = dict(dev)
+        ok["k_cache"], ok["v_cache"] = dev["k_cache"].clone(), dev["v_cache"].clone()
+        call(ok, rotary_cos=cos, rotary_sin=sin)
+        print("validate mode: position beyond the rotary tables", flush=True)
+        with pytest.raises(RuntimeError, match="batch row 3 needs 778 rotary positions but rotary_cos / rotary_sin have seqlen_ro = 777"):
+            call(dev, rotary_cos=cos[:777], rotary_sin=sin[:777])
+        assert torch.equal(dev["k_cache"], before_k), "a rejected call wrote to the cache"
+
+        # paged varlen: seqused_k and the table
+        total = sum(lens)
+        cu_q = torch.tensor([0, 3, 4, 4, 10, 12], dtype=torch.int32, device="cuda")
+        q = torch.randn(12, 32, 128, dtype=torch.bfloat16, device="cuda")
+        used = torch.tensor(lens, dtype=torch.int32, device="cuda")
+        from flash_attn_npu.flash_attn_npu_interface import _varlen_forward_eager
+        _varlen_forward_eager(q, dev["k_cache"], dev["v_cache"], cu_q, None, 6, 777, 0.0, 0.1, True, block_table=dev["block_table"], seqused_k=used)
+        bt = dev["block_table"].clone()
+        bt[0, 1] = dev["k_cache"].shape[0] + 7
+        print("validate mode: paged varlen", flush=True)
+        with pytest.raises(RuntimeError, match="block_table row 0 names page"):
+            _varlen_forward_eager(q, dev["k_cache"], dev["v_cache"], cu_q, None, 6, 777, 0.0, 0.1, True, block_table=bt, seqused_k=used)
+        used[2] = cap + 1
+        with pytest.raises(RuntimeError, match="batch row 2 holds"):
+            _varlen_forward_eager(q, dev["k_cache"], dev["v_cache"], cu_q, None, 6, 777, 0.0, 0.1, True, block_table=dev["block_table"],
+                                  seqused_k=used)
+        torch.cuda.synchronize()
+    del total

@@ -17,8 +17,9 @@ def plan_of(batch, sq, hq, hk, d, max_blocks, page=256, num_splits=0, rotary=Fal
         a.rotary_cos = a.rotary_sin = 256   # only tested for being non-NULL by the planner
         a.k_new = a.v_new = 256
         a.seqlen_new = sq
+        a.rotary_dim, a.seqlen_ro = d, 1 << 20
     plan = _lib.SplitPlan()
-    assert lib.fa_rocm_plan_kvcache(C.byref(a), 256, C.byref(plan)) == 0
+    assert lib.fa_rocm_plan_kvcache(C.byref(a), 256, C.byref(plan)) == 0, _lib.last_error()
     return plan
 
 
