@@ -195,11 +195,13 @@ __device__ __forceinline__ void combine_row_wave(const DecodeParams &p, int b, i
     const int qi = rid.qi, head = rid.head;
     uint16_t *dst = reinterpret_cast<uint16_t *>(p.out) + (int64_t)b * p.o_stride_b + (int64_t)qi * p.o_stride_s +
                     (int64_t)head * p.o_stride_h + lane * CPL;
-    if constexpr (CPL == 1) {
-        dst[0] = from_float<T>(acc[0] * inv);
-    } else {
+    if (lane * CPL < p.headdim) {   // the partials are DV wide; the output row ends at the head dimension
+        if constexpr (CPL == 1) {
+            dst[0] = from_float<T>(acc[0] * inv);
+        } else {
 #pragma unroll
-        for (int c = 0; c < CPL; c += 2) *reinterpret_cast<uint32_t *>(dst + c) = pack2<T>(acc[c] * inv, acc[c + 1] * inv);
+            for (int c = 0; c < CPL; c += 2) *reinterpret_cast<uint32_t *>(dst + c) = pack2<T>(acc[c] * inv, acc[c + 1] * inv);
+        }
     }
     if (lane == 0)
         p.lse[((int64_t)b * p.nheads + head) * p.seqlen_q + qi] = (tot > 0.f) ? (mx + fast_log2(tot)) * kLn2 : INFINITY;
@@ -212,7 +214,7 @@ template <int DV> __device__ __forceinline__ void init_empty_unit(const DecodePa
         const int piece = idx - row * (DV / 8);
         const RowId rid = row_id(p, kvh, row);
         const int qi = rid.qi, head = rid.head;
-        if (head >= p.nheads) continue;
+        if (head >= p.nheads || piece * 8 >= p.headdim) continue;
         uint16_t *dst = reinterpret_cast<uint16_t *>(p.out) + (int64_t)b * p.o_stride_b + (int64_t)qi * p.o_stride_s +
                         (int64_t)head * p.o_stride_h + piece * 8;
         store16(dst, u32x4_t{0, 0, 0, 0});

@@ -36,7 +36,9 @@ template <int D> __device__ __forceinline__ int k_tile_offset(int row, int ch) {
 
 // One piece of work: query block (b, kvh) against keys [range_lo, range_hi).  Writes the final
 // output when `write_final`, else the normalised fp32 partial and its base-2 LSE into `slot`.
-template <typename T, int D, int RT, int NW, bool SOFTCAP>
+// PART: the head dimension p.headdim is below D.  Lanes whose 16-byte pieces of a K / V row lie behind it load nothing
+// and hold zeros, k-steps that only see such pieces are skipped, and the stores stop at the head dimension.
+template <typename T, int D, int RT, int NW, bool SOFTCAP, bool PART>
 __device__ __forceinline__ void process_piece(const DecodeParams &p, const int b, const int kvh, const UnitRange &ur,
                                               const int range_lo, const int range_hi, const bool write_final,
                                               const int64_t slot) {
@@ -98,6 +100,21 @@ __device__ __forceinline__ void process_piece(const DecodeParams &p, const int b
 
     u32x4_t kreg[Cfg::kKLoads];
     uint32_t vreg[8][Cfg::kVH][Cfg::kVW / 2];
+    const int hd = PART ? p.headdim : D;
+    const bool k_live = !PART || (lane % Cfg::kLanesPerRow) * 8 < hd;
+    bool v_live[Cfg::kVH];
+#pragma unroll
+    for (int hh = 0; hh < Cfg::kVH; ++hh) v_live[hh] = !PART || hh * 128 + ln * Cfg::kVW < hd;
+    if constexpr (PART) {
+#pragma unroll
+        for (int j = 0; j < Cfg::kKLoads; ++j) kreg[j] = u32x4_t{0, 0, 0, 0};
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+#pragma unroll
+            for (int hh = 0; hh < Cfg::kVH; ++hh)
+#pragma unroll
+                for (int w2 = 0; w2 < Cfg::kVW / 2; ++w2) vreg[e][hh][w2] = 0u;
+    }
 
     // per-lane byte offsets inside a page that do not change from chunk to chunk; the per-load
     // part is wave-uniform and folds into the scalar base address
@@ -142,27 +159,36 @@ __device__ __forceinline__ void process_piece(const DecodeParams &p, const int b
         const uint8_t *kb = kc_base + (int64_t)blk * p.k_stride_block * 2 + (int64_t)inpage0 * k_row_bytes;
         const uint8_t *vb = vc_base + (int64_t)blk * p.v_stride_block * 2 + (int64_t)inpage0 * v_row_bytes;
         if (last >= kChunk - 1) {
+            if (k_live) {
 #pragma unroll
-            for (int j = 0; j < Cfg::kKLoads; ++j)
-                kreg[j] = load16_stream(kb + (size_t)(j * Cfg::kRowsPerLoad) * k_row_bytes + k_lane_off);
+                for (int j = 0; j < Cfg::kKLoads; ++j)
+                    kreg[j] = load16_stream(kb + (size_t)(j * Cfg::kRowsPerLoad) * k_row_bytes + k_lane_off);
+            }
 #pragma unroll
-            for (int e = 0; e < 8; ++e)
+            for (int hh = 0; hh < Cfg::kVH; ++hh)
+                if (v_live[hh]) {
 #pragma unroll
-                for (int hh = 0; hh < Cfg::kVH; ++hh)
-                    load_v(vb + (size_t)((e >> 2) * 16 + (e & 3)) * v_row_bytes + hh * 256 + v_lane_off, e, hh);
+                    for (int e = 0; e < 8; ++e)
+                        load_v(vb + (size_t)((e >> 2) * 16 + (e & 3)) * v_row_bytes + hh * 256 + v_lane_off, e, hh);
+                }
         } else {
             // tail chunk: rows past the last written key re-read that key (their scores are masked)
+            if (k_live) {
 #pragma unroll
-            for (int j = 0; j < Cfg::kKLoads; ++j) {
-                const int row = min(j * Cfg::kRowsPerLoad + k_lane_row, last);
-                kreg[j] = load16(kb + (uint32_t)row * k_row_bytes + k_lane_col);
+                for (int j = 0; j < Cfg::kKLoads; ++j) {
+                    const int row = min(j * Cfg::kRowsPerLoad + k_lane_row, last);
+                    kreg[j] = load16(kb + (uint32_t)row * k_row_bytes + k_lane_col);
+                }
             }
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const int row = min((e >> 2) * 16 + lq * 4 + (e & 3), last);
+            for (int hh = 0; hh < Cfg::kVH; ++hh)
+                if (v_live[hh]) {
 #pragma unroll
-                for (int hh = 0; hh < Cfg::kVH; ++hh) load_v(vb + (uint32_t)row * v_row_bytes + v_lane_col + hh * 256, e, hh);
-            }
+                    for (int e = 0; e < 8; ++e) {
+                        const int row = min((e >> 2) * 16 + lq * 4 + (e & 3), last);
+                        load_v(vb + (uint32_t)row * v_row_bytes + v_lane_col + hh * 256, e, hh);
+                    }
+                }
         }
     };
 
@@ -191,7 +217,7 @@ __device__ __forceinline__ void process_piece(const DecodeParams &p, const int b
                 d2 = d1 + 1;
             }
             uint16_t o1 = 0, o2 = 0;
-            if (row < p.rows) {
+            if (row < p.rows && (!PART || c < hd / 2)) {   // pairs behind the head dimension stay zero (c < hd/2 <=> d1, d2 < hd)
                 const int qi = row / p.group;
                 const int g = row - qi * p.group;
                 const uint16_t *src = qbase + (int64_t)qi * p.q_stride_s + (int64_t)(kvh * p.group + g) * p.q_stride_h;
@@ -258,7 +284,8 @@ __device__ __forceinline__ void process_piece(const DecodeParams &p, const int b
 #pragma unroll
             for (int r = 0; r < RT; ++r) s[tt][r] = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int t = 0; t < Cfg::kKSteps; ++t)
+        for (int t = 0; t < Cfg::kKSteps; ++t) {
+            if (PART && t * 32 >= hd) continue;   // wave-uniform
 #pragma unroll
             for (int tt = 0; tt < 2; ++tt) {
                 const u32x4_t a =
@@ -266,6 +293,7 @@ __device__ __forceinline__ void process_piece(const DecodeParams &p, const int b
 #pragma unroll
                 for (int r = 0; r < RT; ++r) s[tt][r] = mfma16<T>(a, qreg[r][t], s[tt][r]);
             }
+        }
 
         // ---- online softmax per query row (lane column ln of tile r)
         const int key_base = c * kChunk + lq * 4;
@@ -410,6 +438,7 @@ __device__ __forceinline__ void process_piece(const DecodeParams &p, const int b
         const int g = row - qi * p.group;
         const int head = kvh * p.group + g;
         if (write_final) {
+            if (PART && piece * 8 >= hd) continue;
             u32x4_t o4;
             o4[0] = pack2<T>(v[0], v[1]);
             o4[1] = pack2<T>(v[2], v[3]);
@@ -432,7 +461,7 @@ __device__ __forceinline__ void process_piece(const DecodeParams &p, const int b
 }
 
 // ---- grid mode: blockIdx = (split, kv head, batch row), fixed keys per split -------------------
-template <typename T, int D, int RT, int NW, bool SOFTCAP>
+template <typename T, int D, int RT, int NW, bool SOFTCAP, bool PART>
 __global__ void __launch_bounds__(NW * 64, (D <= 128 && RT <= 2) ? 2 : 1)
 decode_paged_kernel(const DecodeParams p) {
     const int split = blockIdx.x;
@@ -451,7 +480,7 @@ decode_paged_kernel(const DecodeParams p) {
         range_hi = (split == nsplits_row - 1) ? ur.hi : min(ur.hi, lo_al + (split + 1) * p.split_keys);
     }
     const int64_t slot = ((int64_t)b * p.nheads_k + kvh) * p.nsplits + split;
-    process_piece<T, D, RT, NW, SOFTCAP>(p, b, kvh, ur, range_lo, range_hi, nsplits_row == 1, slot);
+    process_piece<T, D, RT, NW, SOFTCAP, PART>(p, b, kvh, ur, range_lo, range_hi, nsplits_row == 1, slot);
 }
 
 // ---- balanced mode ---------------------------------------------------------------------------
@@ -461,12 +490,12 @@ decode_paged_kernel(const DecodeParams p) {
 // every workgroup for itself from the device-resident lengths.  A workgroup writes the final
 // output of every unit that lies wholly inside its share and at most two partials.
 
-template <typename T, int D, int RT, int NW, bool SOFTCAP>
+template <typename T, int D, int RT, int NW, bool SOFTCAP, bool PART>
 __global__ void __launch_bounds__(NW * 64, (D <= 128 && RT <= 2) ? 2 : 1)
 decode_balanced_kernel(const DecodeParams p) {
     static_assert(NW == 4, "the batch scan assumes 256 threads");
     balanced_driver<D>(p, [&](int b, int kvh, const UnitRange &ur, int range_lo, int range_hi, bool whole, int64_t slot) {
-        process_piece<T, D, RT, NW, SOFTCAP>(p, b, kvh, ur, range_lo, range_hi, whole, slot);
+        process_piece<T, D, RT, NW, SOFTCAP, PART>(p, b, kvh, ur, range_lo, range_hi, whole, slot);
     });
 }
 
@@ -547,7 +576,7 @@ __device__ __forceinline__ void combine_row_block(const DecodeParams &p, int b, 
         uint2 o2;
         o2.x = pack2<T>(acc[0] * inv, acc[1] * inv);
         o2.y = pack2<T>(acc[2] * inv, acc[3] * inv);
-        *reinterpret_cast<uint2 *>(out_row + cg * 4) = o2;
+        if (cg * 4 < p.headdim) *reinterpret_cast<uint2 *>(out_row + cg * 4) = o2;
         if (cg == 0)
             p.lse[((int64_t)b * p.nheads + head) * p.seqlen_q + qi] = (tot > 0.f) ? (mx + fast_log2(tot)) * kLn2 : INFINITY;
     }
@@ -582,25 +611,23 @@ __global__ void __launch_bounds__(256) splitkv_combine_balanced_kernel(const Dec
         if (row_id(p, kvh, row).head < p.nheads) combine_row_block<T, D>(p, b, kvh, row, pcs);   // block-uniform
 }
 
+template <typename T, int D, int RT, bool SOFTCAP, bool PART>
+static hipError_t launch_decode_sp(const DecodeParams &p, hipStream_t stream) {
+    constexpr int NW = 4;
+    if (p.balanced)
+        hipLaunchKernelGGL((decode_balanced_kernel<T, D, RT, NW, SOFTCAP, PART>), dim3(p.num_wgs), dim3(NW * 64), 0, stream, p);
+    else
+        hipLaunchKernelGGL((decode_paged_kernel<T, D, RT, NW, SOFTCAP, PART>), dim3(p.nsplits, p.nheads_k, p.batch), dim3(NW * 64), 0,
+                           stream, p);
+    return hipGetLastError();
+}
+
 template <typename T, int D, int RT>
 static hipError_t launch_decode_rt(const DecodeParams &p, hipStream_t stream) {
-    constexpr int NW = 4;
-    dim3 block(NW * 64);
+    if (p.headdim > D || p.headdim < 8 || p.headdim % 8 != 0) return hipErrorInvalidValue;
     const bool softcap = p.softcap_post != 0.f;
-    if (p.balanced) {
-        dim3 grid(p.num_wgs);
-        if (softcap)
-            hipLaunchKernelGGL((decode_balanced_kernel<T, D, RT, NW, true>), grid, block, 0, stream, p);
-        else
-            hipLaunchKernelGGL((decode_balanced_kernel<T, D, RT, NW, false>), grid, block, 0, stream, p);
-    } else {
-        dim3 grid(p.nsplits, p.nheads_k, p.batch);
-        if (softcap)
-            hipLaunchKernelGGL((decode_paged_kernel<T, D, RT, NW, true>), grid, block, 0, stream, p);
-        else
-            hipLaunchKernelGGL((decode_paged_kernel<T, D, RT, NW, false>), grid, block, 0, stream, p);
-    }
-    return hipGetLastError();
+    if (p.headdim < D) return softcap ? launch_decode_sp<T, D, RT, true, true>(p, stream) : launch_decode_sp<T, D, RT, false, true>(p, stream);
+    return softcap ? launch_decode_sp<T, D, RT, true, false>(p, stream) : launch_decode_sp<T, D, RT, false, false>(p, stream);
 }
 
 template <typename T, int D> static hipError_t launch_decode_d(const DecodeParams &p, hipStream_t stream) {

@@ -29,7 +29,7 @@ template <int D> struct WaveCfg {
 // Stage the 16-row query tile of unit (b, kvh), rotated if requested, into this wave's LDS rows.
 // Work item = one 16-byte piece of one row; in the non-interleaved rotary region the item of a
 // first-half piece also produces its partner piece rot/2 elements further on.
-template <typename T, int D>
+template <typename T, int D, bool PART>
 __device__ __forceinline__ void stage_q_wave(const DecodeParams &p, int b, int kvh, int len_cache, uint16_t *sq) {
     using Cfg = WaveCfg<D>;
     const int lane = threadIdx.x & 63;
@@ -43,7 +43,7 @@ __device__ __forceinline__ void stage_q_wave(const DecodeParams &p, int b, int k
         const int ci = item - row * Cfg::kPiecesPerRow;
         const int d0 = ci * 8;
         uint16_t *dst = sq + row * D + d0;
-        if (row >= p.rows) {
+        if (row >= p.rows || (PART && d0 >= p.headdim)) {   // padding rows, and the columns behind a head dimension below D
             *reinterpret_cast<u32x4_t *>(dst) = u32x4_t{0, 0, 0, 0};
             continue;
         }
@@ -124,7 +124,7 @@ __device__ __forceinline__ void append_rows_wave(const DecodeParams &p, int b, i
         const uint16_t *vsrc = reinterpret_cast<const uint16_t *>(p.v_new) + (int64_t)b * p.vn_stride_b +
                                (int64_t)t * p.vn_stride_s + (int64_t)kvh * p.vn_stride_h;
         const int rpos = min(pos, p.seqlen_ro - 1);
-        for (int c = lane; c < D / 2; c += 64) {
+        for (int c = lane; c < p.headdim / 2; c += 64) {
             int d1, d2;
             if (c < half) {
                 d1 = p.rotary_interleaved ? 2 * c : c;
@@ -146,13 +146,16 @@ __device__ __forceinline__ void append_rows_wave(const DecodeParams &p, int b, i
             kdst[d1] = o1;
             kdst[d2] = o2;
         }
-        for (int d = lane; d < D; d += 64) vdst[d] = vsrc[d];
+        for (int d = lane; d < p.headdim; d += 64) vdst[d] = vsrc[d];
     }
     // the wave's own later loads of these rows must find them
     __threadfence_block();
 }
 
-template <typename T, int D, bool SOFTCAP>
+// PART: the head dimension p.headdim is below D (a multiple of 8 above D/2, or below 64 for D = 64).  The lanes whose
+// 16-byte pieces of a K / V row lie behind it load nothing and hold zeros, the k-steps and output tiles that only
+// see such pieces are skipped, and the stores stop at the head dimension.
+template <typename T, int D, bool SOFTCAP, bool PART>
 __device__ __forceinline__ void wave_piece(const DecodeParams &p, const int b, const int kvh, const UnitRange &ur,
                                            const int range_lo, const int range_hi, const bool write_final,
                                            const int64_t slot, uint8_t *ktile, uint16_t *sq) {
@@ -172,6 +175,21 @@ __device__ __forceinline__ void wave_piece(const DecodeParams &p, const int b, c
 
     u32x4_t kreg[Cfg::kKLoads];
     uint32_t vreg[8][Cfg::kVH][Cfg::kVW / 2];
+    const int hd = PART ? p.headdim : D;
+    const bool k_live = !PART || (lane % Cfg::kLanesPerRow) * 8 < hd;
+    bool v_live[Cfg::kVH];
+#pragma unroll
+    for (int hh = 0; hh < Cfg::kVH; ++hh) v_live[hh] = !PART || hh * 128 + ln * Cfg::kVW < hd;
+    if constexpr (PART) {
+#pragma unroll
+        for (int j = 0; j < Cfg::kKLoads; ++j) kreg[j] = u32x4_t{0, 0, 0, 0};
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+#pragma unroll
+            for (int hh = 0; hh < Cfg::kVH; ++hh)
+#pragma unroll
+                for (int w2 = 0; w2 < Cfg::kVW / 2; ++w2) vreg[e][hh][w2] = 0u;
+    }
     const uint32_t k_row_bytes = (uint32_t)p.k_stride_row * 2u;
     const uint32_t v_row_bytes = (uint32_t)p.v_stride_row * 2u;
     const int k_lane_row = lane / Cfg::kLanesPerRow;
@@ -210,27 +228,36 @@ __device__ __forceinline__ void wave_piece(const DecodeParams &p, const int b, c
         const uint8_t *kb = kc_base + (int64_t)blk * p.k_stride_block * 2 + (int64_t)inpage0 * k_row_bytes;
         const uint8_t *vb = vc_base + (int64_t)blk * p.v_stride_block * 2 + (int64_t)inpage0 * v_row_bytes;
         if (last >= kChunk - 1) {
+            if (k_live) {
 #pragma unroll
-            for (int j = 0; j < Cfg::kKLoads; ++j)
-                kreg[j] = load16_stream(kb + (size_t)(j * Cfg::kRowsPerLoad) * k_row_bytes + k_lane_off);
+                for (int j = 0; j < Cfg::kKLoads; ++j)
+                    kreg[j] = load16_stream(kb + (size_t)(j * Cfg::kRowsPerLoad) * k_row_bytes + k_lane_off);
+            }
 #pragma unroll
-            for (int e = 0; e < 8; ++e)
+            for (int hh = 0; hh < Cfg::kVH; ++hh)
+                if (v_live[hh]) {
 #pragma unroll
-                for (int hh = 0; hh < Cfg::kVH; ++hh)
-                    load_v(vb + (size_t)((e >> 2) * 16 + (e & 3)) * v_row_bytes + hh * 256 + v_lane_off, e, hh);
+                    for (int e = 0; e < 8; ++e)
+                        load_v(vb + (size_t)((e >> 2) * 16 + (e & 3)) * v_row_bytes + hh * 256 + v_lane_off, e, hh);
+                }
         } else {
             // tail chunk: rows past the last written key re-read that key (their scores are masked)
+            if (k_live) {
 #pragma unroll
-            for (int j = 0; j < Cfg::kKLoads; ++j) {
-                const int row = min(j * Cfg::kRowsPerLoad + k_lane_row, last);
-                kreg[j] = load16(kb + (uint32_t)row * k_row_bytes + k_lane_col);
+                for (int j = 0; j < Cfg::kKLoads; ++j) {
+                    const int row = min(j * Cfg::kRowsPerLoad + k_lane_row, last);
+                    kreg[j] = load16(kb + (uint32_t)row * k_row_bytes + k_lane_col);
+                }
             }
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const int row = min((e >> 2) * 16 + lq * 4 + (e & 3), last);
+            for (int hh = 0; hh < Cfg::kVH; ++hh)
+                if (v_live[hh]) {
 #pragma unroll
-                for (int hh = 0; hh < Cfg::kVH; ++hh) load_v(vb + (uint32_t)row * v_row_bytes + v_lane_col + hh * 256, e, hh);
-            }
+                    for (int e = 0; e < 8; ++e) {
+                        const int row = min((e >> 2) * 16 + lq * 4 + (e & 3), last);
+                        load_v(vb + (uint32_t)row * v_row_bytes + v_lane_col + hh * 256, e, hh);
+                    }
+                }
         }
     };
 
@@ -242,7 +269,7 @@ __device__ __forceinline__ void wave_piece(const DecodeParams &p, const int b, c
     if (c < c_end) issue_loads(c, blk_next);
     blk_next = fetch_blk(c + 1);
 
-    stage_q_wave<T, D>(p, b, kvh, ur.len_cache, sq);
+    stage_q_wave<T, D, PART>(p, b, kvh, ur.len_cache, sq);
     __builtin_amdgcn_wave_barrier();
     u32x4_t qreg[Cfg::kKSteps];
 #pragma unroll
@@ -302,7 +329,8 @@ __device__ __forceinline__ void wave_piece(const DecodeParams &p, const int b, c
         // S^T = K Q^T, two 16-key tiles
         float4_t s[2] = {float4_t{0.f, 0.f, 0.f, 0.f}, float4_t{0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
-        for (int t = 0; t < Cfg::kKSteps; ++t)
+        for (int t = 0; t < Cfg::kKSteps; ++t) {
+            if (PART && t * 32 >= hd) continue;   // wave-uniform
 #pragma unroll
             for (int tt = 0; tt < 2; ++tt) {
                 const int row = tt * 16 + ln;
@@ -310,6 +338,7 @@ __device__ __forceinline__ void wave_piece(const DecodeParams &p, const int b, c
                     ktile + row * (D * 2) + (((t * 4 + lq) ^ (row & Cfg::kSwzMask)) << 4));
                 s[tt] = mfma16<T>(a, qreg[t], s[tt]);
             }
+        }
 
         // online softmax of query row ln; register i of tile tt is key c*32 + tt*16 + lq*4 + i
         const int key_base = c * kChunk + lq * 4;
@@ -354,6 +383,7 @@ __device__ __forceinline__ void wave_piece(const DecodeParams &p, const int b, c
             o_acc[t][2] *= alpha;
             o_acc[t][3] *= alpha;
         }
+        // (every column tile interleaves columns of the whole 128-column pass, so none is dead as a whole)
 #pragma unroll
         for (int t = 0; t < Cfg::kColTiles; ++t) o_acc[t] = mfma16<T>(vt[t], pk, o_acc[t]);
         c = cn;
@@ -373,6 +403,7 @@ __device__ __forceinline__ void wave_piece(const DecodeParams &p, const int b, c
             for (int hh = 0; hh < Cfg::kVH; ++hh)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
+                    if (PART && hh * 128 + (lq * 4 + i) * Cfg::kVW >= hd) continue;
                     uint16_t *d2 = dst + hh * 128 + (lq * 4 + i) * Cfg::kVW;
 #pragma unroll
                     for (int w = 0; w < Cfg::kVW; w += 2)
@@ -400,7 +431,7 @@ __device__ __forceinline__ void wave_piece(const DecodeParams &p, const int b, c
     __builtin_amdgcn_wave_barrier();   // the wave's LDS rows are reused by its next piece
 }
 
-template <typename T, int D, bool SOFTCAP>
+template <typename T, int D, bool SOFTCAP, bool PART>
 __global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) decode_wave_kernel(const DecodeParams p) {
     using Cfg = WaveCfg<D>;
     __shared__ int s_pref[257];
@@ -410,17 +441,26 @@ __global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) decode_wave_kernel(co
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     walk_share(p, pt, s_pref, (int64_t)blockIdx.x * 4 + wave,
                [&](int b, int kvh, const UnitRange &ur, int range_lo, int range_hi, bool whole, int64_t slot) {
-                   wave_piece<T, D, SOFTCAP>(p, b, kvh, ur, range_lo, range_hi, whole, slot, s_k[wave], s_q[wave]);
+                   wave_piece<T, D, SOFTCAP, PART>(p, b, kvh, ur, range_lo, range_hi, whole, slot, s_k[wave], s_q[wave]);
                });
     init_empty_units<D>(p, pt);
 }
 
 template <typename T, int D> static hipError_t launch_wave_d(const DecodeParams &p, hipStream_t stream) {
     dim3 grid(p.num_wgs), block(256);
-    if (p.softcap_post != 0.f)
-        hipLaunchKernelGGL((decode_wave_kernel<T, D, true>), grid, block, 0, stream, p);
-    else
-        hipLaunchKernelGGL((decode_wave_kernel<T, D, false>), grid, block, 0, stream, p);
+    if (p.headdim > D || p.headdim < 8 || p.headdim % 8 != 0) return hipErrorInvalidValue;
+    const bool part = p.headdim < D;
+    if (p.softcap_post != 0.f) {
+        if (part)
+            hipLaunchKernelGGL((decode_wave_kernel<T, D, true, true>), grid, block, 0, stream, p);
+        else
+            hipLaunchKernelGGL((decode_wave_kernel<T, D, true, false>), grid, block, 0, stream, p);
+    } else {
+        if (part)
+            hipLaunchKernelGGL((decode_wave_kernel<T, D, false, true>), grid, block, 0, stream, p);
+        else
+            hipLaunchKernelGGL((decode_wave_kernel<T, D, false, false>), grid, block, 0, stream, p);
+    }
     return hipGetLastError();
 }
 

@@ -28,6 +28,8 @@ struct DecodeParams {
     float *o_partial;    // (B, Hk, nsplits, rows, Dv) fp32, each normalised by its own sum
     float *lse_partial;  // (B, Hk, nsplits, rows)     fp32, base-2 log-sum-exp, -inf when empty
     int32_t batch, seqlen_q, nheads, nheads_k, group, rows;  // rows = seqlen_q * group
+    int32_t headdim;     // columns of an output row (and of a q / k / v row, except for the latent cache): a multiple of 8;
+                         // the kernels' compile-time width is tile_headdim() of it and the partials are that wide
     int32_t seqlen_new, num_blocks, page_size, max_blocks;
     int32_t rotary_dim, seqlen_ro, rotary_interleaved, rotary_per_token;
     int64_t q_stride_b, q_stride_s, q_stride_h;
@@ -120,6 +122,7 @@ struct PrefillParams {
     const int32_t *seqused_k;      // paged: keys per row (cache_seqlens)
     const int32_t *block_table;    // NULL: dense K/V
     int32_t batch, nheads, nheads_k, group;
+    int32_t headdim;               // columns of a q / k / v / out row, a multiple of 8; the kernel is compiled for tile_headdim() of it
     int32_t pack;                  // set by the launcher: 1, or group when tile rows are (query, head) pairs
     int32_t pack_short;            // set by the launcher: pack == 1, but a short query block packs its heads on its own
     int32_t skip_short;            // token-major q: sequences with 1 .. skip_short query tokens are computed elsewhere (0 = none)
@@ -150,6 +153,9 @@ struct PrefillParams {
     float *o_partial;
     float *lse_partial;
 };
+
+// Width the kernels are compiled for, for a head dimension of d columns.
+inline int tile_headdim(int d) { return d <= 64 ? 64 : d <= 128 ? 128 : 256; }
 
 // ---- planning rules shared by the host API and the launchers (host integer code; 64-bit inside so that no
 // combination of 32-bit dimensions overflows) ----

@@ -51,6 +51,9 @@ int device_cus() {
 
 bool is_mla_i8(const fa_kvcache_args *a) { return a->kv_dtype == FA_INT8; }
 
+// columns of a row of fp32 partials: the width the kernels are compiled for
+int partial_width(const fa_kvcache_args *a) { return is_mla_i8(a) ? a->headdim_v : fa::tile_headdim(a->headdim_v); }
+
 // Experiment knobs and the validation switch, from the environment.  They are read ONCE, on the first call that
 // needs them (or again when fa_rocm_reload_env() is called): nothing on the call path touches the environment.
 struct EnvKnobs {
@@ -240,8 +243,8 @@ int fa_rocm_kvcache_validate(const fa_kvcache_args *a) {
     } else {
         if (a->headdim_qk > 256) return fail(FA_ERR_SHAPE, "FlashAttention only supports head dimension at most 256");
         if (a->headdim_qk != a->headdim_v) return fail(FA_ERR_SHAPE, "k and v head dimensions must match");
-        if (a->headdim_qk != 64 && a->headdim_qk != 128 && a->headdim_qk != 256)
-            return fail(FA_ERR_SHAPE, "head dimension must be 64, 128 or 256");
+        if (a->headdim_qk < 8 || a->headdim_qk % 8 != 0)
+            return fail(FA_ERR_SHAPE, "head dimension must be a positive multiple of 8");
     }
     // the combine and the explicit-split kernels put the batch and the units of a row (kv heads; for the latent cache
     // query tokens x 128-head groups) in the grid's y / z extents
@@ -292,7 +295,7 @@ int fa_rocm_plan_kvcache(const fa_kvcache_args *a, int num_cus, fa_split_plan *p
     const int group = a->nheads / a->nheads_k;
     // the int8 latent kernel works on units of 128 query heads and always uses the balanced partition
     const size_t rows = is_mla_i8(a) ? 128 : (size_t)a->seqlen_q * group;
-    const size_t slot_bytes = rows * ((size_t)a->headdim_v + 1) * sizeof(float);
+    const size_t slot_bytes = rows * ((size_t)partial_width(a) + 1) * sizeof(float);
     if (!is_mla_i8(a) && rows > (size_t)decode_max_rows(a)) {
         // Query block too tall for the decode kernels: the tiled forward.  When its tiles alone
         // cannot fill the device (few sequences, short blocks) the keys of every unit are cut into
@@ -537,9 +540,10 @@ static int fwd_kvcache_impl(const fa_kvcache_args *a, void *stream_, void *const
             pp.nsplits = tplan.nsplits;
             pp.rows = rows;
             pp.o_partial = partials;
-            pp.lse_partial = partials + slot_rows * a->headdim_v;
+            pp.lse_partial = partials + slot_rows * partial_width(a);
         }
-        const hipError_t e = fa::launch_prefill(pp, a->io_dtype, a->headdim_qk, stream);
+        pp.headdim = a->headdim_qk;
+        const hipError_t e = fa::launch_prefill(pp, a->io_dtype, fa::tile_headdim(a->headdim_qk), stream);
         if (e != hipSuccess) return fail(FA_ERR_LAUNCH, "prefill launch failed: %s", hipGetErrorString(e));
         mark(2);
         if (tplan.nsplits > 1) {
@@ -569,7 +573,8 @@ static int fwd_kvcache_impl(const fa_kvcache_args *a, void *stream_, void *const
             cp.split_adaptive = 1;
             cp.o_partial = pp.o_partial;
             cp.lse_partial = pp.lse_partial;
-            const hipError_t ec = fa::launch_splitkv_combine(cp, a->io_dtype, a->headdim_v, stream);
+            cp.headdim = a->headdim_v;
+            const hipError_t ec = fa::launch_splitkv_combine(cp, a->io_dtype, partial_width(a), stream);
             if (ec != hipSuccess) return fail(FA_ERR_LAUNCH, "combine launch failed: %s", hipGetErrorString(ec));
         }
         mark(3);
@@ -605,6 +610,7 @@ static int fwd_kvcache_impl(const fa_kvcache_args *a, void *stream_, void *const
     p.nheads_k = a->nheads_k;
     p.group = group;
     p.rows = rows;
+    p.headdim = a->headdim_v;
     p.seqlen_new = a->seqlen_new;
     p.num_blocks = a->num_blocks;
     p.page_size = a->page_size;
@@ -654,9 +660,9 @@ static int fwd_kvcache_impl(const fa_kvcache_args *a, void *stream_, void *const
                         !env().no_head_interleave;
     const bool needs_combine = need > 0;
     if (needs_combine) {
-        const size_t slot_rows = need / (((size_t)a->headdim_v + 1) * sizeof(float));
+        const size_t slot_rows = need / (((size_t)partial_width(a) + 1) * sizeof(float));
         p.o_partial = static_cast<float *>(a->workspace);
-        p.lse_partial = p.o_partial + slot_rows * a->headdim_v;
+        p.lse_partial = p.o_partial + slot_rows * partial_width(a);
     }
 
     // The wave-level kernel appends on the fly when every new position is certain to be visible
@@ -689,12 +695,12 @@ static int fwd_kvcache_impl(const fa_kvcache_args *a, void *stream_, void *const
         e = fa::launch_decode_mla_i8(p, a->io_dtype, stream);
     }
     else {
-        e = fa::launch_decode_paged(p, a->io_dtype, a->headdim_qk, stream);
+        e = fa::launch_decode_paged(p, a->io_dtype, fa::tile_headdim(a->headdim_qk), stream);
     }
     if (e != hipSuccess) return fail(FA_ERR_LAUNCH, "decode launch failed: %s", hipGetErrorString(e));
     mark(2);
     if (needs_combine) {
-        e = fa::launch_splitkv_combine(p, a->io_dtype, a->headdim_v, stream);
+        e = fa::launch_splitkv_combine(p, a->io_dtype, partial_width(a), stream);
         if (e != hipSuccess) return fail(FA_ERR_LAUNCH, "combine launch failed: %s", hipGetErrorString(e));
     }
     mark(3);
@@ -772,7 +778,7 @@ int fa_rocm_varlen_validate(const fa_varlen_args *a) {
     if (a->nheads <= 0 || a->nheads_k <= 0 || a->nheads % a->nheads_k != 0)
         return fail(FA_ERR_SHAPE, "Number of heads in key/value must divide number of heads in query");
     if (a->headdim > 256) return fail(FA_ERR_SHAPE, "FlashAttention only supports head dimension at most 256");
-    if (a->headdim != 64 && a->headdim != 128 && a->headdim != 256) return fail(FA_ERR_SHAPE, "head dimension must be 64, 128 or 256");
+    if (a->headdim < 8 || a->headdim % 8 != 0) return fail(FA_ERR_SHAPE, "head dimension must be a positive multiple of 8");
     if (a->softcap < 0.f) return fail(FA_ERR_SHAPE, "softcap must be non-negative (0.0 disables softcap)");
     if (a->max_seqlen_q <= 0) return fail(FA_ERR_SHAPE, "max_seqlen_q must be positive");
     if (a->num_splits < 0) return fail(FA_ERR_SHAPE, "num_splits must be non-negative");
@@ -881,7 +887,7 @@ VarlenWorkspace varlen_workspace(const fa_varlen_args *a, int num_cus) {
     w.decode_only = w.short_blocks && a->max_seqlen_q <= w.slots;
     w.nsplits = w.decode_only ? 1 : fa_rocm_varlen_num_splits(a, num_cus);
     size_t off = 0;
-    if (w.nsplits > 1) off = align256((size_t)a->total_q * a->nheads * w.nsplits * ((size_t)a->headdim + 1) * sizeof(float));
+    if (w.nsplits > 1) off = align256((size_t)a->total_q * a->nheads * w.nsplits * ((size_t)fa::tile_headdim(a->headdim) + 1) * sizeof(float));
     if (w.short_blocks) {
         const size_t rows = (size_t)a->batch * w.slots * a->nheads;
         w.q_rows = off;
@@ -1032,6 +1038,7 @@ int fa_rocm_varlen_fwd(const fa_varlen_args *a, void *stream_) {
     pp.v_stride_h = a->v_stride_h;
     pp.v_stride_block = a->v_stride_block;
     pp.bt_stride_b = a->bt_stride_b;
+    pp.headdim = a->headdim;
     pp.lse_stride_b = 0;
     pp.lse_stride_h = a->total_q;
     pp.scale_log2 = a->softmax_scale * kLog2e;
@@ -1047,7 +1054,7 @@ int fa_rocm_varlen_fwd(const fa_varlen_args *a, void *stream_) {
     if (nsplits > 1) {
         pp.nsplits = nsplits;
         pp.o_partial = static_cast<float *>(a->workspace);
-        pp.lse_partial = pp.o_partial + (size_t)a->total_q * a->nheads * nsplits * a->headdim;
+        pp.lse_partial = pp.o_partial + (size_t)a->total_q * a->nheads * nsplits * fa::tile_headdim(a->headdim);
     }
     pp.skip_short = w.short_blocks ? w.slots : 0;
     if (w.short_blocks && !w.decode_only) {
@@ -1057,9 +1064,9 @@ int fa_rocm_varlen_fwd(const fa_varlen_args *a, void *stream_) {
         pp.list_wgs = cus * (a->headdim <= 128 ? 2 : 1);
     }
     if (!w.decode_only) {
-        const hipError_t e = fa::launch_prefill(pp, a->io_dtype, a->headdim, stream);
+        const hipError_t e = fa::launch_prefill(pp, a->io_dtype, fa::tile_headdim(a->headdim), stream);
         if (e != hipSuccess) return fail(FA_ERR_LAUNCH, "prefill launch failed: %s", hipGetErrorString(e));
-        const hipError_t ec = fa::launch_prefill_combine(pp, a->io_dtype, a->headdim, stream);
+        const hipError_t ec = fa::launch_prefill_combine(pp, a->io_dtype, fa::tile_headdim(a->headdim), stream);
         if (ec != hipSuccess) return fail(FA_ERR_LAUNCH, "combine launch failed: %s", hipGetErrorString(ec));
     }
     if (w.short_blocks) {

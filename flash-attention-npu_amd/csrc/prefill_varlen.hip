@@ -44,7 +44,9 @@ template <int D> struct PrefillCfg {
 // One 128-row block of one (sequence, key range, kv head, q head) of the launch: `bid` is its place in the
 // launch's order.  n_long < 0: the units are the launch's batch rows; otherwise they are the first n_long entries of
 // p.long_ids (the sequences the tiled kernel computes, listed on the device).
-template <typename T, int D, bool PAGED, bool SOFTCAP, bool EXT>
+// PART: the head dimension p.headdim is below D: pieces of the q / k / v rows behind it are zeros that nobody loads,
+// k-steps and output tiles that only see such pieces are skipped, and the stores stop at the head dimension.
+template <typename T, int D, bool PAGED, bool SOFTCAP, bool EXT, bool PART>
 __device__ __forceinline__ void prefill_block(const PrefillParams &p, const unsigned bid, const int n_long,
                                               uint8_t (&s_k)[2][PrefillCfg<D>::kTileBytes],
                                               uint8_t (&s_v)[2][PrefillCfg<D>::kVTileBytes]) {
@@ -54,6 +56,7 @@ __device__ __forceinline__ void prefill_block(const PrefillParams &p, const unsi
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lh = lane >> 5;   // half: MFMA k-slot
     const int ln = lane & 31;   // MFMA row / column
+    const int hd = PART ? p.headdim : D;
 
     // Workgroup i of the 1-D grid runs on XCD i % 8.  The grid is ordered by 128-row block, tallest
     // first, and inside a block by position e: XCD lane e % 8 walks the units (sequence, key range,
@@ -185,7 +188,7 @@ __device__ __forceinline__ void prefill_block(const PrefillParams &p, const unsi
     if (k_hi <= k_lo) {
         // nothing visible for the whole block: out = 0, lse = +inf
         if (row_ok && whole) {
-            for (int c = lh * (D / 2); c < (lh + 1) * (D / 2); c += 8) store16(o_row + c, u32x4_t{0, 0, 0, 0});
+            for (int c = lh * (D / 2); c < min((lh + 1) * (D / 2), hd); c += 8) store16(o_row + c, u32x4_t{0, 0, 0, 0});
             if (lh == 0) *lse_row = INFINITY;
         } else if (row_ok) {
             for (int c = lh * (D / 2); c < (lh + 1) * (D / 2); c += 4) *reinterpret_cast<float4 *>(part_row + c) = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -212,6 +215,10 @@ __device__ __forceinline__ void prefill_block(const PrefillParams &p, const unsi
         const uint16_t *src = q_row + lh * 8;
 #pragma unroll
         for (int t = 0; t < Cfg::kKSteps; ++t) {
+            if (PART && t * 16 + lh * 8 >= hd) {
+                qreg[t] = u32x4_t{0, 0, 0, 0};
+                continue;
+            }
             qreg[t] = load16(src + t * 16);
             if (!row_ok) qreg[t] = u32x4_t{0, 0, 0, 0};
         }
@@ -223,18 +230,24 @@ __device__ __forceinline__ void prefill_block(const PrefillParams &p, const unsi
     const int32_t *bt_row = PAGED ? p.block_table + (int64_t)b * p.bt_stride_b : nullptr;
 
     u32x4_t kst[Cfg::kPieces], vst[Cfg::kPieces];
+    if constexpr (PART) {
+#pragma unroll
+        for (int i = 0; i < Cfg::kPieces; ++i) kst[i] = vst[i] = u32x4_t{0, 0, 0, 0};
+    }
     // A thread's pieces of one tile sit 256/kChunks rows apart and tiles kBN rows apart, so one small
     // per-thread byte offset plus wave-uniform (scalar) terms addresses every load of an interior
     // tile of dense K/V, and one per-thread LDS offset plus constants every store.
     constexpr int kRowsPerPass = 256 / Cfg::kChunks;
     const int t_row = tid / Cfg::kChunks;
     const int t_ch = tid % Cfg::kChunks;
+    const bool piece_live = !PART || t_ch * 8 < hd;
     const uint32_t k_thread_off = (uint32_t)t_row * (uint32_t)p.k_stride_t * 2u + t_ch * 16;
     const uint32_t v_thread_off = (uint32_t)t_row * (uint32_t)p.v_stride_t * 2u + t_ch * 16;
     const uint32_t k_lds_off = t_row * (D * 2) + ((t_ch ^ (t_row & Cfg::kSwz)) << 4);   // row + 16*i keeps row & 15
     const uint32_t v_lds_off = t_row * Cfg::kVRowBytes + (t_ch << 4);
     static_assert(kRowsPerPass % (Cfg::kSwz + 1) == 0 && Cfg::kSwz < Cfg::kChunks, "swizzle must survive the row step");
     auto fetch_tile = [&](int kt) {
+        if (!piece_live) return;
         if constexpr (!PAGED) {
             if (kt * kBN + kBN <= Sk) {
                 const uint8_t *kb = reinterpret_cast<const uint8_t *>(kbase) + (int64_t)(k0 + kt * kBN) * p.k_stride_t * 2;
@@ -319,6 +332,7 @@ __device__ __forceinline__ void prefill_block(const PrefillParams &p, const unsi
         for (int t = 0; t < kPf; ++t) read_k(t);
 #pragma unroll
         for (int t = 0; t < Cfg::kKSteps; ++t) {
+            if (PART && t * 16 >= hd) break;   // wave-uniform; at least D/2 columns are live
             if (t + kPf < Cfg::kKSteps) read_k(t + kPf);
             s[0] = mfma32<T>(ka[t][0], qreg[t], s[0]);
             s[1] = mfma32<T>(ka[t][1], qreg[t], s[1]);
@@ -444,6 +458,7 @@ __device__ __forceinline__ void prefill_block(const PrefillParams &p, const unsi
                 for (int t = 0; t < Cfg::kMT; ++t)
 #pragma unroll
                     for (int hv = 0; hv < 2; ++hv) {
+                        if (PART && t * 32 >= hd) continue;
                         const int row = tt * 32 + 16 * ks + 8 * hv + tr_row;
                         const v4s_t r4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
                             (__attribute__((address_space(3))) v4s_t *)(&s_v[cur][row * Cfg::kVRowBytes + (t * 32 + tr_col) * 2]));
@@ -452,7 +467,10 @@ __device__ __forceinline__ void prefill_block(const PrefillParams &p, const unsi
                         va[t][2 * hv + 1] = r2.y;
                     }
 #pragma unroll
-                for (int t = 0; t < Cfg::kMT; ++t) o_acc[t] = mfma32<T>(va[t], pk[tt][ks], o_acc[t]);
+                for (int t = 0; t < Cfg::kMT; ++t) {
+                    if (PART && t * 32 >= hd) continue;
+                    o_acc[t] = mfma32<T>(va[t], pk[tt][ks], o_acc[t]);
+                }
             }
         }   // wave_live
 
@@ -506,7 +524,7 @@ __device__ __forceinline__ void prefill_block(const PrefillParams &p, const unsi
     for (int r0 = 0; r0 < 32; r0 += kStageRows) {
         const int rr = r0 + lane / kLanesPerRow;               // row of the wave's tile
         const int R = R0 + wave * 32 + rr;
-        if (R < n_rows) {
+        if (R < n_rows && (!PART || piece * 8 < hd)) {
             const int row = R / pg;
             const int head = h_base + (R - row * pg);
             uint16_t *dst = reinterpret_cast<uint16_t *>(p.out) + (int64_t)b * p.o_stride_b + (int64_t)head * p.o_stride_h +
@@ -516,12 +534,12 @@ __device__ __forceinline__ void prefill_block(const PrefillParams &p, const unsi
     }
 }
 
-template <typename T, int D, bool PAGED, bool SOFTCAP, bool EXT>
+template <typename T, int D, bool PAGED, bool SOFTCAP, bool EXT, bool PART>
 __global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) prefill_kernel(const PrefillParams p) {
     using Cfg = PrefillCfg<D>;
     __shared__ __attribute__((aligned(16))) uint8_t s_k[2][Cfg::kTileBytes];
     __shared__ __attribute__((aligned(16))) uint8_t s_v[2][Cfg::kVTileBytes];
-    prefill_block<T, D, PAGED, SOFTCAP, EXT>(p, blockIdx.x, -1, s_k, s_v);
+    prefill_block<T, D, PAGED, SOFTCAP, EXT, PART>(p, blockIdx.x, -1, s_k, s_v);
 }
 
 // The same blocks for a launch whose live sequences are known on the device only (token-major batches whose
@@ -531,7 +549,7 @@ __global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) prefill_kernel(const 
 // the ordered list until it ends: workgroup w (on XCD w % 8) takes the blocks congruent to w % 8, so that the heads
 // of a unit still meet in one L2, through one counter per XCD (p.list_state[1 + x], zeroed by the kernel that
 // wrote the list).  Every workgroup leaves when its counter passes the end of the list.
-template <typename T, int D, bool SOFTCAP>
+template <typename T, int D, bool SOFTCAP, bool PART>
 __global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) prefill_list_kernel(const PrefillParams p) {
     using Cfg = PrefillCfg<D>;
     __shared__ __attribute__((aligned(16))) uint8_t s_k[2][Cfg::kTileBytes];
@@ -548,7 +566,7 @@ __global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) prefill_list_kernel(c
         __syncthreads();
         const int64_t bid = (int64_t)s_item * 8 + x;
         if (bid >= total) break;
-        prefill_block<T, D, true, SOFTCAP, true>(p, (unsigned)bid, n_long, s_k, s_v);
+        prefill_block<T, D, true, SOFTCAP, true, PART>(p, (unsigned)bid, n_long, s_k, s_v);
     }
 }
 
@@ -605,8 +623,10 @@ __global__ void __launch_bounds__(256) prefill_combine_kernel(const PrefillParam
     }
     const float inv = (tot > 0.f) ? 1.f / tot : 0.f;
     uint16_t *dst = reinterpret_cast<uint16_t *>(p.out) + (int64_t)tok * p.o_stride_t + (int64_t)head * p.o_stride_h + lane * C;
+    if (lane * C < p.headdim) {   // the partials are D wide; the output row ends at the head dimension
 #pragma unroll
-    for (int c = 0; c < C; ++c) dst[c] = from_float<T>(acc[c] * inv);
+        for (int c = 0; c < C; ++c) dst[c] = from_float<T>(acc[c] * inv);
+    }
     if (lane == 0) p.lse[(int64_t)head * p.lse_stride_h + tok] = (tot > 0.f) ? (mx + fast_log2(tot)) * kLn2 : INFINITY;
 }
 
@@ -626,20 +646,38 @@ template <typename T, int D> static hipError_t launch_prefill_d(const PrefillPar
     const bool softcap = p.softcap_post != 0.f;
     const bool paged = p.block_table != nullptr;
     p.pack_short = p.cu_seqlens_q ? prefill_pack_short(p.group, p.max_seqlen_q, p.total_q, p.batch) : 0;
-    const bool ext = p.pack > 1 || p.nsplits > 1 || p.pack_short || p.skip_short > 0;
+    if (p.headdim > D || p.headdim < 8 || p.headdim % 8 != 0) return hipErrorInvalidValue;
+    const bool part = p.headdim < D;
+    // a head dimension below the compiled width always takes the kernels with every extension compiled in
+    const bool ext = part || p.pack > 1 || p.nsplits > 1 || p.pack_short || p.skip_short > 0;
     if (p.long_ids) {
         // live sequences listed on the device: workgroups that stay and take blocks from the list
         if (!paged || !p.list_state || p.list_wgs <= 0 || !p.cu_seqlens_q) return hipErrorInvalidValue;
         dim3 lgrid((unsigned)std::min<int64_t>(p.list_wgs, wgs));
-        if (softcap)
-            hipLaunchKernelGGL((prefill_list_kernel<T, D, true>), lgrid, block, 0, stream, p);
-        else
-            hipLaunchKernelGGL((prefill_list_kernel<T, D, false>), lgrid, block, 0, stream, p);
+        if (softcap) {
+            if (part)
+                hipLaunchKernelGGL((prefill_list_kernel<T, D, true, true>), lgrid, block, 0, stream, p);
+            else
+                hipLaunchKernelGGL((prefill_list_kernel<T, D, true, false>), lgrid, block, 0, stream, p);
+        } else {
+            if (part)
+                hipLaunchKernelGGL((prefill_list_kernel<T, D, false, true>), lgrid, block, 0, stream, p);
+            else
+                hipLaunchKernelGGL((prefill_list_kernel<T, D, false, false>), lgrid, block, 0, stream, p);
+        }
         return hipGetLastError();
     }
     auto launch = [&](auto paged_c, auto softcap_c, auto ext_c) {
-        hipLaunchKernelGGL((prefill_kernel<T, D, decltype(paged_c)::value, decltype(softcap_c)::value, decltype(ext_c)::value>),
-                           grid, block, 0, stream, p);
+        constexpr bool kExt = decltype(ext_c)::value;
+        if constexpr (kExt) {
+            if (part) {
+                hipLaunchKernelGGL((prefill_kernel<T, D, decltype(paged_c)::value, decltype(softcap_c)::value, true, true>), grid, block,
+                                   0, stream, p);
+                return;
+            }
+        }
+        hipLaunchKernelGGL((prefill_kernel<T, D, decltype(paged_c)::value, decltype(softcap_c)::value, kExt, false>), grid, block, 0,
+                           stream, p);
     };
     auto pick_ext = [&](auto paged_c, auto softcap_c) {
         if (ext) launch(paged_c, softcap_c, std::true_type{}); else launch(paged_c, softcap_c, std::false_type{});

@@ -59,7 +59,7 @@ def fwd_kvcache(q, kcache, vcache, k_, v_, seqlens_k_, rotary_cos_, rotary_sin_,
                 ) -> List[torch.Tensor]:
     """mha_fwd_kvcache (flash_api.cpp:356-637) on a paged cache.  Returns [out, softmax_lse]."""
     if (isinstance(q, torch.Tensor) and q.dim() == 4 and kcache.dtype != torch.int8
-            and q.shape[-1] not in (64, 128, 256) and q.shape[-1] <= 256 and q.shape[-1] == kcache.shape[-1]
+            and q.shape[-1] % 8 != 0 and q.shape[-1] <= 256 and q.shape[-1] == kcache.shape[-1]
             and q.dtype in (torch.bfloat16, torch.float16) and q.is_cuda and kcache.is_cuda):
         return _fwd_kvcache_padded(q, kcache, vcache, k_, v_, seqlens_k_, rotary_cos_, rotary_sin_, cache_batch_idx_,
                                    leftpad_k_, block_table_, alibi_slopes_, out_, softmax_scale, is_causal,
@@ -74,13 +74,14 @@ def fwd_kvcache(q, kcache, vcache, k_, v_, seqlens_k_, rotary_cos_, rotary_sin_,
 def _fwd_kvcache_padded(q, kcache, vcache, k_, v_, seqlens_k_, rotary_cos_, rotary_sin_, cache_batch_idx_, leftpad_k_,
                         block_table_, alibi_slopes_, out_, softmax_scale, is_causal, window_size_left,
                         window_size_right, softcap, is_rotary_interleaved, num_splits) -> List[torch.Tensor]:
-    """Head dimensions the kernels are not built for (the reference's tests go down to 1 and 4,
-    tests/test_flash_attn_npu_v2.py:178-183): zero-padded COPIES of q and of the caches go through the
-    kernels (zero columns change neither the scores nor the kept output columns), then the rows the
-    call appended are copied back into the caller's caches.  A slow path: it copies the whole cache."""
+    """Head dimensions that are not a multiple of 8 (the reference's tests go down to 1 and 4,
+    tests/test_flash_attn_npu_v2.py:178-183; every multiple of 8 up to 256 runs on the caller's cache as it is): the
+    rows are not 16-byte pieces, so zero-padded COPIES of q and of the caches, to the next multiple of 8, go through
+    the kernels (zero columns change neither the scores nor the kept output columns), then the rows the call
+    appended are copied back into the caller's caches.  A slow path: it copies the whole cache."""
     import torch.nn.functional as F
     d, dv = q.shape[-1], vcache.shape[-1]
-    dp = 64 if max(d, dv) <= 64 else (128 if max(d, dv) <= 128 else 256)
+    dp = (max(d, dv) + 7) // 8 * 8
     _require(kcache.dim() == 4 and vcache.dim() == 4, "q, kcache and vcache must be 4-D")
     _require(dv == d, "k and v head dimensions must match")
 
@@ -282,6 +283,25 @@ def varlen_fwd(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k_, leftpad_k_
     num_splits (paged K/V only; not an argument of the reference's function): 0 cuts every sequence's keys into
     as many ranges as it takes to fill the device when the query tiles alone cannot, 1 never, n at most n."""
     lib = _lib.load()
+    if (isinstance(q, torch.Tensor) and q.dim() == 3 and q.shape[-1] % 8 != 0 and q.shape[-1] <= 256 and q.is_cuda
+            and k.shape[-1] == q.shape[-1] and v.shape[-1] == q.shape[-1]):
+        # rows that are not 16-byte pieces: zero-padded copies to the next multiple of 8, as the reference's front end
+        # does (flash_attn_npu_interface.py:897-901); with paged k / v this copies the cache
+        import torch.nn.functional as F
+        d = q.shape[-1]
+        extra = (d + 7) // 8 * 8 - d
+        res = varlen_fwd(F.pad(q, (0, extra)), F.pad(k, (0, extra)), F.pad(v, (0, extra)), None, cu_seqlens_q, cu_seqlens_k,
+                         seqused_k_, leftpad_k_, block_table_, alibi_slopes_, max_seqlen_q, max_seqlen_k, p_dropout,
+                         softmax_scale, zero_tensors, is_causal, window_size_left, window_size_right, softcap, return_softmax,
+                         gen_, num_splits=num_splits)
+        out = res[0][..., :d]
+        if out_ is not None:
+            _require(out_.dtype == q.dtype and out_.shape == q.shape, "out must match q")
+            out_.copy_(out)
+            out = out_
+        else:
+            out = out.contiguous()
+        return [out] + list(res[1:])
     _require(q.dtype in (torch.bfloat16, torch.float16), "FlashAttention only supports FP16 and BF16 data types")
     _require(k.dtype == q.dtype, "query and key must have the same dtype")
     _require(v.dtype == q.dtype, "query and value must have the same dtype")

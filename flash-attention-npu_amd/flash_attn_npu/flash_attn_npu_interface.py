@@ -175,11 +175,12 @@ class FlashAttnVarlenFunc(torch.autograd.Function):
         if softmax_scale is None:
             softmax_scale = q.shape[-1] ** (-0.5)
         head_size_og = q.size(2)
-        # The reference pads the head dimension to a multiple of 8 (flash_attn_npu_interface.py:897-901);
-        # the gfx950 kernels are built for 64, 128 and 256, so pad with zeros to the next of those
-        # (zero columns change neither QK^T nor the kept columns of PV).
-        head_size_pad = next((x for x in (64, 128, 256) if x >= head_size_og), head_size_og)
-        if head_size_pad != head_size_og and block_table is None:
+        # As the reference does (flash_attn_npu_interface.py:897-901): a head dimension that is not a multiple of 8 is
+        # padded with zeros to the next one (zero columns change neither QK^T nor the kept columns of PV); every
+        # multiple of 8 up to 256 runs as it is.  Paged k / v are padded the same way, which copies the cache: rows
+        # of such a width are not 16-byte pieces.
+        head_size_pad = (head_size_og + 7) // 8 * 8
+        if head_size_pad != head_size_og:
             q = torch.nn.functional.pad(q, [0, head_size_pad - head_size_og])
             k = torch.nn.functional.pad(k, [0, head_size_pad - head_size_og])
             v = torch.nn.functional.pad(v, [0, head_size_pad - head_size_og])

@@ -73,7 +73,7 @@ typedef struct fa_kvcache_args {
 
     /* dimensions */
     int32_t batch, seqlen_q, nheads, nheads_k;
-    int32_t headdim_qk, headdim_v;
+    int32_t headdim_qk, headdim_v;   /* equal, a multiple of 8, at most 256 (int8 latent cache: 576 / 512) */
     int32_t seqlen_new;          /* 0 when k_new == NULL */
     int32_t num_blocks, page_size, max_blocks_per_seq;
     int32_t rotary_dim, seqlen_ro;
