@@ -1,7 +1,8 @@
-"""Build libfa_rocm.so (C ABI + gfx950 kernels) in-tree with hipcc.
+"""Build libfa_rocm.so (C ABI + gfx950 kernels) in-tree with hipcc, then the PyTorch extension module over it.
 
     python flash-attention-npu_amd/build.py            # compile every translation unit, link
-The objects and the library land next to the sources (csrc/build/, csrc/libfa_rocm.so)."""
+The objects and the library land next to the sources (csrc/build/, csrc/libfa_rocm.so); the extension module
+(csrc/torch_binding.cpp, host C++ only, linked against the library) lands in the package as flash_attn_npu/_C*.so."""
 from __future__ import annotations
 
 import os
@@ -66,15 +67,16 @@ def _compile(src: str) -> str:
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"hipcc failed for {src}:\n{r.stdout}\n{r.stderr}")
-    if src in ACC_PINNED:
-        _check_acc_registers(src)
     return obj
 
 
 def build_all(jobs: int = 8, verbose: bool = True) -> str:
     os.makedirs(OUT_DIR, exist_ok=True)
-    with ThreadPoolExecutor(max_workers=min(jobs, len(SOURCES))) as ex:
+    with ThreadPoolExecutor(max_workers=min(jobs, len(SOURCES) + len(ACC_PINNED))) as ex:
+        checks = [ex.submit(_check_acc_registers, src) for src in SOURCES if src in ACC_PINNED]   # the long pole: start first
         objs = list(ex.map(_compile, SOURCES))
+        for c in checks:
+            c.result()
     cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
@@ -84,6 +86,27 @@ def build_all(jobs: int = 8, verbose: bool = True) -> str:
     return LIB
 
 
+def build_binding(verbose: bool = True) -> str:
+    """flash_attn_npu/_C: pybind11 + libtorch operator layer (torch_binding.cpp), host code only, g++."""
+    import sysconfig
+    from torch.utils import cpp_extension as ce
+    out = os.path.join(HERE, "flash_attn_npu", "_C" + sysconfig.get_config_var("EXT_SUFFIX"))
+    torch_lib = ce.library_paths()[0]
+    cmd = ([os.environ.get("CXX", "g++"), "-O2", "-fPIC", "-shared", "-std=c++17", "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+            "-DTORCH_EXTENSION_NAME=_C", "-DTORCH_API_INCLUDE_EXTENSION_H", "-D_GLIBCXX_USE_CXX11_ABI=1", "-Wno-deprecated-declarations"]
+           + [f"-I{p}" for p in ce.include_paths()] + [f"-I{sysconfig.get_paths()['include']}", "-I/opt/rocm/include",
+              os.path.join(CSRC, "torch_binding.cpp"), "-o", out,
+              f"-L{torch_lib}", "-lc10", "-lc10_hip", "-ltorch_cpu", "-ltorch_hip", "-ltorch", "-ltorch_python",
+              f"-L{CSRC}", "-lfa_rocm", "-Wl,-rpath,$ORIGIN/../csrc", f"-Wl,-rpath,{torch_lib}", "-L/opt/rocm/lib", "-lamdhip64"])
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"building the extension module failed:\n{r.stdout}\n{r.stderr}")
+    if verbose:
+        print(f"built {out}")
+    return out
+
+
 if __name__ == "__main__":
     build_all()
+    build_binding()
     sys.exit(0)

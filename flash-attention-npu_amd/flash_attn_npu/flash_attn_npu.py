@@ -1,9 +1,12 @@
 """Operator layer: `fwd_kvcache` and `varlen_fwd` with the argument order of the reference's
 extension module (csrc/ascend910/flash_attn_npu/flash_api.cpp:356-377, :848-869, exported at
-:1335-1336), implemented over the C ABI of libfa_rocm.so.
+:1335-1336).  Both are the compiled extension module `flash_attn_npu._C` (csrc/torch_binding.cpp: checks, argument
+record, allocation and the call into the C ABI of libfa_rocm.so, all in C++); what stays in Python here is the
+padded-copy path for head dimensions that are not multiples of 8, and `bind_kvcache` / `KvcacheCall`, a ctypes
+binding of one call that can be run many times (benchmarks, graph capture).
 
 Checks that the reference performs with TORCH_CHECK raise RuntimeError with the same text.
-There is no fallback: tensors must live on a ROCm device and the library must be built."""
+There is no fallback: tensors must live on a ROCm device and both the library and the module must be built."""
 from __future__ import annotations
 
 import ctypes as C
@@ -14,6 +17,23 @@ import torch
 from . import _lib
 
 _DT = {torch.bfloat16: _lib.FA_BF16, torch.float16: _lib.FA_FP16, torch.int8: _lib.FA_INT8}
+
+
+_ext = None
+
+
+def _C():
+    """The compiled extension module; a missing build is an error, never a slower path."""
+    global _ext
+    if _ext is None:
+        _lib.load()
+        try:
+            from . import _C as ext
+        except ImportError as e:
+            raise RuntimeError("flash_attn_npu._C (the compiled operator layer) is not built: run "
+                               "`python flash-attention-npu_amd/build.py`; there is no CPU or PyTorch fallback") from e
+        _ext = ext
+    return _ext
 
 
 def _ptr(t: Optional[torch.Tensor]):
@@ -64,11 +84,9 @@ def fwd_kvcache(q, kcache, vcache, k_, v_, seqlens_k_, rotary_cos_, rotary_sin_,
         return _fwd_kvcache_padded(q, kcache, vcache, k_, v_, seqlens_k_, rotary_cos_, rotary_sin_, cache_batch_idx_,
                                    leftpad_k_, block_table_, alibi_slopes_, out_, softmax_scale, is_causal,
                                    window_size_left, window_size_right, softcap, is_rotary_interleaved, num_splits)
-    call = bind_kvcache(q, kcache, vcache, k_, v_, seqlens_k_, rotary_cos_, rotary_sin_, cache_batch_idx_, leftpad_k_,
-                        block_table_, alibi_slopes_, out_, softmax_scale, is_causal, window_size_left,
-                        window_size_right, softcap, is_rotary_interleaved, num_splits, k_scale_cache_, v_scale_cache_)
-    call.run()
-    return [call.out, call.lse]
+    return _C().fwd_kvcache(q, kcache, vcache, k_, v_, seqlens_k_, rotary_cos_, rotary_sin_, cache_batch_idx_, leftpad_k_,
+                            block_table_, alibi_slopes_, out_, softmax_scale, is_causal, window_size_left, window_size_right,
+                            softcap, is_rotary_interleaved, num_splits, k_scale_cache_, v_scale_cache_)
 
 
 def _fwd_kvcache_padded(q, kcache, vcache, k_, v_, seqlens_k_, rotary_cos_, rotary_sin_, cache_batch_idx_, leftpad_k_,
@@ -282,7 +300,6 @@ def varlen_fwd(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k_, leftpad_k_
     """mha_varlen_fwd (flash_api.cpp:848-1089).  Returns [out, softmax_lse (Hq, total_q), p, rng_state].
     num_splits (paged K/V only; not an argument of the reference's function): 0 cuts every sequence's keys into
     as many ranges as it takes to fill the device when the query tiles alone cannot, 1 never, n at most n."""
-    lib = _lib.load()
     if (isinstance(q, torch.Tensor) and q.dim() == 3 and q.shape[-1] % 8 != 0 and q.shape[-1] <= 256 and q.is_cuda
             and k.shape[-1] == q.shape[-1] and v.shape[-1] == q.shape[-1]):
         # rows that are not 16-byte pieces: zero-padded copies to the next multiple of 8, as the reference's front end
@@ -302,77 +319,7 @@ def varlen_fwd(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k_, leftpad_k_
         else:
             out = out.contiguous()
         return [out] + list(res[1:])
-    _require(q.dtype in (torch.bfloat16, torch.float16), "FlashAttention only supports FP16 and BF16 data types")
-    _require(k.dtype == q.dtype, "query and key must have the same dtype")
-    _require(v.dtype == q.dtype, "query and value must have the same dtype")
-    _require(cu_seqlens_q.dtype == torch.int32, "cu_seqlens_q must have dtype int32")
-    _require(q.stride(-1) == 1 and k.stride(-1) == 1 and v.stride(-1) == 1, "Input tensor must have contiguous last dimension")
-    _require(leftpad_k_ is None, "NPU FlashAttention does not support leftpad_k")
-    _require(alibi_slopes_ is None, "NPU FlashAttention does not support alibi_slopes")
-    _require(p_dropout == 0.0, "NPU FlashAttention does not support dropout")
-    _require(not return_softmax, "NPU FlashAttention does not support return_softmax")
-    _require(softcap >= 0.0, "softcap must be non-negative (0.0 disables softcap)")
-    # flash_api.cpp:890 (the outputs are written in full either way, nothing is left to clear)
-    _require(not zero_tensors, "NPU FlashAttention does not support zero_tensors.")
-    paged = block_table_ is not None
-    # flash_api.cpp:886 rejects seqused_k always; here it is the length array of paged K/V and has no meaning for
-    # packed keys, whose lengths are the differences of cu_seqlens_k
-    _require(paged or seqused_k_ is None, "NPU FlashAttention does not support seqused_k.")
-    _require_device(q, k, v, cu_seqlens_q, cu_seqlens_k, seqused_k_, block_table_)
-    total_q, hq, d = q.shape
-    B = cu_seqlens_q.numel() - 1
-    _require(B > 0, "batch size must be positive")
-    a = _lib.VarlenArgs()
-    if paged:
-        _require(block_table_.dtype == torch.int32, "block_table must have dtype int32")
-        _require(block_table_.stride(-1) == 1, "block_table must have contiguous last dimension")
-        _require(k.dim() == 4 and v.dim() == 4, "paged k / v must be (num_blocks, page_block_size, nheads_k, headdim)")
-        if seqused_k_ is None:
-            _require(cu_seqlens_k is not None, "paged K/V needs seqused_k or cu_seqlens_k")
-            seqused_k_ = (cu_seqlens_k[1:] - cu_seqlens_k[:-1]).to(torch.int32)
-        _require(seqused_k_.dtype == torch.int32, "seqused_k must have dtype int32")
-        seqused_k_ = seqused_k_.contiguous()
-        hk = k.shape[2]
-        a.page_size, a.max_blocks_per_seq, a.num_blocks = k.shape[1], block_table_.shape[1], k.shape[0]
-        a.k_stride_block, a.k_stride_t, a.k_stride_h = k.stride(0), k.stride(1), k.stride(2)
-        a.v_stride_block, a.v_stride_t, a.v_stride_h = v.stride(0), v.stride(1), v.stride(2)
-        a.block_table, a.seqused_k, a.bt_stride_b = _ptr(block_table_), _ptr(seqused_k_), block_table_.stride(0)
-    else:
-        _require(cu_seqlens_k is not None and cu_seqlens_k.dtype == torch.int32, "cu_seqlens_k must have dtype int32")
-        _require(k.dim() == 3 and v.dim() == 3, "k / v must be (total_k, nheads_k, headdim)")
-        hk = k.shape[1]
-        a.k_stride_t, a.k_stride_h = k.stride(0), k.stride(1)
-        a.v_stride_t, a.v_stride_h = v.stride(0), v.stride(1)
-    _require(k.shape[-1] == d and v.shape[-1] == d, "q, k and v must have the same head dimension")
-    _require(d <= 256, "FlashAttention only supports head dimension at most 256")
-    _require(hq % hk == 0, "Number of heads in key/value must divide number of heads in query")
-    cu_q = cu_seqlens_q.contiguous()
-    cu_k = cu_seqlens_k.contiguous() if cu_seqlens_k is not None else None
-    if out_ is not None:
-        out = out_
-        _require(out.dtype == q.dtype and out.shape == q.shape and out.stride(-1) == 1, "out must match q")
-    else:
-        out = torch.empty_like(q, memory_format=torch.contiguous_format)
-    lse = torch.empty((hq, total_q), dtype=torch.float32, device=q.device)
-    a.q, a.k, a.v, a.out, a.softmax_lse = _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse)
-    a.cu_seqlens_q, a.cu_seqlens_k = _ptr(cu_q), _ptr(cu_k)
-    a.batch, a.total_q, a.nheads, a.nheads_k, a.headdim = B, total_q, hq, hk, d
-    a.max_seqlen_q, a.max_seqlen_k = int(max_seqlen_q), int(max_seqlen_k)
-    a.q_stride_t, a.q_stride_h = q.stride(0), q.stride(1)
-    a.o_stride_t, a.o_stride_h = out.stride(0), out.stride(1)
-    a.io_dtype = _DT[q.dtype]
-    a.softmax_scale, a.softcap = float(softmax_scale), float(softcap)
-    a.causal = int(bool(is_causal))
-    a.window_left, a.window_right = int(window_size_left), int(window_size_right)
-    _require(num_splits >= 0, "num_splits must be non-negative")
-    a.num_splits = int(num_splits)
-    if total_q > 0:
-        with torch.cuda.device(q.device):
-            need = lib.fa_rocm_varlen_workspace_bytes(C.byref(a), lib.fa_rocm_num_cus())
-            if need:
-                ws = torch.empty(((need + 3) // 4,), dtype=torch.float32, device=q.device)
-                a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel() * 4
-            _lib.check(lib.fa_rocm_varlen_fwd(C.byref(a), _stream(q)))
-    p = torch.empty((0,), dtype=q.dtype, device=q.device)
-    rng_state = torch.empty((2,), dtype=torch.int64, device=q.device)
-    return [out, lse, p, rng_state]
+    return _C().varlen_fwd(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k_, leftpad_k_, block_table_, alibi_slopes_,
+                           int(max_seqlen_q), int(max_seqlen_k), float(p_dropout), float(softmax_scale), bool(zero_tensors),
+                           bool(is_causal), int(window_size_left), int(window_size_right), float(softcap), bool(return_softmax),
+                           int(num_splits))

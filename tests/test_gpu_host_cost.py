@@ -1,0 +1,64 @@
+"""Host cost of the public flash_attn_with_kvcache call.
+
+The call is asynchronous: the host checks the arguments, allocates the outputs and the split workspace, fills the C
+argument record and enqueues the kernels.  Timed here is the host side alone (no synchronisation inside the timed
+loop, a problem so small that the device keeps up), next to the bare C-ABI call on a record bound once, which is the
+part no binding can remove (the kernel launches themselves).  The difference is what the operator layer costs."""
+import ctypes as C
+import time
+
+import pytest
+import torch
+
+from helpers import make_paged_case, to_dev
+
+pytestmark = pytest.mark.gpu
+
+BINDING_BUDGET_US = 8.0
+
+
+def per_call_us(fn, n=300, repeats=7):
+    best = float("inf")
+    for _ in range(repeats):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n):
+            fn()
+        t1 = time.perf_counter()
+        torch.cuda.synchronize()
+        best = min(best, (t1 - t0) / n * 1e6)
+    return best
+
+
+@pytest.mark.parametrize("snew", [0, 1])
+def test_operator_layer_costs_at_most_8_us(snew):
+    from flash_attn_npu import _lib, flash_attn_with_kvcache
+    from flash_attn_npu.flash_attn_npu import _C, bind_kvcache
+    case = make_paged_case(1, 8, 2, 128, 256, [40], seqlen_new=snew, seed=0)
+    dev = to_dev(case)
+    q, kc, vc, kn, vn, lens, bt = (dev[n] for n in ("q", "k_cache", "v_cache", "k", "v", "cache_seqlens", "block_table"))
+
+    def public():
+        return flash_attn_with_kvcache(q, kc, vc, kn, vn, cache_seqlens=lens, block_table=bt, causal=True)
+
+    ext = _C()
+
+    def module():
+        return ext.fwd_kvcache(q, kc, vc, kn, vn, lens, None, None, None, None, bt, None, None, 128 ** -0.5, True, -1, -1, 0.0, True, 0,
+                               None, None)
+
+    call = bind_kvcache(q, kc, vc, kn, vn, lens, None, None, None, None, bt, None, None, 128 ** -0.5, True, -1, -1, 0.0, True, 0)
+    lib = _lib.load()
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    args = C.byref(call.args)
+
+    def raw():
+        return lib.fa_rocm_fwd_kvcache(args, stream)
+
+    for f in (public, module, raw):
+        for _ in range(50):
+            f()
+    t_raw, t_mod, t_pub = per_call_us(raw), per_call_us(module), per_call_us(public)
+    print(f"host us/call (snew={snew}): C ABI on a bound record {t_raw:.2f}, extension module {t_mod:.2f}, public function {t_pub:.2f}; "
+          f"operator layer = {t_pub - t_raw:.2f}", flush=True)
+    assert t_pub - t_raw <= BINDING_BUDGET_US, f"the operator layer costs {t_pub - t_raw:.2f} us per call on the host"
