@@ -127,13 +127,13 @@ __device__ __forceinline__ void process_piece(const DecodeParams &p, const int b
     const uint32_t v_lane_off = (uint32_t)(lq * 4) * v_row_bytes + v_lane_col;
 
     // page id of chunk c (clamped into the pool so a corrupt table cannot fault)
-    auto fetch_blk = [&](int c) -> int {
+    auto load_blk = [&](int c) -> int {   // the table entry as loaded (every lane the same address); not waited for
         if (c >= c_end) return 0;
         int page = (c * kChunk) / p.page_size;
         page = min(page, p.max_blocks - 1);
-        const int blk = __builtin_amdgcn_readfirstlane(bt_row[page]);
-        return min(max(blk, 0), p.num_blocks - 1);
+        return bt_row[page];
     };
+    auto use_blk = [&](int raw) -> int { return min(max(__builtin_amdgcn_readfirstlane(raw), 0), p.num_blocks - 1); };
 
     auto load_v = [&](const uint8_t *s2, int e, int hh) {
         if constexpr (Cfg::kVW == 8) {
@@ -193,9 +193,15 @@ __device__ __forceinline__ void process_piece(const DecodeParams &p, const int b
     };
 
     int c = c_begin + wave;
-    int blk_next = fetch_blk(c);
-    if (c < c_end) issue_loads(c, blk_next);
-    blk_next = fetch_blk(c + NW);
+    int blk_next;
+    {
+        // Both table entries are asked for before the first chunk's loads.  Loads return in order: asked for behind
+        // them, the second entry would only be there when the whole chunk is, and the q rows would be requested a
+        // memory latency later than they need be.
+        const int blk0 = load_blk(c);
+        blk_next = load_blk(c + NW);
+        if (c < c_end) issue_loads(c, use_blk(blk0));
+    }
 
     // (the first chunk is already in flight while Q is staged)
     // ---- stage Q (with rotary) into LDS as 16-bit rows -------------------------------------
@@ -273,8 +279,10 @@ __device__ __forceinline__ void process_piece(const DecodeParams &p, const int b
         __builtin_amdgcn_wave_barrier();
 
         const int cn = c + NW;
-        if (cn < c_end) issue_loads(cn, blk_next);
-        blk_next = fetch_blk(cn + NW);
+        if (cn < c_end) issue_loads(cn, use_blk(blk_next));
+        // asked for behind the chunk's loads, the next table entry is there when they all are: the wave rests here
+        // until chunk cn has landed and only then works on chunk c
+        blk_next = __builtin_amdgcn_readfirstlane(load_blk(cn + NW));
         __builtin_amdgcn_sched_barrier(0);
 
         // ---- S^T = K Q^T : two 16-key tiles x RT row tiles

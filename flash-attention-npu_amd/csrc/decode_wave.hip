@@ -198,13 +198,13 @@ __device__ __forceinline__ void wave_piece(const DecodeParams &p, const int b, c
     const uint32_t k_lane_off = (uint32_t)k_lane_row * k_row_bytes + k_lane_col;
     const uint32_t v_lane_off = (uint32_t)(lq * 4) * v_row_bytes + v_lane_col;
 
-    auto fetch_blk = [&](int c) -> int {
+    auto load_blk = [&](int c) -> int {   // the table entry as loaded (every lane the same address); not waited for
         if (c >= c_end) return 0;
         int page = (c * kChunk) / p.page_size;
         page = min(page, p.max_blocks - 1);
-        const int blk = __builtin_amdgcn_readfirstlane(bt_row[page]);
-        return min(max(blk, 0), p.num_blocks - 1);
+        return bt_row[page];
     };
+    auto use_blk = [&](int raw) -> int { return min(max(__builtin_amdgcn_readfirstlane(raw), 0), p.num_blocks - 1); };
     auto load_v = [&](const uint8_t *s2, int e, int hh) {
         if constexpr (Cfg::kVW == 8) {
             const u32x4_t t4 = load16_stream(s2);
@@ -265,9 +265,15 @@ __device__ __forceinline__ void wave_piece(const DecodeParams &p, const int b, c
 
     // first chunk in flight while Q is staged
     int c = c_begin;
-    int blk_next = fetch_blk(c);
-    if (c < c_end) issue_loads(c, blk_next);
-    blk_next = fetch_blk(c + 1);
+    int blk_next;
+    {
+        // Both table entries are asked for before the first chunk's loads.  Loads return in order: asked for behind
+        // them, the second entry would only be there when the whole chunk is, and the q rows would be requested a
+        // memory latency later than they need be.
+        const int blk0 = load_blk(c);
+        blk_next = load_blk(c + 1);
+        if (c < c_end) issue_loads(c, use_blk(blk0));
+    }
 
     stage_q_wave<T, D, PART>(p, b, kvh, ur.len_cache, sq);
     __builtin_amdgcn_wave_barrier();
@@ -322,8 +328,10 @@ __device__ __forceinline__ void wave_piece(const DecodeParams &p, const int b, c
         __builtin_amdgcn_wave_barrier();
 
         const int cn = c + 1;
-        if (cn < c_end) issue_loads(cn, blk_next);
-        blk_next = fetch_blk(cn + 1);
+        if (cn < c_end) issue_loads(cn, use_blk(blk_next));
+        // asked for behind the chunk's loads, the next table entry is there when they all are: the wave rests here
+        // until chunk cn has landed and only then works on chunk c
+        blk_next = __builtin_amdgcn_readfirstlane(load_blk(cn + 1));
         __builtin_amdgcn_sched_barrier(0);
 
         // S^T = K Q^T, two 16-key tiles
