@@ -312,6 +312,9 @@ __device__ __forceinline__ void prefill_block(const PrefillParams &p, const unsi
         // fills four rows of one wave) only helps to move the tiles, and leaves the matrix pipe to the others
         if (wave_live) {
         // ---- S^T = K Q^T for the two 32-key halves of the tile
+        // the wave in a matrix phase goes first: its MFMAs then issue back to back and the vector work of the SIMD's other
+        // wave fills the gaps between them (c5: 870 -> 856 us)
+        __builtin_amdgcn_s_setprio(1);
         float16_t s[2];
 #pragma unroll
         for (int tt = 0; tt < 2; ++tt)
@@ -339,6 +342,7 @@ __device__ __forceinline__ void prefill_block(const PrefillParams &p, const unsi
             __builtin_amdgcn_sched_barrier(0);
         }
 
+        __builtin_amdgcn_s_setprio(0);
         // ---- online softmax; lane column = query row, register r of half tt = key
         //      kt*64 + tt*32 + 8*(r/4) + 4*lh + r%4
         const int tile0 = kt * kBN;
@@ -442,6 +446,7 @@ __device__ __forceinline__ void prefill_block(const PrefillParams &p, const unsi
         }
         l_run += psum;
 
+        __builtin_amdgcn_s_setprio(1);
         // ---- O^T += V^T P^T, 16 keys per step.  The V^T operand comes from the transposing LDS read
         //      (ds_read_b64_tr_b16): in every 16-lane group, lane s points at 4 columns of key row
         //      s/4 and receives column s (of the group's 16) for the group's 4 key rows.  Column tile
@@ -472,6 +477,7 @@ __device__ __forceinline__ void prefill_block(const PrefillParams &p, const unsi
                     o_acc[t] = mfma32<T>(va[t], pk[tt][ks], o_acc[t]);
                 }
             }
+        __builtin_amdgcn_s_setprio(0);
         }   // wave_live
 
         if (more) stash_tile(cur ^ 1);
