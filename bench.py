@@ -35,7 +35,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
 # FETCH_SIZE / WRITE_SIZE counter passes whose summaries are tracked under profiles/ (a line
 # "traffic_bytes_per_launch: N" in the summary of that kernel and workload).  The workloads are seeded, so the
 # figure belongs to the kernel as it was when the summary was made; the record names the file it was read from.
-PROFILE_OF = {"c2": "decode_wave_kernel_c2.txt", "c3a": "decode_wave_kernel_c3a.txt", "c3b": "decode_wave_kernel_c3b.txt",
+PROFILE_OF = {"c2": "decode_wave_kernel_c2.txt", "c2_8k": "decode_wave_kernel_c2_8k.txt", "c3a": "decode_wave_kernel_c3a.txt", "c3b": "decode_wave_kernel_c3b.txt",
               "c4": "decode_mla_i8_kernel_c4.txt", "c5": "prefill_kernel_c5.txt"}
 
 
