@@ -173,22 +173,62 @@ __device__ __forceinline__ void combine_row_wave(const DecodeParams &p, int b, i
     static_assert(CPL == 1 || CPL == 2 || CPL == 4 || CPL == 8, "column split");
     if (row_id(p, kvh, row).head >= p.nheads) return;   // a row of the latent kernel's last, partly empty head group
     const int lane = threadIdx.x & 63;
+    constexpr int PB = (CPL >= 8) ? 4 : 8;   // pieces whose rows are in flight together
     float mx = -INFINITY;
-    for (int s = lane; s < ns; s += 64) mx = fmaxf(mx, p.lse_partial[slot_of(s) * p.rows + row]);
-#pragma unroll
-    for (int d = 32; d >= 1; d >>= 1) mx = fmaxf(mx, __shfl_xor(mx, d, 64));
-    const float mx_use = (mx == -INFINITY) ? 0.f : mx;
     float tot = 0.f;
     float acc[CPL];
 #pragma unroll
     for (int c = 0; c < CPL; ++c) acc[c] = 0.f;
-    for (int s = 0; s < ns; ++s) {
-        const int64_t srow = slot_of(s) * p.rows + row;
-        const float w = fast_exp2(p.lse_partial[srow] - mx_use);
-        tot += w;
-        const float *src = p.o_partial + srow * DV + lane * CPL;
+    // The pieces of a unit were written by other compute units: every dependent load is a trip to memory.  Rows and
+    // log-sum-exps of PB pieces are therefore requested together and only then used; a unit of at most PB pieces (the
+    // common case) is merged with a single trip, the maximum taken from the values every lane then holds.
+    auto fetch = [&](int s0, float (&lw)[PB], float (&v)[PB][CPL]) {
 #pragma unroll
-        for (int c = 0; c < CPL; ++c) acc[c] += w * src[c];
+        for (int i = 0; i < PB; ++i) {
+            const int64_t srow = slot_of(min(s0 + i, ns - 1)) * p.rows + row;
+            lw[i] = (s0 + i < ns) ? p.lse_partial[srow] : -INFINITY;
+            const float *src = p.o_partial + srow * DV + lane * CPL;
+            if constexpr (CPL == 1) {
+                v[i][0] = src[0];
+            } else if constexpr (CPL == 2) {
+                const float2 t = *reinterpret_cast<const float2 *>(src);
+                v[i][0] = t.x, v[i][1] = t.y;
+            } else {
+#pragma unroll
+                for (int c = 0; c < CPL; c += 4) {
+                    const float4 t = *reinterpret_cast<const float4 *>(src + c);
+                    v[i][c] = t.x, v[i][c + 1] = t.y, v[i][c + 2] = t.z, v[i][c + 3] = t.w;
+                }
+            }
+        }
+    };
+    auto add = [&](const float (&lw)[PB], const float (&v)[PB][CPL], float mx_use) {
+#pragma unroll
+        for (int i = 0; i < PB; ++i) {
+            const float w = fast_exp2(lw[i] - mx_use);   // 0 behind the last piece (-inf)
+            tot += w;
+#pragma unroll
+            for (int c = 0; c < CPL; ++c) acc[c] += w * v[i][c];
+        }
+    };
+    if (ns <= PB) {
+        float lw[PB];
+        float v[PB][CPL];
+        fetch(0, lw, v);
+#pragma unroll
+        for (int i = 0; i < PB; ++i) mx = fmaxf(mx, lw[i]);
+        add(lw, v, (mx == -INFINITY) ? 0.f : mx);
+    } else {
+        for (int s = lane; s < ns; s += 64) mx = fmaxf(mx, p.lse_partial[slot_of(s) * p.rows + row]);
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) mx = fmaxf(mx, __shfl_xor(mx, d, 64));
+        const float mx_use = (mx == -INFINITY) ? 0.f : mx;
+        for (int s0 = 0; s0 < ns; s0 += PB) {
+            float lw[PB];
+            float v[PB][CPL];
+            fetch(s0, lw, v);
+            add(lw, v, mx_use);
+        }
     }
     const float inv = (tot > 0.f) ? 1.f / tot : 0.f;
     const RowId rid = row_id(p, kvh, row);

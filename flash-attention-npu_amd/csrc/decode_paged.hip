@@ -551,15 +551,25 @@ __device__ __forceinline__ void combine_row_block(const DecodeParams &p, int b, 
     const int pl = tid / CG;
     float tot = 0.f;
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
-    for (int s2 = pl; s2 < ns; s2 += NPL) {
-        const int64_t srow = pcs.slot(s2) * p.rows + row;
-        const float w = fast_exp2(p.lse_partial[srow] - mx_use);
-        tot += w;
-        const float4 o = *reinterpret_cast<const float4 *>(p.o_partial + srow * D + cg * 4);
-        acc[0] += w * o.x;
-        acc[1] += w * o.y;
-        acc[2] += w * o.z;
-        acc[3] += w * o.w;
+    // four of the thread's pieces are requested before the first is used (one trip to memory per four)
+    for (int s0 = pl; s0 < ns; s0 += 4 * NPL) {
+        float lw[4];
+        float4 o[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int64_t srow = pcs.slot(min(s0 + i * NPL, ns - 1)) * p.rows + row;
+            lw[i] = p.lse_partial[srow];
+            o[i] = *reinterpret_cast<const float4 *>(p.o_partial + srow * D + cg * 4);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float w = (s0 + i * NPL < ns) ? fast_exp2(lw[i] - mx_use) : 0.f;
+            tot += w;
+            acc[0] += w * o[i].x;
+            acc[1] += w * o[i].y;
+            acc[2] += w * o[i].z;
+            acc[3] += w * o[i].w;
+        }
     }
     *reinterpret_cast<float4 *>(&s_acc[pl][cg * 4]) = make_float4(acc[0], acc[1], acc[2], acc[3]);
     if (cg == 0) s_tot[pl] = tot;
