@@ -610,29 +610,61 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
         }
     }
     __syncthreads();
-    // ---- write this wave's 128-column slice of every head
+    // ---- write this wave's 128-column slice of every head.  A lane holds 16-byte pieces of 32 different rows: stored as
+    //      they are, every instruction would touch 32 rows of the output.  The slice of one head group (32 rows x 128
+    //      columns, fp32) goes through a staging area of the wave's own inside the key tiles (free after the barrier
+    //      above) and leaves as whole rows, 16 bytes per lane.
+    constexpr int kStageRowBytes = 128 * 4 + 16;                     // padded: the 16 lanes the LDS serves per cycle hit 64 banks
+    static_assert(4 * 32 * kStageRowBytes <= 3 * kMlaTileBytes, "the staging areas must fit the key tiles");
+    uint8_t *stage = &sh.k[0][0] + wave * (32 * kStageRowBytes);
+    // Everything the stores need is derived from the lane number HERE: the walk over the pieces of a share is a loop,
+    // and per-lane constants computed outside it would be kept alive through the main loop, where there is no
+    // register to spare (they were spilled, and every reload waited for the store before it).
+    int lane_e = lane;
+    asm volatile("" : "+v"(lane_e));
+    const int ln_e = lane_e & 31, lh_e = lane_e >> 5;
     static_for<0, 4>([&](auto hg_) {
         constexpr int hg = decltype(hg_)::value;
-        const int row = hg * 32 + ln;
-        const int hd = hgrp * kMlaUnitHeads + row;
-        const float lg = sh.l[row];
+        const float lg = sh.l[hg * 32 + ln_e];
         const float inv = (lg > 0.f) ? 1.f / lg : 0.f;
-        const bool live = hd < p.nheads;
-        uint16_t *dst16 = reinterpret_cast<uint16_t *>(p.out) + (int64_t)b * p.o_stride_b + (int64_t)qi * p.o_stride_s +
-                          (int64_t)hd * p.o_stride_h + wave * 128 + 4 * lh;
-        float *dst32 = p.o_partial + (slot * p.rows + row) * kMlaDv + wave * 128 + 4 * lh;
         static_for<0, 16>([&](auto t_) {
             constexpr int cc = decltype(t_)::value >> 2, g = decltype(t_)::value & 3;
             constexpr int base = 16 * (4 * cc + hg) + 4 * g;
             const float o0 = acc_read<base>() * inv, o1 = acc_read<base + 1>() * inv;
             const float o2 = acc_read<base + 2>() * inv, o3 = acc_read<base + 3>() * inv;
-            if (live) {
-                if (write_final)
-                    *reinterpret_cast<uint2 *>(dst16 + cc * 32 + g * 8) = make_uint2(pack2<T>(o0, o1), pack2<T>(o2, o3));
-                else
-                    *reinterpret_cast<float4 *>(dst32 + cc * 32 + g * 8) = make_float4(o0, o1, o2, o3);
-            }
+            *reinterpret_cast<float4 *>(stage + ln_e * kStageRowBytes + (cc * 32 + g * 8 + 4 * lh_e) * 4) = make_float4(o0, o1, o2, o3);
         });
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        const int hd0 = hgrp * kMlaUnitHeads + hg * 32;               // head of the staged row 0
+        if (write_final) {
+            // 128 columns of the 16-bit type = 256 bytes = 16 lanes: four rows per instruction
+            const int c = lane_e & 15;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int r = (lane_e >> 4) + 4 * i;
+                const float4 x = *reinterpret_cast<const float4 *>(stage + r * kStageRowBytes + c * 32);
+                const float4 y = *reinterpret_cast<const float4 *>(stage + r * kStageRowBytes + c * 32 + 16);
+                if (hd0 + r < p.nheads) {
+                    uint16_t *dst = reinterpret_cast<uint16_t *>(p.out) + (int64_t)b * p.o_stride_b + (int64_t)qi * p.o_stride_s +
+                                    (int64_t)(hd0 + r) * p.o_stride_h + wave * 128 + c * 8;
+                    store16(dst, u32x4_t{pack2<T>(x.x, x.y), pack2<T>(x.z, x.w), pack2<T>(y.x, y.y), pack2<T>(y.z, y.w)});
+                }
+            }
+        } else {
+            // 128 fp32 columns = 512 bytes = 32 lanes: two rows per instruction
+            const int c = lane_e & 31;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int r = (lane_e >> 5) + 2 * i;
+                const float4 x = *reinterpret_cast<const float4 *>(stage + r * kStageRowBytes + c * 16);
+                if (hd0 + r < p.nheads)
+                    *reinterpret_cast<float4 *>(p.o_partial + (slot * p.rows + hg * 32 + r) * kMlaDv + wave * 128 + c * 4) = x;
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();   // the staging area is rewritten by the next head group
     });
     __syncthreads();   // the LDS tiles and sums are reused by the next piece
 }
