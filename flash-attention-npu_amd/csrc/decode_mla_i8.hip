@@ -144,6 +144,25 @@ template <int R> __device__ __forceinline__ void acc_scale(float f) {
 // registers (and back): the hazards the compiler would cover for instructions it knows
 __device__ __forceinline__ void mfma_settle() { asm volatile("s_nop 15\n\ts_nop 3" ::: "memory", MLA_ALL_ACC); }
 
+// Eight 16-byte LDS reads at constant offsets from one address, issued back to back, then one wait.  Written out by
+// hand because the compiler pairs every such read with the store that uses it (sixteen exposed LDS latencies per pass
+// of the epilogue) whatever the source order is.
+template <int STRIDE> __device__ __forceinline__ void lds_read8x16(uint32_t addr, float4 (&v)[8]) {
+    asm volatile(
+        "ds_read_b128 %0, %8\n\t"
+        "ds_read_b128 %1, %8 offset:%9\n\t"
+        "ds_read_b128 %2, %8 offset:%10\n\t"
+        "ds_read_b128 %3, %8 offset:%11\n\t"
+        "ds_read_b128 %4, %8 offset:%12\n\t"
+        "ds_read_b128 %5, %8 offset:%13\n\t"
+        "ds_read_b128 %6, %8 offset:%14\n\t"
+        "ds_read_b128 %7, %8 offset:%15\n\t"
+        "s_waitcnt lgkmcnt(0)"
+        : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3]), "=&v"(v[4]), "=&v"(v[5]), "=&v"(v[6]), "=&v"(v[7])
+        : "v"(addr), "n"(STRIDE), "n"(2 * STRIDE), "n"(3 * STRIDE), "n"(4 * STRIDE), "n"(5 * STRIDE), "n"(6 * STRIDE), "n"(7 * STRIDE)
+        : "memory");
+}
+
 struct MlaShared {
     __attribute__((aligned(16))) uint8_t k[3][kMlaTileBytes];   // widened key tiles
     struct __attribute__((aligned(16))) Scales {                 // per-token scales of a tile, side by side: one LDS base address
@@ -171,7 +190,11 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
     const int row_off = ur.Lk - p.seqlen_q + qi;                       // key aligned with this query token
     const int mask_lo = max(range_lo, ur.wl >= 0 ? row_off - ur.wl : 0);
     const int mask_hi = min(range_hi, ur.wr >= 0 ? row_off + ur.wr + 1 : ur.Lk);
-    const int tid = threadIdx.x;
+    // The thread number is made opaque here: a worker walks the pieces of its share in a loop, and everything derived
+    // from the lane (LDS offsets, swizzles, row numbers) would otherwise be computed once outside that loop and kept
+    // alive through prologue and epilogue, where the registers are needed for other things.
+    int tid = threadIdx.x;
+    asm volatile("" : "+v"(tid));
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lane = tid & 63;
     const int ln = lane & 31;     // MFMA column: head of the wave's group (scores), head of a group (output)
@@ -638,29 +661,52 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         const int hd0 = hgrp * kMlaUnitHeads + hg * 32;               // head of the staged row 0
+        // all LDS reads of the pass first (constant offsets from one address), then the stores (one pointer, constant
+        // strides); a head group that is complete - every one but possibly the unit's last - needs no per-row test
+        const bool full = hd0 + 32 <= p.nheads;                       // wave-uniform
         if (write_final) {
             // 128 columns of the 16-bit type = 256 bytes = 16 lanes: four rows per instruction
-            const int c = lane_e & 15;
+            const int c = lane_e & 15, r0 = lane_e >> 4;
+            const uint8_t *src = stage + r0 * kStageRowBytes + c * 32;
+            float4 x[8], y[8];
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
-                const int r = (lane_e >> 4) + 4 * i;
-                const float4 x = *reinterpret_cast<const float4 *>(stage + r * kStageRowBytes + c * 32);
-                const float4 y = *reinterpret_cast<const float4 *>(stage + r * kStageRowBytes + c * 32 + 16);
-                if (hd0 + r < p.nheads) {
-                    uint16_t *dst = reinterpret_cast<uint16_t *>(p.out) + (int64_t)b * p.o_stride_b + (int64_t)qi * p.o_stride_s +
-                                    (int64_t)(hd0 + r) * p.o_stride_h + wave * 128 + c * 8;
-                    store16(dst, u32x4_t{pack2<T>(x.x, x.y), pack2<T>(x.z, x.w), pack2<T>(y.x, y.y), pack2<T>(y.z, y.w)});
-                }
+                x[i] = *reinterpret_cast<const float4 *>(src + 4 * i * kStageRowBytes);
+                y[i] = *reinterpret_cast<const float4 *>(src + 4 * i * kStageRowBytes + 16);
+            }
+            uint16_t *dst = reinterpret_cast<uint16_t *>(p.out) + (int64_t)b * p.o_stride_b + (int64_t)qi * p.o_stride_s +
+                            (int64_t)(hd0 + r0) * p.o_stride_h + wave * 128 + c * 8;
+            const int64_t step = 4 * p.o_stride_h;
+            auto put = [&](int i) {
+                store16(dst + i * step, u32x4_t{pack2<T>(x[i].x, x[i].y), pack2<T>(x[i].z, x[i].w), pack2<T>(y[i].x, y[i].y),
+                                                pack2<T>(y[i].z, y[i].w)});
+            };
+            if (full) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) put(i);
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i)
+                    if (hd0 + r0 + 4 * i < p.nheads) put(i);
             }
         } else {
             // 128 fp32 columns = 512 bytes = 32 lanes: two rows per instruction
-            const int c = lane_e & 31;
+            const int c = lane_e & 31, r0 = lane_e >> 5;
+            const uint8_t *src = stage + r0 * kStageRowBytes + c * 16;
+            const uint32_t src_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const uint8_t *)src;
+            float *dst = p.o_partial + (slot * p.rows + hg * 32 + r0) * kMlaDv + wave * 128 + c * 4;
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const int r = (lane_e >> 5) + 2 * i;
-                const float4 x = *reinterpret_cast<const float4 *>(stage + r * kStageRowBytes + c * 16);
-                if (hd0 + r < p.nheads)
-                    *reinterpret_cast<float4 *>(p.o_partial + (slot * p.rows + hg * 32 + r) * kMlaDv + wave * 128 + c * 4) = x;
+            for (int i0 = 0; i0 < 16; i0 += 8) {
+                float4 x[8];
+                lds_read8x16<2 * kStageRowBytes>(src_lds + 2 * i0 * kStageRowBytes, x);
+                if (full) {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) *reinterpret_cast<float4 *>(dst + 2 * (i0 + i) * kMlaDv) = x[i];
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i)
+                        if (hd0 + r0 + 2 * (i0 + i) < p.nheads) *reinterpret_cast<float4 *>(dst + 2 * (i0 + i) * kMlaDv) = x[i];
+                }
             }
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
