@@ -173,7 +173,8 @@ __device__ __forceinline__ void combine_row_wave(const DecodeParams &p, int b, i
     static_assert(CPL == 1 || CPL == 2 || CPL == 4 || CPL == 8, "column split");
     if (row_id(p, kvh, row).head >= p.nheads) return;   // a row of the latent kernel's last, partly empty head group
     const int lane = threadIdx.x & 63;
-    constexpr int PB = (CPL >= 8) ? 4 : 8;   // pieces whose rows are in flight together
+    constexpr bool HALF = partials_are_half(DV);
+    constexpr int PB = (CPL >= 8 && !HALF) ? 4 : 8;   // pieces whose rows are in flight together
     float mx = -INFINITY;
     float tot = 0.f;
     float acc[CPL];
@@ -188,7 +189,15 @@ __device__ __forceinline__ void combine_row_wave(const DecodeParams &p, int b, i
             const int64_t srow = slot_of(min(s0 + i, ns - 1)) * p.rows + row;
             lw[i] = (s0 + i < ns) ? p.lse_partial[srow] : -INFINITY;
             const float *src = p.o_partial + srow * DV + lane * CPL;
-            if constexpr (CPL == 1) {
+            if constexpr (HALF) {
+                static_assert(!HALF || CPL == 8, "16-bit partial rows are read 16 bytes per lane");
+                const u32x4_t t = *reinterpret_cast<const u32x4_t *>(reinterpret_cast<const uint16_t *>(p.o_partial) + srow * DV + lane * CPL);
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    v[i][2 * c] = to_float<FP16>((uint16_t)(t[c] & 0xffffu));
+                    v[i][2 * c + 1] = to_float<FP16>((uint16_t)(t[c] >> 16));
+                }
+            } else if constexpr (CPL == 1) {
                 v[i][0] = src[0];
             } else if constexpr (CPL == 2) {
                 const float2 t = *reinterpret_cast<const float2 *>(src);

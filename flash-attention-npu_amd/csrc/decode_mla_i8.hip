@@ -664,50 +664,42 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
         // all LDS reads of the pass first (constant offsets from one address), then the stores (one pointer, constant
         // strides); a head group that is complete - every one but possibly the unit's last - needs no per-row test
         const bool full = hd0 + 32 <= p.nheads;                       // wave-uniform
+        // 128 columns of a 16-bit type = 256 bytes = 16 lanes: four rows per instruction.  The final output is in the
+        // I/O type; the partial rows of a split unit are fp16 (partials_are_half), clamped to its range.
+        const int c = lane_e & 15, r0 = lane_e >> 4;
+        const uint8_t *src = stage + r0 * kStageRowBytes + c * 32;
+        const uint32_t src_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const uint8_t *)src;
+        float4 x[8], y[8];
+        lds_read8x16<4 * kStageRowBytes>(src_lds, x);
+        lds_read8x16<4 * kStageRowBytes>(src_lds + 16, y);
+        uint16_t *dst;
+        int64_t step;
         if (write_final) {
-            // 128 columns of the 16-bit type = 256 bytes = 16 lanes: four rows per instruction
-            const int c = lane_e & 15, r0 = lane_e >> 4;
-            const uint8_t *src = stage + r0 * kStageRowBytes + c * 32;
-            float4 x[8], y[8];
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                x[i] = *reinterpret_cast<const float4 *>(src + 4 * i * kStageRowBytes);
-                y[i] = *reinterpret_cast<const float4 *>(src + 4 * i * kStageRowBytes + 16);
-            }
-            uint16_t *dst = reinterpret_cast<uint16_t *>(p.out) + (int64_t)b * p.o_stride_b + (int64_t)qi * p.o_stride_s +
-                            (int64_t)(hd0 + r0) * p.o_stride_h + wave * 128 + c * 8;
-            const int64_t step = 4 * p.o_stride_h;
-            auto put = [&](int i) {
+            dst = reinterpret_cast<uint16_t *>(p.out) + (int64_t)b * p.o_stride_b + (int64_t)qi * p.o_stride_s +
+                  (int64_t)(hd0 + r0) * p.o_stride_h + wave * 128 + c * 8;
+            step = 4 * p.o_stride_h;
+        } else {
+            static_assert(partials_are_half(kMlaDv), "the merge reads these rows as fp16");
+            dst = reinterpret_cast<uint16_t *>(p.o_partial) + (slot * p.rows + hg * 32 + r0) * kMlaDv + wave * 128 + c * 8;
+            step = 4 * kMlaDv;
+        }
+        auto put = [&](int i) {
+            if (write_final) {
                 store16(dst + i * step, u32x4_t{pack2<T>(x[i].x, x[i].y), pack2<T>(x[i].z, x[i].w), pack2<T>(y[i].x, y[i].y),
                                                 pack2<T>(y[i].z, y[i].w)});
-            };
-            if (full) {
-#pragma unroll
-                for (int i = 0; i < 8; ++i) put(i);
             } else {
-#pragma unroll
-                for (int i = 0; i < 8; ++i)
-                    if (hd0 + r0 + 4 * i < p.nheads) put(i);
+                auto cl = [](float v) { return __builtin_amdgcn_fmed3f(v, -65504.f, 65504.f); };
+                store16(dst + i * step, u32x4_t{pack2<FP16>(cl(x[i].x), cl(x[i].y)), pack2<FP16>(cl(x[i].z), cl(x[i].w)),
+                                                pack2<FP16>(cl(y[i].x), cl(y[i].y)), pack2<FP16>(cl(y[i].z), cl(y[i].w))});
             }
+        };
+        if (full) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) put(i);
         } else {
-            // 128 fp32 columns = 512 bytes = 32 lanes: two rows per instruction
-            const int c = lane_e & 31, r0 = lane_e >> 5;
-            const uint8_t *src = stage + r0 * kStageRowBytes + c * 16;
-            const uint32_t src_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const uint8_t *)src;
-            float *dst = p.o_partial + (slot * p.rows + hg * 32 + r0) * kMlaDv + wave * 128 + c * 4;
 #pragma unroll
-            for (int i0 = 0; i0 < 16; i0 += 8) {
-                float4 x[8];
-                lds_read8x16<2 * kStageRowBytes>(src_lds + 2 * i0 * kStageRowBytes, x);
-                if (full) {
-#pragma unroll
-                    for (int i = 0; i < 8; ++i) *reinterpret_cast<float4 *>(dst + 2 * (i0 + i) * kMlaDv) = x[i];
-                } else {
-#pragma unroll
-                    for (int i = 0; i < 8; ++i)
-                        if (hd0 + r0 + 2 * (i0 + i) < p.nheads) *reinterpret_cast<float4 *>(dst + 2 * (i0 + i) * kMlaDv) = x[i];
-                }
-            }
+            for (int i = 0; i < 8; ++i)
+                if (hd0 + r0 + 4 * i < p.nheads) put(i);
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();   // the staging area is rewritten by the next head group

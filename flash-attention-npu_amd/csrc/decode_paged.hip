@@ -559,7 +559,13 @@ __device__ __forceinline__ void combine_row_block(const DecodeParams &p, int b, 
         for (int i = 0; i < 4; ++i) {
             const int64_t srow = pcs.slot(min(s0 + i * NPL, ns - 1)) * p.rows + row;
             lw[i] = p.lse_partial[srow];
-            o[i] = *reinterpret_cast<const float4 *>(p.o_partial + srow * D + cg * 4);
+            if constexpr (partials_are_half(D)) {
+                const uint2 t = *reinterpret_cast<const uint2 *>(reinterpret_cast<const uint16_t *>(p.o_partial) + srow * D + cg * 4);
+                o[i] = make_float4(to_float<FP16>((uint16_t)(t.x & 0xffffu)), to_float<FP16>((uint16_t)(t.x >> 16)),
+                                   to_float<FP16>((uint16_t)(t.y & 0xffffu)), to_float<FP16>((uint16_t)(t.y >> 16)));
+            } else {
+                o[i] = *reinterpret_cast<const float4 *>(p.o_partial + srow * D + cg * 4);
+            }
         }
 #pragma unroll
         for (int i = 0; i < 4; ++i) {

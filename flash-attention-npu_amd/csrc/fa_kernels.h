@@ -154,6 +154,13 @@ struct PrefillParams {
     float *lse_partial;
 };
 
+// The partial rows of the 512-column kernel (the int8 latent cache: 128 heads x 512 columns per piece) are kept as
+// fp16: they are normalised outputs, i.e. averages of dequantised cache rows (11 significant bits against the 8 or 11
+// of the final rounding), and halving them halves what the split costs in writes and in the merge's reads.  Their
+// writer clamps to the fp16 range.  Every other width keeps fp32 partials.
+constexpr bool partials_are_half(int dv) { return dv == 512; }
+
+
 // Width the kernels are compiled for, for a head dimension of d columns.
 inline int tile_headdim(int d) { return d <= 64 ? 64 : d <= 128 ? 128 : 256; }
 

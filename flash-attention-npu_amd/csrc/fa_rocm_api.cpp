@@ -53,6 +53,12 @@ bool is_mla_i8(const fa_kvcache_args *a) { return a->kv_dtype == FA_INT8; }
 
 // columns of a row of fp32 partials: the width the kernels are compiled for
 int partial_width(const fa_kvcache_args *a) { return is_mla_i8(a) ? a->headdim_v : fa::tile_headdim(a->headdim_v); }
+// bytes of one partial row in the workspace: its columns (fp16 for the 512-column latent kernel, fp32 otherwise) and
+// its fp32 log-sum-exp
+size_t partial_row_bytes(const fa_kvcache_args *a) {
+    const int w = partial_width(a);
+    return (size_t)w * (fa::partials_are_half(w) ? sizeof(uint16_t) : sizeof(float)) + sizeof(float);
+}
 
 // Experiment knobs and the validation switch, from the environment.  They are read ONCE, on the first call that
 // needs them (or again when fa_rocm_reload_env() is called): nothing on the call path touches the environment.
@@ -295,7 +301,7 @@ int fa_rocm_plan_kvcache(const fa_kvcache_args *a, int num_cus, fa_split_plan *p
     const int group = a->nheads / a->nheads_k;
     // the int8 latent kernel works on units of 128 query heads and always uses the balanced partition
     const size_t rows = is_mla_i8(a) ? 128 : (size_t)a->seqlen_q * group;
-    const size_t slot_bytes = rows * ((size_t)partial_width(a) + 1) * sizeof(float);
+    const size_t slot_bytes = rows * partial_row_bytes(a);
     if (!is_mla_i8(a) && rows > (size_t)decode_max_rows(a)) {
         // Query block too tall for the decode kernels: the tiled forward.  When its tiles alone
         // cannot fill the device (few sequences, short blocks) the keys of every unit are cut into
@@ -660,9 +666,9 @@ static int fwd_kvcache_impl(const fa_kvcache_args *a, void *stream_, void *const
                         !env().no_head_interleave;
     const bool needs_combine = need > 0;
     if (needs_combine) {
-        const size_t slot_rows = need / (((size_t)partial_width(a) + 1) * sizeof(float));
+        const size_t slot_rows = need / partial_row_bytes(a);
         p.o_partial = static_cast<float *>(a->workspace);
-        p.lse_partial = p.o_partial + slot_rows * partial_width(a);
+        p.lse_partial = reinterpret_cast<float *>(static_cast<char *>(a->workspace) + slot_rows * (partial_row_bytes(a) - sizeof(float)));
     }
 
     // The wave-level kernel appends on the fly when every new position is certain to be visible
