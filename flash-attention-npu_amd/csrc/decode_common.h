@@ -390,12 +390,12 @@ template <int DV> __device__ __forceinline__ void init_empty_units(const DecodeP
     }
 }
 
-// Workgroup-level worker: the share of workgroup blockIdx.x, then the empty-unit duty.
+// Workgroup-level worker: the share `worker` (a permutation of the workgroup numbers), then the empty-unit duty.
 template <int DV, typename PieceFn>
-__device__ __forceinline__ void balanced_driver(const DecodeParams &p, PieceFn piece) {
+__device__ __forceinline__ void balanced_driver(const DecodeParams &p, int worker, PieceFn piece) {
     __shared__ int s_pref[257];
     const Partition pt = make_partition(p, s_pref);
-    walk_share(p, pt, s_pref, blockIdx.x, piece);
+    walk_share(p, pt, s_pref, worker, piece);
     init_empty_units<DV>(p, pt);
 }
 

@@ -710,7 +710,11 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
 template <typename T, bool SOFTCAP>
 __global__ void __launch_bounds__(kMlaThreads) decode_mla_i8_kernel(const DecodeParams p) {
     __shared__ MlaShared sh;
-    balanced_driver<kMlaDv>(p, [&](int b, int unit, const UnitRange &ur, int range_lo, int range_hi, bool whole, int64_t slot) {
+    // Neighbouring shares are mostly pieces of one batch row and read the same 147 KB of Q.  Workgroup x runs on XCD
+    // x % 8 (each XCD has its own L2): the shares are dealt so that eight neighbours meet in one L2.
+    const int G = gridDim.x;
+    const int worker = (G & 7) ? (int)blockIdx.x : (int)(blockIdx.x & 7) * (G >> 3) + (int)(blockIdx.x >> 3);
+    balanced_driver<kMlaDv>(p, worker, [&](int b, int unit, const UnitRange &ur, int range_lo, int range_hi, bool whole, int64_t slot) {
         mla_piece<T, SOFTCAP>(p, b, unit, ur, range_lo, range_hi, whole, slot, sh);
     });
 }

@@ -502,7 +502,7 @@ template <typename T, int D, int RT, int NW, bool SOFTCAP, bool PART>
 __global__ void __launch_bounds__(NW * 64, (D <= 128 && RT <= 2) ? 2 : 1)
 decode_balanced_kernel(const DecodeParams p) {
     static_assert(NW == 4, "the batch scan assumes 256 threads");
-    balanced_driver<D>(p, [&](int b, int kvh, const UnitRange &ur, int range_lo, int range_hi, bool whole, int64_t slot) {
+    balanced_driver<D>(p, blockIdx.x, [&](int b, int kvh, const UnitRange &ur, int range_lo, int range_hi, bool whole, int64_t slot) {
         process_piece<T, D, RT, NW, SOFTCAP, PART>(p, b, kvh, ur, range_lo, range_hi, whole, slot);
     });
 }

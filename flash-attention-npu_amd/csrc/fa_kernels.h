@@ -25,7 +25,7 @@ struct DecodeParams {
     const int32_t *block_table;
     const int32_t *q_live;   // per batch row: how many query tokens, at the END of the block, are real; the rows of the
                              // others are computed but neither written nor merged.  NULL: all (balanced wave-level launch only)
-    float *o_partial;    // (B, Hk, nsplits, rows, Dv) fp32, each normalised by its own sum
+    float *o_partial;    // (B, Hk, nsplits, rows, Dv) fp32 (fp16 where partials_are_half(Dv)), each normalised by its own sum
     float *lse_partial;  // (B, Hk, nsplits, rows)     fp32, base-2 log-sum-exp, -inf when empty
     int32_t batch, seqlen_q, nheads, nheads_k, group, rows;  // rows = seqlen_q * group
     int32_t headdim;     // columns of an output row (and of a q / k / v row, except for the latent cache): a multiple of 8;

@@ -196,7 +196,7 @@ typedef struct fa_split_plan {
     int32_t num_wgs;          /* balanced mode: workgroups launched              */
     int32_t num_workers;      /* balanced mode: workers sharing the chunk list (a workgroup, or each of its 4 waves) */
     int32_t min_share;        /* balanced mode: least 32-key chunks per share    */
-    size_t workspace_bytes;   /* fp32 partial outputs + LSEs the call needs      */
+    size_t workspace_bytes;   /* partial outputs + LSEs the call needs           */
 } fa_split_plan;
 int fa_rocm_plan_kvcache(const fa_kvcache_args *args, int num_cus, fa_split_plan *plan);
 
