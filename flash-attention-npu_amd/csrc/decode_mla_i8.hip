@@ -210,18 +210,53 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
     const int blk_first = bt_row[min((c_begin * kChunk) / p.page_size, p.max_blocks - 1)];
     const int blk_second = bt_row[min(((c_begin + min(1, nch - 1)) * kChunk) / p.page_size, p.max_blocks - 1)];
 
-    // ---- Q^T operands: lane (ln, lh) holds head 32*wave + ln, dims 16t + 8lh .. +7 of k-step t
+    // ---- Q^T operands: lane (ln, lh) holds head 32*wave + ln, dims 16t + 8lh .. +7 of k-step t.  Loaded in that
+    //      layout, one instruction would touch 32 rows of q, 32 bytes each (measured: 9 us of the kernel).  The wave's 32
+    //      rows are fetched as they lie instead - half a row (576 bytes = 36 lanes) after the other, two rounds of 18
+    //      instructions, all requested here - and turned into the operand layout through a staging area of the wave's
+    //      own (stage_q below, once the first chunk's loads are out as well).
     const int row_u = wave * 32 + ln;                                  // row of the unit
     const int head = hgrp * kMlaUnitHeads + row_u;
+    constexpr int kQHalfSteps = kMlaKSteps / 2;                        // k-steps of a round
+    constexpr int kQHalfBytes = kQHalfSteps * 32;                      // 576 bytes of a row
+    static_assert(4 * 32 * kQHalfBytes <= 2 * kMlaTileBytes, "the Q staging areas live in key tiles 1 and 2");
     u32x4_t qreg[kMlaQReg];
+    u32x4_t qraw[2][kQHalfSteps];
     {
-        const uint16_t *src = reinterpret_cast<const uint16_t *>(p.q) + (int64_t)b * p.q_stride_b + (int64_t)qi * p.q_stride_s +
-                              (int64_t)min(head, p.nheads - 1) * p.q_stride_h + lh * 8;
+        const uint16_t *src = reinterpret_cast<const uint16_t *>(p.q) + (int64_t)b * p.q_stride_b + (int64_t)qi * p.q_stride_s;
+        const int head0 = hgrp * kMlaUnitHeads + wave * 32;
 #pragma unroll
-        for (int t = 0; t < kMlaQReg; ++t) qreg[t] = load16(src + t * 16);
+        for (int r = 0; r < 2; ++r)
 #pragma unroll
-        for (int t = kMlaQReg; t < kMlaKSteps; ++t) sh.q[wave][t - kMlaQReg][lane] = load16(src + t * 16);   // wave-private
+            for (int i = 0; i < kQHalfSteps; ++i) {
+                const int j = i * 64 + lane;                           // 16-byte piece j of the round: row j / 36
+                const int row = j / (kQHalfBytes / 16);
+                const int c = j - row * (kQHalfBytes / 16);
+                qraw[r][i] = load16(src + (int64_t)min(head0 + row, p.nheads - 1) * p.q_stride_h + r * (kQHalfBytes / 2) + c * 8);
+            }
     }
+    auto stage_q = [&]() {
+        uint8_t *stg = &sh.k[1][0] + wave * (32 * kQHalfBytes);        // tiles 1 and 2 are written from the first step on
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+#pragma unroll
+            for (int i = 0; i < kQHalfSteps; ++i) *reinterpret_cast<u32x4_t *>(stg + (i * 64 + lane) * 16) = qraw[r][i];
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+            for (int t = 0; t < kQHalfSteps; ++t) {
+                const u32x4_t v = *reinterpret_cast<const u32x4_t *>(stg + ln * kQHalfBytes + t * 32 + lh * 16);
+                const int tt = r * kQHalfSteps + t;
+                if (tt < kMlaQReg)
+                    qreg[tt < kMlaQReg ? tt : 0] = v;
+                else
+                    sh.q[wave][tt >= kMlaQReg ? tt - kMlaQReg : 0][lane] = v;   // wave-private
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();   // the area is rewritten by the second round
+        }
+    };
 
     // ---- staging: thread -> (key row tid / 8, eight-code pieces tid % 8 + 8i): one address per chunk serves all
     //      loads and one LDS address all stores.  Rows past the last key of the sequence re-read the last key
@@ -587,6 +622,7 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
         for (int i = 0; i < kMlaRounds; ++i) fetch_piece(i);
         fetch_scales();
         blk_next = blk_second;
+        stage_q();   // q was requested before the chunk: it is here first
 #pragma unroll
         for (int i = 0; i < kMlaRounds; ++i)
 #pragma unroll
