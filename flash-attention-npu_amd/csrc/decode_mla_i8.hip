@@ -206,9 +206,35 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
     const int8_t *kc = reinterpret_cast<const int8_t *>(p.k_cache);
     const int32_t *bt_row = p.block_table + (int64_t)b * p.bt_stride_b;
 
+    // The chunks of a piece are consecutive, so the page of a chunk and its offset inside the page are carried along
+    // from chunk to chunk (page sizes are multiples of the chunk, or the cache is one page): a division and four
+    // 64-bit products per chunk were 90 scalar instructions, and in this loop of one wave per SIMD every instruction
+    // of any kind costs its 4-5 cycles.  Two cursors: fb_* runs ahead and requests table entries, fs_* sets up the
+    // loads.  Both stop at the piece's last chunk (requests past it repeat it).
+    const uint32_t page_size = (uint32_t)p.page_size;
+    uint32_t fb_page = (uint32_t)(c_begin * kChunk) / page_size;
+    uint32_t fb_in = (uint32_t)(c_begin * kChunk) - fb_page * page_size;
+    int fb_left = nch - 1;                                             // chunks the cursor may still advance
+    uint32_t fs_in = fb_in;
+    int fs_last = Lk - 1 - c_begin * kChunk;                           // last key of the sequence, relative to the chunk
+    int fs_left = nch - 1;
+    const int64_t row32_k = (int64_t)kChunk * p.k_stride_row, row32_s = (int64_t)kChunk * p.ks_stride_row;
+    int64_t fs_off_k = (int64_t)fs_in * p.k_stride_row, fs_off_s = (int64_t)fs_in * p.ks_stride_row;
+    auto fetch_blk = [&]() -> int {
+        const int v = bt_row[min(fb_page, (uint32_t)p.max_blocks - 1)];   // clamped and made wave-uniform where it is used, an iteration later: no wait here
+        if (fb_left > 0) {
+            --fb_left;
+            fb_in += kChunk;
+            if (fb_in >= page_size) {
+                fb_in -= page_size;
+                ++fb_page;
+            }
+        }
+        return v;
+    };
     // page ids of the first two chunks: requested first, they come back while Q^T is loaded
-    const int blk_first = bt_row[min((c_begin * kChunk) / p.page_size, p.max_blocks - 1)];
-    const int blk_second = bt_row[min(((c_begin + min(1, nch - 1)) * kChunk) / p.page_size, p.max_blocks - 1)];
+    const int blk_first = fetch_blk();
+    const int blk_second = fetch_blk();
 
     // ---- Q^T operands: lane (ln, lh) holds head 32*wave + ln, dims 16t + 8lh .. +7 of k-step t.  Loaded in that
     //      layout, one instruction would touch 32 rows of q, 32 bytes each (measured: 9 us of the kernel).  The wave's 32
@@ -263,28 +289,34 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
     //      (never memory nobody wrote); they are masked.
     MlaCodes8 st[kMlaRounds];
     float st_ks = 0.f, st_vs = 0.f;
-    auto fetch_blk = [&](int j) -> int {
-        int page = ((c_begin + min(j, nch - 1)) * kChunk) / p.page_size;
-        page = min(page, p.max_blocks - 1);
-        return bt_row[page];   // clamped and made wave-uniform where it is used, an iteration later: no wait here
-    };
     // the loads of a chunk leave piece by piece (fetch_piece), right behind the widening of the piece that held the
     // registers before: they have a whole step to come back
     const int8_t *f_src = nullptr;
     const float *f_ks = nullptr, *f_vs = nullptr;
-    uint32_t f_voff = 0, f_soff = 0;
-    auto fetch_setup = [&](int j_any, int blk_raw) {
+    // per-thread offsets of a chunk that lies wholly inside the sequence; only the sequence's last chunk clamps its rows
+    uint32_t f_voff = (uint32_t)(tid >> 3) * (uint32_t)p.k_stride_row + (tid & 7) * 8;
+    uint32_t f_soff = (uint32_t)(tid & (kChunk - 1)) * (uint32_t)p.ks_stride_row;
+    auto fetch_setup = [&](int blk_raw) {
         const int blk = __builtin_amdgcn_readfirstlane(min(max(blk_raw, 0), p.num_blocks - 1));
-        const int j = min(j_any, nch - 1);
-        const int key0 = (c_begin + j) * kChunk;
-        const int inpage0 = key0 % p.page_size;
-        const int last = Lk - 1 - key0;
-        f_src = kc + (int64_t)blk * p.k_stride_block + (int64_t)inpage0 * p.k_stride_row;
-        f_voff = (uint32_t)min(tid >> 3, last) * (uint32_t)p.k_stride_row + (tid & 7) * 8;
-        const int64_t so = (int64_t)blk * p.ks_stride_block + (int64_t)inpage0 * p.ks_stride_row;
-        f_soff = (uint32_t)min(tid & (kChunk - 1), last) * (uint32_t)p.ks_stride_row;
+        f_src = kc + (int64_t)blk * p.k_stride_block + fs_off_k;
+        const int64_t so = (int64_t)blk * p.ks_stride_block + fs_off_s;
         f_ks = p.k_scale + so;
         f_vs = p.v_scale + so;
+        if (fs_last < kChunk - 1) {   // wave-uniform, the end of the sequence
+            f_voff = (uint32_t)min(tid >> 3, fs_last) * (uint32_t)p.k_stride_row + (tid & 7) * 8;
+            f_soff = (uint32_t)min(tid & (kChunk - 1), fs_last) * (uint32_t)p.ks_stride_row;
+        }
+        if (fs_left > 0) {
+            --fs_left;
+            fs_last -= kChunk;
+            fs_in += kChunk;
+            fs_off_k += row32_k;
+            fs_off_s += row32_s;
+            if (fs_in >= page_size) {   // only with pages that are multiples of the chunk: the next page starts at 0
+                fs_in = 0;
+                fs_off_k = fs_off_s = 0;
+            }
+        }
     };
     auto fetch_piece = [&](int i) { st[i] = *reinterpret_cast<const MlaCodes8 *>(f_src + f_voff + i * 64); };
     auto fetch_scales = [&]() {
@@ -617,7 +649,7 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
     //              softmax of chunk i beside the output products of chunk i-1, one barrier.
     int blk_next;
     {
-        fetch_setup(0, blk_first);
+        fetch_setup(blk_first);
 #pragma unroll
         for (int i = 0; i < kMlaRounds; ++i) fetch_piece(i);
         fetch_scales();
@@ -628,11 +660,11 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
 #pragma unroll
             for (int q = 0; q < 4; ++q) widen_quarter(0, i, q);
         stash_scales(0);
-        fetch_setup(1, blk_next);
+        fetch_setup(blk_next);
 #pragma unroll
         for (int i = 0; i < kMlaRounds; ++i) fetch_piece(i);
         fetch_scales();
-        blk_next = fetch_blk(2);
+        blk_next = fetch_blk();
     }
     __syncthreads();
     int t_cur = 0;   // tile of chunk i
@@ -640,10 +672,10 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
         const int t_nxt = (t_cur == 2) ? 0 : t_cur + 1;
         const int t_prv = (t_cur == 0) ? 2 : t_cur - 1;
         stash_scales(t_nxt);                // chunk i+1 (past the end: the last chunk again, into a tile nobody reads)
-        fetch_setup(i + 2, blk_next);
+        fetch_setup(blk_next);
         fetch_scales();
         scores(t_cur, t_nxt);
-        blk_next = fetch_blk(i + 3);
+        blk_next = fetch_blk();
         mfma_settle();
         __builtin_amdgcn_sched_barrier(0);
         if (i > 0)
