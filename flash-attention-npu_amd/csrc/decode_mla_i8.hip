@@ -409,38 +409,46 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
     auto load_vsi = [&](int tile, int g) { return *reinterpret_cast<const float4 *>(&sh.sc[tile].vsi[4 * lh + 8 * g]); };
     auto load_vsi_hi = [&](int tile, int g) { return *reinterpret_cast<const uint2 *>(&sh.sc[tile].vsi_hi[4 * lh + 8 * g]); };
     auto load_vsi_lo = [&](int tile, int g) { return *reinterpret_cast<const uint2 *>(&sh.sc[tile].vsi_lo[4 * lh + 8 * g]); };
-    // scores in log2 units, in place, and their maximum (registers 4g .. 4g+3)
+    // scores in log2 units RELATIVE TO THE STANDING REFERENCE, in place, and their maximum (registers 4g .. 4g+3): the
+    // subtraction rides in the scaling's fused multiply-add, and the common chunk exponentiates what it finds here
     float xmax = -INFINITY;
     auto softmax_scale4 = [&](int g, const float4 &kq) {
         const float kv[4] = {kq.x, kq.y, kq.z, kq.w};
+        const float m_std = (m_ref == -INFINITY) ? 0.f : m_ref;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
+        for (int e = 0; e < 4; e += 2) {
             const int r = 4 * g + e;
-            float v = s_acc[r] * kv[e];
+            float v0, v1;
             if constexpr (SOFTCAP) {
-                const float e2 = __expf(2.f * v);
-                v = p.softcap_post * (1.f - 2.f / (e2 + 1.f));
+                const float y0 = s_acc[r] * kv[e], y1 = s_acc[r + 1] * kv[e + 1];
+                v0 = p.softcap_post * (1.f - 2.f / (__expf(2.f * y0) + 1.f)) - m_std;
+                v1 = p.softcap_post * (1.f - 2.f / (__expf(2.f * y1) + 1.f)) - m_std;
+            } else {
+                v0 = __builtin_fmaf(s_acc[r], kv[e], -m_std);
+                v1 = __builtin_fmaf(s_acc[r + 1], kv[e + 1], -m_std);
             }
-            s_acc[r] = v;
-            xmax = fmaxf(xmax, v);
+            s_acc[r] = v0;
+            s_acc[r + 1] = v1;
+            xmax = fmaxf(fmaxf(xmax, v0), v1);   // one three-input maximum
         }
     };
     // The common chunk keeps the standing reference.  Anything else (the first chunk: the reference is -inf; a maximum
     // beyond the lazy bound; a chunk with masked keys) goes through here: masks, a moved reference, the rescale
-    // factors for the column owners.  Returns the value the exponentials subtract.
-    auto softmax_check = [&](int j) -> float {
+    // factors for the column owners; the scores are then re-expressed relative to the reference the exponentials use.
+    auto softmax_check = [&](int j) {
         const int pb = j & 1;
         const int key0 = (c_begin + j) * kChunk;
         const bool edge = key0 < mask_lo || key0 + kChunk > mask_hi;   // wave-uniform
         xmax = halves_max(xmax);
-        const bool slow = edge || __any(!(xmax <= m_ref + MlaLazy<T>::kLog2));
+        const bool slow = edge || __any(m_ref == -INFINITY || !(xmax <= MlaLazy<T>::kLog2));
         int moved = 0;
         if (__builtin_expect(slow, 0)) {
+            const float m_std = (m_ref == -INFINITY) ? 0.f : m_ref;
             float mloc = -INFINITY;
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int key = key0 + 8 * (r >> 2) + 4 * lh + (r & 3);
-                s_acc[r] = (key >= mask_lo && key < mask_hi) ? s_acc[r] : -INFINITY;
+                s_acc[r] = (key >= mask_lo && key < mask_hi) ? s_acc[r] + m_std : -INFINITY;   // absolute again
                 mloc = fmaxf(mloc, s_acc[r]);
             }
             mloc = halves_max(mloc);
@@ -452,15 +460,17 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
             l_run *= alpha;
             l_norm *= alpha;
             m_ref = m_new;
+            const float m_use = (m_ref == -INFINITY) ? 0.f : m_ref;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s_acc[r] -= m_use;
         }
         if (lane == 0) sh.moved[pb][wave] = moved;
         xmax = -INFINITY;
-        return (m_ref == -INFINITY) ? 0.f : m_ref;
     };
     // exponentials (registers 4g .. 4g+3)
-    auto softmax_exp4 = [&](int g, float m_use) {
+    auto softmax_exp4 = [&](int g) {
 #pragma unroll
-        for (int e = 0; e < 4; ++e) s_acc[4 * g + e] = fast_exp2(s_acc[4 * g + e] - m_use);
+        for (int e = 0; e < 4; ++e) s_acc[4 * g + e] = fast_exp2(s_acc[4 * g + e]);
     };
     // sums, V-side scale, rounding to the 16-bit type (registers 4g .. 4g+3); the weights really applied are summed
     // with the inverse scales: exactly for fp16, with a two-term bf16 inverse (2^-17 relative) on the dot-product path
@@ -568,7 +578,6 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
             va[1] = read_va(tb0, 1);
         }
         if constexpr (SM) sc0 = load_ksl(tile_sm, 0);
-        float m_use = 0.f;
         // quarter 0: half 0, column tiles 0 and 1; scaled scores and their maximum
         static_for<0, 8>([&](auto slot_) {
             constexpr int slot = decltype(slot_)::value;
@@ -587,7 +596,7 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
             __builtin_amdgcn_sched_barrier(0);
         });
         if constexpr (SM) {
-            m_use = softmax_check(j_sm);
+            softmax_check(j_sm);
             sc1 = load_vs(tile_sm, 0);
             if constexpr (__is_same(T, BF16)) {
                 sh2 = load_vsi_hi(tile_sm, 0);
@@ -607,7 +616,7 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
                 if constexpr (slot == 2) va[0] = read_va(tb1, 0);
                 if constexpr (slot == 4) va[1] = read_va(tb1, 1);
             }
-            if constexpr (SM && (slot & 1)) softmax_exp4(slot >> 1, m_use);
+            if constexpr (SM && (slot & 1)) softmax_exp4(slot >> 1);
             __builtin_amdgcn_sched_barrier(0);
         });
         // quarters 2 and 3: half 1; sums, V-side scale, rounding
