@@ -163,8 +163,9 @@ template <int STRIDE> __device__ __forceinline__ void lds_read8x16(uint32_t addr
         : "memory");
 }
 
+// The small arrays come first: an LDS instruction carries a 16-bit byte offset, so everything below 64 KB is reached as
+// (lane's register + constant); behind the 108 KB of key tiles every access needed an add of its own.
 struct MlaShared {
-    __attribute__((aligned(16))) uint8_t k[3][kMlaTileBytes];   // widened key tiles
     struct __attribute__((aligned(16))) Scales {                 // per-token scales of a tile, side by side: one LDS base address
         float ksl[kChunk];                                       // key-side scale x softmax scale (log2 units)
         float vs[kChunk];                                        // V-side scale
@@ -177,6 +178,7 @@ struct MlaShared {
     __attribute__((aligned(16))) int32_t moved[2][4];                                         // head group moved its reference in this chunk
     float l[kMlaUnitHeads];                                      // final normaliser per head
     __attribute__((aligned(16))) u32x4_t q[4][kMlaQLds][64];     // Q^T operands of the last k-steps: [wave][k-step][lane]
+    __attribute__((aligned(16))) uint8_t k[3][kMlaTileBytes];   // widened key tiles
 };
 
 template <typename T, bool SOFTCAP>
@@ -544,12 +546,19 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
         }
     };
     typedef short v4s_t __attribute__((ext_vector_type(4)));
-    auto read_va = [&](const uint8_t *tile_base, int cc) -> u32x4_t {
+    // LDS addresses that depend on the tile or the parity of the chunk are formed once per step and HELD (made opaque):
+    // left to itself the compiler re-adds the tile's base to the lane's offset in front of every read, and an add
+    // costs this loop as much as any other instruction.
+    auto lds_addr = [](const void *ptr) -> uint32_t {
+        return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void *)ptr;
+    };
+    uint32_t va_addr[2][2];   // V^T operand reads of the output chunk's tile: [second four keys][odd column tile]
+    auto read_va = [&](int half, int cc) -> u32x4_t {
         u32x4_t va;
 #pragma unroll
         for (int jj = 0; jj < 2; ++jj) {
             const v4s_t r4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                (__attribute__((address_space(3))) v4s_t *)(tile_base + tr_off[jj][cc & 1] + (cc >> 1) * 128));
+                (__attribute__((address_space(3))) v4s_t *)(uintptr_t)(va_addr[jj][cc & 1] + half * (16 * kMlaRowBytes) + (cc >> 1) * 128));
             const uint2 r2 = __builtin_bit_cast(uint2, r4);
             va[2 * jj] = r2.x;
             va[2 * jj + 1] = r2.y;
@@ -565,8 +574,17 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
     auto phase_b = [&](auto out_, auto sm_, int j_out, int tile_out, int j_sm, int tile_sm) {
         constexpr bool OUT = decltype(out_)::value, SM = decltype(sm_)::value;
         const int pb = j_out & 1;
-        const uint8_t *tb0 = &sh.k[tile_out][0];
-        const uint8_t *tb1 = tb0 + 16 * kMlaRowBytes;
+        constexpr int tb0 = 0, tb1 = 1;   // the tile's two 16-key halves
+        if constexpr (OUT) {
+            const uint32_t tb = lds_addr(&sh.k[tile_out][0]);
+#pragma unroll
+            for (int jj = 0; jj < 2; ++jj)
+#pragma unroll
+                for (int c1 = 0; c1 < 2; ++c1) {
+                    va_addr[jj][c1] = tb + (uint32_t)tr_off[jj][c1];
+                    asm volatile("" : "+v"(va_addr[jj][c1]));
+                }
+        }
         u32x4_t pkg[4], va[2], vb[2];
         float4 sc0, sc1, sc2;
         uint2 sh2, sl2;
