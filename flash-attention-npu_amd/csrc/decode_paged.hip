@@ -538,43 +538,79 @@ __device__ __forceinline__ void combine_row_block(const DecodeParams &p, int b, 
     const int tid = threadIdx.x;
     const int ns = pcs.ns;
 
-    float mx = -INFINITY;
-    for (int s2 = tid; s2 < ns; s2 += 256) mx = fmaxf(mx, p.lse_partial[pcs.slot(s2) * p.rows + row]);
-#pragma unroll
-    for (int d = 32; d >= 1; d >>= 1) mx = fmaxf(mx, __shfl_xor(mx, d, 64));
-    if ((tid & 63) == 0) s_red[tid >> 6] = mx;
-    __syncthreads();
-    mx = fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
-    const float mx_use = (mx == -INFINITY) ? 0.f : mx;
-
     const int cg = tid % CG;
     const int pl = tid / CG;
+    auto load_row = [&](int64_t srow) -> float4 {
+        if constexpr (partials_are_half(D)) {
+            const uint2 t = *reinterpret_cast<const uint2 *>(reinterpret_cast<const uint16_t *>(p.o_partial) + srow * D + cg * 4);
+            return make_float4(to_float<FP16>((uint16_t)(t.x & 0xffffu)), to_float<FP16>((uint16_t)(t.x >> 16)),
+                               to_float<FP16>((uint16_t)(t.y & 0xffffu)), to_float<FP16>((uint16_t)(t.y >> 16)));
+        } else {
+            return *reinterpret_cast<const float4 *>(p.o_partial + srow * D + cg * 4);
+        }
+    };
+    auto block_max = [&](float mx) -> float {
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) mx = fmaxf(mx, __shfl_xor(mx, d, 64));
+        if ((tid & 63) == 0) s_red[tid >> 6] = mx;
+        __syncthreads();
+        return fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
+    };
     float tot = 0.f;
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
-    // four of the thread's pieces are requested before the first is used (one trip to memory per four)
-    for (int s0 = pl; s0 < ns; s0 += 4 * NPL) {
-        float lw[4];
-        float4 o[4];
+    float mx;
+    constexpr int PL = 8;   // pieces of a thread in flight
+    if (ns <= PL * NPL) {
+        // The pieces were written by other compute units: every dependent load is a trip to memory.  All log-sum-exps
+        // and rows of the unit are requested at once (a thread holds up to PL of each); the maximum is then taken
+        // over what the threads hold, while the rows are still on their way.
+        float lw[PL];
+        float4 o[PL];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int64_t srow = pcs.slot(min(s0 + i * NPL, ns - 1)) * p.rows + row;
-            lw[i] = p.lse_partial[srow];
-            if constexpr (partials_are_half(D)) {
-                const uint2 t = *reinterpret_cast<const uint2 *>(reinterpret_cast<const uint16_t *>(p.o_partial) + srow * D + cg * 4);
-                o[i] = make_float4(to_float<FP16>((uint16_t)(t.x & 0xffffu)), to_float<FP16>((uint16_t)(t.x >> 16)),
-                                   to_float<FP16>((uint16_t)(t.y & 0xffffu)), to_float<FP16>((uint16_t)(t.y >> 16)));
-            } else {
-                o[i] = *reinterpret_cast<const float4 *>(p.o_partial + srow * D + cg * 4);
-            }
+        for (int i = 0; i < PL; ++i) {
+            const int s2 = pl + i * NPL;
+            const int64_t srow = pcs.slot(min(s2, ns - 1)) * p.rows + row;
+            lw[i] = (s2 < ns) ? p.lse_partial[srow] : -INFINITY;
+            o[i] = load_row(srow);
         }
+        mx = -INFINITY;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const float w = (s0 + i * NPL < ns) ? fast_exp2(lw[i] - mx_use) : 0.f;
+        for (int i = 0; i < PL; ++i) mx = fmaxf(mx, lw[i]);
+        mx = block_max(mx);
+        const float mx_use = (mx == -INFINITY) ? 0.f : mx;
+#pragma unroll
+        for (int i = 0; i < PL; ++i) {
+            const float w = fast_exp2(lw[i] - mx_use);   // 0 behind the last piece (-inf)
             tot += w;
             acc[0] += w * o[i].x;
             acc[1] += w * o[i].y;
             acc[2] += w * o[i].z;
             acc[3] += w * o[i].w;
+        }
+    } else {
+        mx = -INFINITY;
+        for (int s2 = tid; s2 < ns; s2 += 256) mx = fmaxf(mx, p.lse_partial[pcs.slot(s2) * p.rows + row]);
+        mx = block_max(mx);
+        const float mx_use = (mx == -INFINITY) ? 0.f : mx;
+        // four of the thread's pieces are requested before the first is used (one trip to memory per four)
+        for (int s0 = pl; s0 < ns; s0 += 4 * NPL) {
+            float lw[4];
+            float4 o[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int64_t srow = pcs.slot(min(s0 + i * NPL, ns - 1)) * p.rows + row;
+                lw[i] = p.lse_partial[srow];
+                o[i] = load_row(srow);
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float w = (s0 + i * NPL < ns) ? fast_exp2(lw[i] - mx_use) : 0.f;
+                tot += w;
+                acc[0] += w * o[i].x;
+                acc[1] += w * o[i].y;
+                acc[2] += w * o[i].z;
+                acc[3] += w * o[i].w;
+            }
         }
     }
     *reinterpret_cast<float4 *>(&s_acc[pl][cg * 4]) = make_float4(acc[0], acc[1], acc[2], acc[3]);
