@@ -52,6 +52,35 @@ def test_mla_basic(hq):
     check_vs_golden(got[0], gold[0], got[1], gold[1], "mla")
 
 
+@pytest.mark.parametrize("page,hq", [(32, 128), (96, 16), (64, 192), (256, 200)])
+def test_mla_page_sizes_and_head_counts(page, hq):
+    """The chunk cursors carry page and in-page offset from chunk to chunk: pages of one chunk, of three, lengths that
+    end inside a chunk and on a page boundary; head counts below, at and above one 128-head unit (the last unit partly
+    empty), whose q rows are fetched row-wise."""
+    case = mla_case(4, hq, [page, 3 * page + 1, 1500, 31], page=page, seed=20 + page)
+    got, ref, gold = run(case)
+    check_out(got[0], ref[0], got[1], ref[1], f"mla page {page} heads {hq}")
+    check_vs_golden(got[0], gold[0], got[1], gold[1], f"mla page {page} heads {hq}")
+
+
+def test_mla_q_with_padded_head_stride():
+    """q as a view whose head stride is not the head dimension (each row still contiguous and 16-byte aligned)."""
+    case = mla_case(2, 128, [1000, 77], seed=31)
+    got_c, ref, gold = run(case)
+    wide = torch.zeros(2, 1, 128, 640, dtype=torch.bfloat16)
+    wide[..., :576] = case["q"]
+    strided = dict(case)
+    strided["q"] = wide[..., :576]                       # stride (128*640, 128*640, 640, 1)
+    assert not strided["q"].is_contiguous()
+    from flash_attn_npu import flash_attn_with_kvcache
+    kc = case["k_cache"].cuda()
+    out, lse = flash_attn_with_kvcache(wide.cuda()[..., :576], kc, kc[..., :512], cache_seqlens=case["cache_seqlens"].cuda(),
+                                       block_table=case["block_table"].cuda(), softmax_scale=192 ** -0.5, causal=True,
+                                       return_softmax_lse=True, k_scale_cache=case["k_scale"].cuda())
+    torch.cuda.synchronize()
+    assert torch.equal(out.cpu(), got_c[0].cpu()) and torch.equal(lse.cpu(), got_c[1].cpu())
+
+
 def test_mla_ragged_and_empty():
     case = mla_case(5, 128, [1, 0, 255, 257, 5000], seed=2, zero_token=True)
     got, ref, gold = run(case)
