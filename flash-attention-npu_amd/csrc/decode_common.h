@@ -311,6 +311,37 @@ __device__ __forceinline__ Partition make_partition(const DecodeParams &p, int *
     return pt;
 }
 
+// Workgroup 0 of a decode launch leaves the partition in the workspace: the merge kernel that follows then finds a
+// unit's pieces from a handful of values it reads in one trip, instead of loading every length and redoing the
+// block-wide prefix pass with its barriers.  Only for batches of one row per prefix segment.
+__device__ __forceinline__ void publish_partition(const DecodeParams &p, const Partition &pt, const int *s_pref) {
+    if (!p.part_hdr || blockIdx.x != 0 || pt.seg != 1) return;
+    for (int t = threadIdx.x; t <= p.batch; t += blockDim.x) p.part_hdr[kPartitionHeaderInts + t] = s_pref[t];
+    if (threadIdx.x == 0) {
+        p.part_hdr[0] = pt.M;
+        p.part_hdr[1] = pt.cost;
+        p.part_hdr[2] = (int32_t)(uint32_t)pt.W;
+        p.part_hdr[3] = (int32_t)((uint64_t)pt.W >> 32);
+        p.part_hdr[4] = (int32_t)(uint32_t)pt.S;
+        p.part_hdr[5] = (int32_t)((uint64_t)pt.S >> 32);
+    }
+}
+__device__ __forceinline__ bool partition_published(const DecodeParams &p) { return p.part_hdr && p.batch <= 256; }
+// the published partition; *pref_b: chunks of the batch rows before b
+__device__ __forceinline__ Partition read_partition(const DecodeParams &p, int b, int *pref_b) {
+    const int32_t *h = p.part_hdr;
+    Partition pt;
+    pt.seg = 1;
+    pt.M = h[0];
+    pt.cost = h[1];
+    pt.W = (int64_t)(((uint64_t)(uint32_t)h[3] << 32) | (uint32_t)h[2]);
+    pt.S = (int64_t)(((uint64_t)(uint32_t)h[5] << 32) | (uint32_t)h[4]);
+    pt.list_heads = p.head_interleave ? 1 : p.nheads_k;
+    pt.any_empty = false;   // not kept: the merge has no use for it
+    *pref_b = h[kPartitionHeaderInts + b];
+    return pt;
+}
+
 // chunks of batch rows before b (one kv head's worth)
 __device__ __forceinline__ int chunks_before(const DecodeParams &p, const Partition &pt, const int *s_pref, int b) {
     const int t = b / pt.seg;
@@ -395,6 +426,7 @@ template <int DV, typename PieceFn>
 __device__ __forceinline__ void balanced_driver(const DecodeParams &p, int worker, PieceFn piece) {
     __shared__ int s_pref[257];
     const Partition pt = make_partition(p, s_pref);
+    publish_partition(p, pt, s_pref);
     walk_share(p, pt, s_pref, worker, piece);
     init_empty_units<DV>(p, pt);
 }

@@ -650,10 +650,17 @@ __global__ void __launch_bounds__(256) splitkv_combine_balanced_kernel(const Dec
     __shared__ int s_pref[257];
     const int kvh = blockIdx.y;
     const int b = blockIdx.z;
-    const Partition pt = make_partition(p, s_pref);
+    Partition pt;
+    int pref_b;
+    if (partition_published(p)) {   // launch-uniform
+        pt = read_partition(p, b, &pref_b);
+    } else {
+        pt = make_partition(p, s_pref);
+        pref_b = chunks_before(p, pt, s_pref, b);
+    }
     const UnitRange ur = unit_range(p, b, pt.M);
     if (ur.nchunks == 0) return;   // the decode kernel initialised this unit
-    const int64_t start = (int64_t)chunks_before(p, pt, s_pref, b) * pt.list_heads +
+    const int64_t start = (int64_t)pref_b * pt.list_heads +
                           (pt.list_heads == 1 ? 0 : (int64_t)kvh * unit_cost(ur.nchunks, pt.cost));
     const UnitPieces pcs = unit_pieces(pt, start, ur.nchunks, kvh, p.nheads_k, pt.cost);
     if (pcs.ns == 1) return;       // written whole by one worker

@@ -446,6 +446,7 @@ __global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) decode_wave_kernel(co
     __shared__ __attribute__((aligned(16))) uint8_t s_k[4][Cfg::kTileBytes];
     __shared__ __attribute__((aligned(16))) uint16_t s_q[4][16 * D];
     const Partition pt = make_partition(p, s_pref);
+    publish_partition(p, pt, s_pref);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     walk_share(p, pt, s_pref, (int64_t)blockIdx.x * 4 + wave,
                [&](int b, int kvh, const UnitRange &ur, int range_lo, int range_hi, bool whole, int64_t slot) {

@@ -27,6 +27,8 @@ struct DecodeParams {
                              // others are computed but neither written nor merged.  NULL: all (balanced wave-level launch only)
     float *o_partial;    // (B, Hk, nsplits, rows, Dv) fp32 (fp16 where partials_are_half(Dv)), each normalised by its own sum
     float *lse_partial;  // (B, Hk, nsplits, rows)     fp32, base-2 log-sum-exp, -inf when empty
+    int32_t *part_hdr;   // balanced mode, batches of at most 256 rows: kPartitionHeaderBytes in which the decode kernel leaves
+                         // its partition for the merge kernel (NULL: the merge kernel recomputes it)
     int32_t batch, seqlen_q, nheads, nheads_k, group, rows;  // rows = seqlen_q * group
     int32_t headdim;     // columns of an output row (and of a q / k / v row, except for the latent cache): a multiple of 8;
                          // the kernels' compile-time width is tile_headdim() of it and the partials are that wide
@@ -159,6 +161,11 @@ struct PrefillParams {
 // of the final rounding), and halving them halves what the split costs in writes and in the merge's reads.  Their
 // writer clamps to the fp16 range.  Every other width keeps fp32 partials.
 constexpr bool partials_are_half(int dv) { return dv == 512; }
+
+// Balanced mode: the partition of a launch (share size, list length, prefix of the rows' chunk counts) as the decode
+// kernel computed it, left behind the partials for the merge kernel.
+constexpr int kPartitionHeaderInts = 8;                 // M, cost, W (2), S (2), 2 spare; then prefix[0 .. batch]
+constexpr size_t kPartitionHeaderBytes = 2048;          // 8 + 257 ints, rounded up
 
 
 // Width the kernels are compiled for, for a head dimension of d columns.

@@ -345,7 +345,8 @@ int fa_rocm_plan_kvcache(const fa_kvcache_args *a, int num_cus, fa_split_plan *p
         if (wave_workers) plan->min_share = 2;   // short shares: the pipeline fill dominates tiny contexts otherwise
         if (env().min_share > 0) plan->min_share = env().min_share;
         // every worker writes at most two partials (the units cut at the two ends of its share)
-        plan->workspace_bytes = (size_t)plan->num_workers * 2 * slot_bytes;
+        // ... and workgroup 0 leaves the partition behind them for the merge kernel
+        plan->workspace_bytes = (size_t)plan->num_workers * 2 * slot_bytes + fa::kPartitionHeaderBytes;
         return FA_OK;
     }
     const int64_t bound = live_keys_bound(a);
@@ -666,7 +667,9 @@ static int fwd_kvcache_impl(const fa_kvcache_args *a, void *stream_, void *const
                         !env().no_head_interleave;
     const bool needs_combine = need > 0;
     if (needs_combine) {
-        const size_t slot_rows = need / partial_row_bytes(a);
+        const size_t hdr = p.balanced ? fa::kPartitionHeaderBytes : 0;
+        const size_t slot_rows = (need - hdr) / partial_row_bytes(a);
+        if (p.balanced) p.part_hdr = reinterpret_cast<int32_t *>(static_cast<char *>(a->workspace) + need - hdr);
         p.o_partial = static_cast<float *>(a->workspace);
         p.lse_partial = reinterpret_cast<float *>(static_cast<char *>(a->workspace) + slot_rows * (partial_row_bytes(a) - sizeof(float)));
     }

@@ -133,10 +133,10 @@ def test_split_plan_invariants():
     assert plan.mode == 1 and plan.num_wgs == 512                      # balanced: two workgroups per CU
     assert plan.num_workers == 2048 and plan.min_share == 2            # one 16-row tile: every wave is a worker
     rows = 4
-    assert plan.workspace_bytes == 2048 * 2 * rows * (128 + 1) * 4 == lib.fa_rocm_kvcache_workspace_bytes(C.byref(a), 256)
+    assert plan.workspace_bytes == 2048 * 2 * rows * (128 + 1) * 4 + 2048 == lib.fa_rocm_kvcache_workspace_bytes(C.byref(a), 256)
     a.seqlen_q = 5                                                      # 20 rows: two tiles, the workgroup is the worker
     lib.fa_rocm_plan_kvcache(C.byref(a), 256, C.byref(plan))
-    assert plan.num_workers == plan.num_wgs == 512 and plan.workspace_bytes == 512 * 2 * 20 * 129 * 4
+    assert plan.num_workers == plan.num_wgs == 512 and plan.workspace_bytes == 512 * 2 * 20 * 129 * 4 + 2048
     a.seqlen_q = 1
     a.num_splits = 1
     lib.fa_rocm_plan_kvcache(C.byref(a), 256, C.byref(plan))

@@ -161,4 +161,4 @@ def test_abi_rejects_rows_that_are_not_16_byte_pieces():
     assert _lib.load().fa_rocm_kvcache_validate(C.byref(a)) == 0, _lib.last_error()
     plan = _lib.SplitPlan()
     _lib.load().fa_rocm_plan_kvcache(C.byref(a), 256, C.byref(plan))
-    assert plan.workspace_bytes == 2048 * 2 * 4 * (128 + 1) * 4       # partial rows are as wide as the compiled kernel
+    assert plan.workspace_bytes == 2048 * 2 * 4 * (128 + 1) * 4 + 2048   # partial rows are as wide as the compiled kernel; + the partition header
