@@ -307,7 +307,8 @@ __device__ __forceinline__ Partition make_partition(const DecodeParams &p, int *
         __syncthreads();
     }
     pt.W = (int64_t)s_pref[256] * pt.list_heads;
-    pt.S = max((pt.W + shares - 1) / shares, (int64_t)max(p.min_share, 1));
+    const bool long_units = p.min_share_long > 0 && (int64_t)s_pref[256] >= (int64_t)kLongUnitChunks * max(s_cnt[256], 1) + (int64_t)pt.cost * s_cnt[256];
+    pt.S = max((pt.W + shares - 1) / shares, (int64_t)max(long_units ? p.min_share_long : p.min_share, 1));
     return pt;
 }
 

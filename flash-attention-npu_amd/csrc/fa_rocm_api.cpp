@@ -656,6 +656,7 @@ static int fwd_kvcache_impl(const fa_kvcache_args *a, void *stream_, void *const
     p.num_workers = plan.num_workers;
     p.min_share = plan.min_share;
     p.wave_workers = plan.num_workers != plan.num_wgs;
+    p.min_share_long = (p.wave_workers && env().min_share <= 0) ? 4 : 0;
     // wave workers of neighbouring kv heads walk the same token range together
     // Fixed cost of starting on a unit, in chunk times.  Latent kernel: ~15 us of q staging and pipeline
     // fill against ~2 us per chunk; charging 7 chunks takes the workgroups that start a second unit off
