@@ -116,11 +116,14 @@ template <typename T, int BASE> __device__ __forceinline__ void acc_mfma(const u
                          : MLA_ALL_ACC);
     }
 }
-template <int R> __device__ __forceinline__ void acc_zero() {
-    if constexpr (R < 10)
-        asm volatile("v_accvgpr_write_b32 a%0, 0" ::"n"(R) : MLA_ALL_ACC);
+// a[BASE : BASE+15] = 0 (z must hold zeros)
+template <typename T, int BASE> __device__ __forceinline__ void acc_mfma_zero(const u32x4_t &z) {
+    if constexpr (BASE == 0)
+        asm volatile("v_mfma_f32_32x32x16_bf16 a[0:15], %0, %0, 0" ::"v"(z) : MLA_ALL_ACC);
     else
-        asm volatile("v_accvgpr_write_b32 a%0%1, 0" ::"n"(R / 10), "n"(R % 10) : MLA_ALL_ACC);
+        asm volatile("v_mfma_f32_32x32x16_bf16 a[%1%2:%3%4], %0, %0, 0" ::"v"(z), "n"(BASE / 10), "n"(BASE % 10),
+                     "n"((BASE + 15) / 10), "n"((BASE + 15) % 10)
+                     : MLA_ALL_ACC);
 }
 template <int R> __device__ __forceinline__ float acc_read() {
     float v;
@@ -240,49 +243,59 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
 
     // ---- Q^T operands: lane (ln, lh) holds head 32*wave + ln, dims 16t + 8lh .. +7 of k-step t.  Loaded in that
     //      layout, one instruction would touch 32 rows of q, 32 bytes each (measured: 9 us of the kernel).  The wave's 32
-    //      rows are fetched as they lie instead - half a row (576 bytes = 36 lanes) after the other, two rounds of 18
-    //      instructions, all requested here - and turned into the operand layout through a staging area of the wave's
-    //      own (stage_q below, once the first chunk's loads are out as well).
+    //      rows are fetched as they lie instead - a third of a row (384 bytes = 24 lanes) after the other, three rounds
+    //      of 12 instructions, all requested here - and turned into the operand layout through a staging area of the
+    //      wave's own (stage_q below, once the first chunk's loads are out as well).
     const int row_u = wave * 32 + ln;                                  // row of the unit
     const int head = hgrp * kMlaUnitHeads + row_u;
-    constexpr int kQHalfSteps = kMlaKSteps / 2;                        // k-steps of a round
-    constexpr int kQHalfBytes = kQHalfSteps * 32;                      // 576 bytes of a row
-    static_assert(4 * 32 * kQHalfBytes <= 2 * kMlaTileBytes, "the Q staging areas live in key tiles 1 and 2");
+    constexpr int kQRounds = 3;
+    constexpr int kQRoundSteps = kMlaKSteps / kQRounds;                // k-steps of a round
+    constexpr int kQRoundBytes = kQRoundSteps * 32;                    // 384 bytes of a row
+    constexpr int kQRowPieces = kQRoundBytes / 16;
+    // staged rows lie 100 words apart: the 16 lanes the LDS serves per cycle, 4 banks each, then tile all 64 banks.
+    // Unpadded, the reads of the operand layout were 4-way bank conflicts, and staging q cost the LDS 6 us per piece.
+    constexpr int kQStageRow = kQRoundBytes + 16;
+    static_assert(kQRounds * kQRoundSteps == kMlaKSteps && kQRoundSteps * 64 == 32 * kQRowPieces, "rounds tile q");
+    static_assert(4 * 32 * kQStageRow <= 2 * kMlaTileBytes, "the Q staging areas live in key tiles 1 and 2");
     u32x4_t qreg[kMlaQReg];
-    u32x4_t qraw[2][kQHalfSteps];
+    u32x4_t qraw[kQRounds][kQRoundSteps];
     {
         const uint16_t *src = reinterpret_cast<const uint16_t *>(p.q) + (int64_t)b * p.q_stride_b + (int64_t)qi * p.q_stride_s;
         const int head0 = hgrp * kMlaUnitHeads + wave * 32;
 #pragma unroll
-        for (int r = 0; r < 2; ++r)
+        for (int r = 0; r < kQRounds; ++r)
 #pragma unroll
-            for (int i = 0; i < kQHalfSteps; ++i) {
-                const int j = i * 64 + lane;                           // 16-byte piece j of the round: row j / 36
-                const int row = j / (kQHalfBytes / 16);
-                const int c = j - row * (kQHalfBytes / 16);
-                qraw[r][i] = load16(src + (int64_t)min(head0 + row, p.nheads - 1) * p.q_stride_h + r * (kQHalfBytes / 2) + c * 8);
+            for (int i = 0; i < kQRoundSteps; ++i) {
+                const int j = i * 64 + lane;                           // 16-byte piece j of the round: row j / 24
+                const int row = j / kQRowPieces;
+                const int c = j - row * kQRowPieces;
+                qraw[r][i] = load16(src + (int64_t)min(head0 + row, p.nheads - 1) * p.q_stride_h + r * (kQRoundBytes / 2) + c * 8);
             }
     }
     auto stage_q = [&]() {
-        uint8_t *stg = &sh.k[1][0] + wave * (32 * kQHalfBytes);        // tiles 1 and 2 are written from the first step on
+        uint8_t *stg = &sh.k[1][0] + wave * (32 * kQStageRow);         // tiles 1 and 2 are written from the first step on
 #pragma unroll
-        for (int r = 0; r < 2; ++r) {
+        for (int r = 0; r < kQRounds; ++r) {
 #pragma unroll
-            for (int i = 0; i < kQHalfSteps; ++i) *reinterpret_cast<u32x4_t *>(stg + (i * 64 + lane) * 16) = qraw[r][i];
+            for (int i = 0; i < kQRoundSteps; ++i) {
+                const int j = i * 64 + lane;
+                const int row = j / kQRowPieces;
+                *reinterpret_cast<u32x4_t *>(stg + row * kQStageRow + (j - row * kQRowPieces) * 16) = qraw[r][i];
+            }
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
             __builtin_amdgcn_wave_barrier();
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
-            for (int t = 0; t < kQHalfSteps; ++t) {
-                const u32x4_t v = *reinterpret_cast<const u32x4_t *>(stg + ln * kQHalfBytes + t * 32 + lh * 16);
-                const int tt = r * kQHalfSteps + t;
+            for (int t = 0; t < kQRoundSteps; ++t) {
+                const u32x4_t v = *reinterpret_cast<const u32x4_t *>(stg + ln * kQStageRow + t * 32 + lh * 16);
+                const int tt = r * kQRoundSteps + t;
                 if (tt < kMlaQReg)
                     qreg[tt < kMlaQReg ? tt : 0] = v;
                 else
                     sh.q[wave][tt >= kMlaQReg ? tt - kMlaQReg : 0][lane] = v;   // wave-private
             }
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();   // the area is rewritten by the second round
+            __builtin_amdgcn_wave_barrier();   // the area is rewritten by the next round
         }
     };
 
@@ -510,7 +523,11 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
     //      The V^T operand comes from two transposing reads: in a 16-lane group, lane s points at 4 columns
     //      (4*(s%4)..) of key row s/4 and receives column s of the group's 16 for its 4 key rows.
     // accumulator tile (cc, hg) = a[16 * (4*cc + hg) .. +15]
-    static_for<0, 256>([&](auto r) { acc_zero<decltype(r)::value>(); });
+    // zeroed sixteen registers at a time: a product of zero operands with a zero addend
+    {
+        const u32x4_t z = {0u, 0u, 0u, 0u};
+        static_for<0, 16>([&](auto t_) { acc_mfma_zero<T, 16 * decltype(t_)::value>(z); });
+    }
     int tr_off[2][2];   // [second four keys][odd column tile]
     {
         const int g16 = lane >> 4, s16 = lane & 15;
