@@ -21,8 +21,11 @@
 //   staging all four waves: the loads of chunk c+2 leave (global -> registers) piece by piece while chunk c+1 is
 //           widened into LDS beside the score products of chunk c, and the softmax of chunk c stands beside the
 //           output products of chunk c-1; one workgroup barrier per chunk, three LDS tiles.
-// Measured on this machine, vector and matrix instructions of one wave overlap little (a step costs about the sum
-// of the two), so what counts is the instruction count: per chunk and wave 68 MFMAs, ~300 vector instructions.
+// Measured on this machine, a wave that is alone on its SIMD issues one instruction per turn whatever its kind, and
+// its matrix instructions overlap little with the rest: a chunk costs its 68 MFMAs plus 4-5 cycles for EVERY other
+// instruction (vector, scalar, LDS, wait: ~540 of them), so what counts is the instruction count of the loop.
+// Split units leave fp16 partial rows (partials_are_half), and neighbouring shares are dealt to one XCD (their q
+// rows meet in one L2).
 //
 // The exponent reference of a head moves only when a chunk's maximum passes it by more than kLazy (the lazy rescale of
 // the reference's fourth-generation kernels, csrc/ascend910/flash_attn_npu_4/online_softmax.hpp:633-666): rescaling
