@@ -30,30 +30,40 @@ int dtype_code(const at::Tensor &t) {
     }
 }
 
+// Every tensor of a call lives on one ROCm device: the kernels dereference all of them from the same launch.
 void require_device(std::initializer_list<const at::Tensor *> tensors) {
-    for (const at::Tensor *t : tensors)
-        TORCH_CHECK(t == nullptr || !t->defined() || t->is_cuda(),
-                    "flash_attn_npu (MI355X build) needs tensors on a ROCm device; there is no CPU path");
+    const at::Tensor *first = nullptr;
+    for (const at::Tensor *t : tensors) {
+        if (t == nullptr || !t->defined()) continue;
+        TORCH_CHECK(t->is_cuda(), "flash_attn_npu (MI355X build) needs tensors on a ROCm device; there is no CPU path");
+        if (first == nullptr) first = t;
+        TORCH_CHECK(t->device() == first->device(), "all tensors of a call must be on the same device");
+    }
 }
 
 const at::Tensor *ptr_of(const OptTensor &t) { return t.has_value() ? &t.value() : nullptr; }
 
 void check_rc(int rc) { TORCH_CHECK(rc == FA_OK, fa_rocm_last_error()); }
 
-// Small constant tensors, one per (kind, device, shape), never evicted: a captured HIP graph may hold their addresses
-// long after the call that made them.
+// Small constant tensors for dense caches called without a table or lengths, one per (kind, device, shape).  The
+// first kCachedTables distinct shapes are kept for the life of the process, so a captured HIP graph may hold their
+// addresses; past that bound a call gets a fresh tensor of its own, which lives as long as the caller's results do
+// (callers that capture such calls pass cache_seqlens / block_table themselves).
+constexpr size_t kCachedTables = 256;
 at::Tensor cached_table(int kind, const at::Device &dev, int64_t batch, int64_t value) {
     static std::mutex mu;
     static std::map<std::tuple<int, int, int64_t, int64_t>, at::Tensor> cache;
+    const auto opts = at::TensorOptions().dtype(at::kInt).device(dev);
+    const auto make = [&]() {
+        return kind == 0 ? at::arange(batch, opts).view({batch, 1})   // identity block table of a dense cache
+                         : at::full({batch}, value, opts);            // every row holds `value` keys
+    };
     std::lock_guard<std::mutex> lock(mu);
     const auto key = std::make_tuple(kind, (int)dev.index(), batch, value);
     auto it = cache.find(key);
     if (it != cache.end()) return it->second;
-    const auto opts = at::TensorOptions().dtype(at::kInt).device(dev);
-    at::Tensor t = kind == 0 ? at::arange(batch, opts).view({batch, 1})   // identity block table of a dense cache
-                             : at::full({batch}, value, opts);            // every row holds `value` keys
-    cache.emplace(key, t);
-    return t;
+    if (cache.size() >= kCachedTables) return make();
+    return cache.emplace(key, make()).first->second;
 }
 
 // mha_fwd_kvcache (flash_api.cpp:356-637).  Returns {out, softmax_lse}.
@@ -102,12 +112,14 @@ std::vector<at::Tensor> fwd_kvcache(const at::Tensor &q, const at::Tensor &kcach
         block_table = block_table_.value();
     }
     TORCH_CHECK(block_table.scalar_type() == at::kInt, "block_table must have dtype int32");
+    TORCH_CHECK(block_table.dim() == 2, "block_table must be (batch_size, max_num_blocks_per_seq)");
     TORCH_CHECK(block_table.stride(-1) == 1, "block_table must have contiguous last dimension");
     if (!seqlens_k.defined()) {
         TORCH_CHECK(seqlens_k_.has_value(), "cache_seqlens must be given with a paged KV cache");
         seqlens_k = seqlens_k_.value();
     }
     TORCH_CHECK(seqlens_k.scalar_type() == at::kInt, "seqlens_k must have dtype int32");
+    TORCH_CHECK(seqlens_k.dim() == 1, "seqlens_k must be (batch_size,)");
     TORCH_CHECK(!alibi_slopes_.has_value(), "NPU FlashAttention does not support alibi_slopes");
     TORCH_CHECK(!leftpad_k_.has_value(), "NPU FlashAttention does not support leftpad_k");
     TORCH_CHECK(softcap >= 0.0, "softcap must be non-negative (0.0 disables softcap)");
@@ -115,15 +127,30 @@ std::vector<at::Tensor> fwd_kvcache(const at::Tensor &q, const at::Tensor &kcach
     // tables would be silently unused
     TORCH_CHECK(k_.has_value() || v_.has_value() || (!rotary_cos_.has_value() && !rotary_sin_.has_value()),
                 "rotary_cos / rotary_sin are only applied together with new k / v");
-    require_device({&q, &kcache, &vcache, ptr_of(k_), ptr_of(v_), &seqlens_k, &block_table, ptr_of(rotary_cos_), ptr_of(rotary_sin_)});
 
     const int64_t B = q.size(0), sq = q.size(1), hq = q.size(2), d = q.size(3);
     const int64_t num_blocks = kcache.size(0), page = kcache.size(1), hk = kcache.size(2), dk = kcache.size(3);
     const int64_t dv = vcache.size(3);
     TORCH_CHECK(B > 0, "batch size must be positive");
     TORCH_CHECK(d == dk, "q and kcache must have the same head dimension");
+    // the kernels index both caches (and the scale caches) with the page ids, rows and heads of kcache
+    TORCH_CHECK(vcache.size(0) == num_blocks && vcache.size(1) == page && vcache.size(2) == hk,
+                "vcache must have the num_blocks, page_block_size and nheads_k of kcache");
     TORCH_CHECK(hq % hk == 0, "Number of heads in key/value must divide number of heads in query");
     TORCH_CHECK(block_table.size(0) == B && seqlens_k.size(0) == B, "block_table / cache_seqlens batch mismatch");
+    if (k_scale_cache_.has_value()) {
+        const at::Tensor &ks = k_scale_cache_.value();
+        TORCH_CHECK(ks.scalar_type() == at::kFloat && ks.dim() == 3 && ks.stride(-1) == 1 && ks.size(0) == num_blocks &&
+                        ks.size(1) == page && ks.size(2) == hk,
+                    "k_scale_cache must be fp32 (num_blocks, page_block_size, nheads_k)");
+        if (v_scale_cache_.has_value()) {
+            const at::Tensor &vs = v_scale_cache_.value();
+            TORCH_CHECK(vs.scalar_type() == at::kFloat && vs.sizes() == ks.sizes() && vs.strides() == ks.strides(),
+                        "v_scale_cache must match k_scale_cache's layout");
+        }
+    }
+    require_device({&q, &kcache, &vcache, ptr_of(k_), ptr_of(v_), &seqlens_k, &block_table, ptr_of(rotary_cos_), ptr_of(rotary_sin_),
+                    ptr_of(out_), ptr_of(k_scale_cache_), ptr_of(v_scale_cache_)});
     seqlens_k = seqlens_k.contiguous();
 
     const c10::hip::HIPGuardMasqueradingAsCUDA guard(q.device());
@@ -156,16 +183,9 @@ std::vector<at::Tensor> fwd_kvcache(const at::Tensor &q, const at::Tensor &kcach
     a.bt_stride_b = block_table.stride(0);
     if (k_scale_cache_.has_value()) {
         const at::Tensor &ks = k_scale_cache_.value();
-        TORCH_CHECK(ks.scalar_type() == at::kFloat && ks.dim() == 3 && ks.stride(-1) == 1 && ks.is_cuda(),
-                    "k_scale_cache must be fp32 (num_blocks, page_block_size, nheads_k)");
         a.k_scale_cache = ks.data_ptr<float>();
         a.ks_stride_block = ks.stride(0), a.ks_stride_row = ks.stride(1);
-        if (v_scale_cache_.has_value()) {
-            const at::Tensor &vs = v_scale_cache_.value();
-            TORCH_CHECK(vs.scalar_type() == at::kFloat && vs.strides() == ks.strides() && vs.is_cuda(),
-                        "v_scale_cache must match k_scale_cache's layout");
-            a.v_scale_cache = vs.data_ptr<float>();
-        }
+        if (v_scale_cache_.has_value()) a.v_scale_cache = v_scale_cache_->data_ptr<float>();
     }
     at::Tensor k, v, rc, rs;   // kept alive until the call is enqueued
     if (k_.has_value() || v_.has_value()) {
@@ -219,15 +239,18 @@ std::vector<at::Tensor> fwd_kvcache(const at::Tensor &q, const at::Tensor &kcach
     return {out, lse};
 }
 
-// mha_varlen_fwd (flash_api.cpp:848-1089).  Returns {out, softmax_lse (Hq, total_q), p, rng_state}.  num_splits (paged
-// K/V only; not an argument of the reference's function): 0 cuts every sequence's keys into as many ranges as it
-// takes to fill the device when the query tiles alone cannot, 1 never, n at most n.
+// mha_varlen_fwd (flash_api.cpp:848-1089), its 21 arguments in its order: the last of them is the random generator
+// (flash_api.cpp:868; unused without dropout, callers pass None).  Returns {out, softmax_lse (Hq, total_q), p,
+// rng_state}.  num_splits is a trailing extra with a default (paged K/V only; not an argument of the reference's
+// function): 0 cuts every sequence's keys into as many ranges as it takes to fill the device when the query tiles
+// alone cannot, 1 never, n at most n.
 std::vector<at::Tensor> varlen_fwd(const at::Tensor &q, const at::Tensor &k, const at::Tensor &v, const OptTensor &out_,
                                    const at::Tensor &cu_seqlens_q, const OptTensor &cu_seqlens_k, const OptTensor &seqused_k_,
                                    const OptTensor &leftpad_k_, const OptTensor &block_table_, const OptTensor &alibi_slopes_,
                                    int64_t max_seqlen_q, int64_t max_seqlen_k, double p_dropout, double softmax_scale, bool zero_tensors,
                                    bool is_causal, int64_t window_size_left, int64_t window_size_right, double softcap,
-                                   bool return_softmax, int64_t num_splits) {
+                                   bool return_softmax, const std::optional<at::Generator> &gen_, int64_t num_splits) {
+    (void)gen_;
     TORCH_CHECK(q.scalar_type() == at::kBFloat16 || q.scalar_type() == at::kHalf,
                 "FlashAttention only supports FP16 and BF16 data types");
     TORCH_CHECK(k.scalar_type() == q.scalar_type(), "query and key must have the same dtype");
@@ -246,11 +269,9 @@ std::vector<at::Tensor> varlen_fwd(const at::Tensor &q, const at::Tensor &k, con
     // flash_api.cpp:886 rejects seqused_k always; here it is the length array of paged K/V and has no meaning for
     // packed keys, whose lengths are the differences of cu_seqlens_k
     TORCH_CHECK(paged || !seqused_k_.has_value(), "NPU FlashAttention does not support seqused_k.");
-    require_device({&q, &k, &v, &cu_seqlens_q, ptr_of(cu_seqlens_k), ptr_of(seqused_k_), ptr_of(block_table_)});
     const int64_t total_q = q.size(0), hq = q.size(1), d = q.size(2);
     const int64_t B = cu_seqlens_q.numel() - 1;
     TORCH_CHECK(B > 0, "batch size must be positive");
-    const c10::hip::HIPGuardMasqueradingAsCUDA guard(q.device());
 
     fa_varlen_args a = {};
     at::Tensor seqused_k, cu_k;
@@ -258,8 +279,11 @@ std::vector<at::Tensor> varlen_fwd(const at::Tensor &q, const at::Tensor &k, con
     if (paged) {
         const at::Tensor &bt = block_table_.value();
         TORCH_CHECK(bt.scalar_type() == at::kInt, "block_table must have dtype int32");
+        TORCH_CHECK(bt.dim() == 2 && bt.size(0) == B, "block_table must be (batch_size, max_num_blocks_per_seq)");
         TORCH_CHECK(bt.stride(-1) == 1, "block_table must have contiguous last dimension");
         TORCH_CHECK(k.dim() == 4 && v.dim() == 4, "paged k / v must be (num_blocks, page_block_size, nheads_k, headdim)");
+        TORCH_CHECK(v.size(0) == k.size(0) && v.size(1) == k.size(1) && v.size(2) == k.size(2),
+                    "paged v must have the num_blocks, page_block_size and nheads_k of k");
         if (seqused_k_.has_value()) {
             seqused_k = seqused_k_.value();
         } else {
@@ -267,6 +291,7 @@ std::vector<at::Tensor> varlen_fwd(const at::Tensor &q, const at::Tensor &k, con
             seqused_k = (cu_seqlens_k->slice(0, 1) - cu_seqlens_k->slice(0, 0, -1)).to(at::kInt);
         }
         TORCH_CHECK(seqused_k.scalar_type() == at::kInt, "seqused_k must have dtype int32");
+        TORCH_CHECK(seqused_k.dim() == 1 && seqused_k.size(0) == B, "seqused_k must be (batch_size,)");
         seqused_k = seqused_k.contiguous();
         hk = k.size(2);
         a.page_size = (int32_t)k.size(1), a.max_blocks_per_seq = (int32_t)bt.size(1), a.num_blocks = (int32_t)k.size(0);
@@ -276,6 +301,8 @@ std::vector<at::Tensor> varlen_fwd(const at::Tensor &q, const at::Tensor &k, con
     } else {
         TORCH_CHECK(cu_seqlens_k.has_value() && cu_seqlens_k->scalar_type() == at::kInt, "cu_seqlens_k must have dtype int32");
         TORCH_CHECK(k.dim() == 3 && v.dim() == 3, "k / v must be (total_k, nheads_k, headdim)");
+        TORCH_CHECK(v.size(0) == k.size(0) && v.size(1) == k.size(1), "v must have the total_k and nheads_k of k");
+        TORCH_CHECK(cu_seqlens_k->numel() == B + 1, "cu_seqlens_k must have batch_size + 1 entries");
         hk = k.size(1);
         a.k_stride_t = k.stride(0), a.k_stride_h = k.stride(1);
         a.v_stride_t = v.stride(0), a.v_stride_h = v.stride(1);
@@ -283,6 +310,8 @@ std::vector<at::Tensor> varlen_fwd(const at::Tensor &q, const at::Tensor &k, con
     TORCH_CHECK(k.size(-1) == d && v.size(-1) == d, "q, k and v must have the same head dimension");
     TORCH_CHECK(d <= 256, "FlashAttention only supports head dimension at most 256");
     TORCH_CHECK(hq % hk == 0, "Number of heads in key/value must divide number of heads in query");
+    require_device({&q, &k, &v, &cu_seqlens_q, ptr_of(cu_seqlens_k), ptr_of(seqused_k_), ptr_of(block_table_), ptr_of(out_)});
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(q.device());
     const at::Tensor cu_q = cu_seqlens_q.contiguous();
     if (cu_seqlens_k.has_value()) cu_k = cu_seqlens_k->contiguous();
     at::Tensor out;
@@ -324,7 +353,18 @@ std::vector<at::Tensor> varlen_fwd(const at::Tensor &q, const at::Tensor &k, con
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.doc() = "flash_attn_npu on MI355X: operator layer over libfa_rocm.so";
-    m.def("fwd_kvcache", &fwd_kvcache, "Forward pass, with KV-cache (paged, optional in-place append)");
-    m.def("varlen_fwd", &varlen_fwd, "Forward pass (variable length)");
+    namespace py = pybind11;
+    // the reference's 20 arguments (flash_api.cpp:356-377), then the scale caches of an int8 cache as optional extras
+    m.def("fwd_kvcache", &fwd_kvcache, "Forward pass, with KV-cache (paged, optional in-place append)", py::arg("q"), py::arg("kcache"),
+          py::arg("vcache"), py::arg("k"), py::arg("v"), py::arg("seqlens_k"), py::arg("rotary_cos"), py::arg("rotary_sin"),
+          py::arg("cache_batch_idx"), py::arg("leftpad_k"), py::arg("block_table"), py::arg("alibi_slopes"), py::arg("out"),
+          py::arg("softmax_scale"), py::arg("is_causal"), py::arg("window_size_left"), py::arg("window_size_right"), py::arg("softcap"),
+          py::arg("is_rotary_interleaved"), py::arg("num_splits"), py::arg("k_scale_cache") = py::none(),
+          py::arg("v_scale_cache") = py::none());
+    m.def("varlen_fwd", &varlen_fwd, "Forward pass (variable length)", py::arg("q"), py::arg("k"), py::arg("v"), py::arg("out"),
+          py::arg("cu_seqlens_q"), py::arg("cu_seqlens_k"), py::arg("seqused_k"), py::arg("leftpad_k"), py::arg("block_table"),
+          py::arg("alibi_slopes"), py::arg("max_seqlen_q"), py::arg("max_seqlen_k"), py::arg("p_dropout"), py::arg("softmax_scale"),
+          py::arg("zero_tensors"), py::arg("is_causal"), py::arg("window_size_left"), py::arg("window_size_right"), py::arg("softcap"),
+          py::arg("return_softmax"), py::arg("gen") = py::none(), py::arg("num_splits") = 0);
     m.def("abi_version", []() { return fa_rocm_abi_version(); });
 }

@@ -197,9 +197,11 @@ def bind_kvcache(q, kcache, vcache, k_, v_, seqlens_k_, rotary_cos_, rotary_sin_
     else:
         _require(cache_batch_idx_ is None, "Paged KVcache does not support cache_batch_idx")
     _require(block_table_.dtype == torch.int32, "block_table must have dtype int32")
+    _require(block_table_.dim() == 2, "block_table must be (batch_size, max_num_blocks_per_seq)")
     _require(block_table_.stride(-1) == 1, "block_table must have contiguous last dimension")
     _require(seqlens_k_ is not None, "cache_seqlens must be given with a paged KV cache")
     _require(seqlens_k_.dtype == torch.int32, "seqlens_k must have dtype int32")
+    _require(seqlens_k_.dim() == 1, "seqlens_k must be (batch_size,)")
     _require(alibi_slopes_ is None, "NPU FlashAttention does not support alibi_slopes")
     _require(leftpad_k_ is None, "NPU FlashAttention does not support leftpad_k")
     _require(softcap >= 0.0, "softcap must be non-negative (0.0 disables softcap)")
@@ -215,6 +217,8 @@ def bind_kvcache(q, kcache, vcache, k_, v_, seqlens_k_, rotary_cos_, rotary_sin_
     dv = vcache.shape[-1]
     _require(B > 0, "batch size must be positive")
     _require(d == dk, "q and kcache must have the same head dimension")
+    _require(tuple(vcache.shape[:3]) == (num_blocks, page, hk),
+             "vcache must have the num_blocks, page_block_size and nheads_k of kcache")
     _require(hq % hk == 0, "Number of heads in key/value must divide number of heads in query")
     _require(block_table_.shape[0] == B and seqlens_k_.shape[0] == B, "block_table / cache_seqlens batch mismatch")
     seqlens_k = seqlens_k_.contiguous()
@@ -241,11 +245,13 @@ def bind_kvcache(q, kcache, vcache, k_, v_, seqlens_k_, rotary_cos_, rotary_sin_
     a.v_stride_block, a.v_stride_row, a.v_stride_h = vcache.stride(0), vcache.stride(1), vcache.stride(2)
     a.bt_stride_b = block_table_.stride(0)
     if k_scale_cache_ is not None:
-        _require(k_scale_cache_.dtype == torch.float32 and k_scale_cache_.dim() == 3 and k_scale_cache_.stride(-1) == 1,
+        _require(k_scale_cache_.dtype == torch.float32 and k_scale_cache_.dim() == 3 and k_scale_cache_.stride(-1) == 1
+                 and tuple(k_scale_cache_.shape) == (num_blocks, page, hk) and k_scale_cache_.is_cuda,
                  "k_scale_cache must be fp32 (num_blocks, page_block_size, nheads_k)")
         a.ks_stride_block, a.ks_stride_row = k_scale_cache_.stride(0), k_scale_cache_.stride(1)
         if v_scale_cache_ is not None:
-            _require(v_scale_cache_.stride() == k_scale_cache_.stride() and v_scale_cache_.dtype == torch.float32,
+            _require(v_scale_cache_.stride() == k_scale_cache_.stride() and v_scale_cache_.dtype == torch.float32
+                     and v_scale_cache_.shape == k_scale_cache_.shape and v_scale_cache_.is_cuda,
                      "v_scale_cache must match k_scale_cache's layout")
     keep = [q, kcache, vcache, seqlens_k, block_table_, k_scale_cache_, v_scale_cache_]
     if k_ is not None or v_ is not None:
@@ -322,4 +328,4 @@ def varlen_fwd(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k_, leftpad_k_
     return _C().varlen_fwd(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k_, leftpad_k_, block_table_, alibi_slopes_,
                            int(max_seqlen_q), int(max_seqlen_k), float(p_dropout), float(softmax_scale), bool(zero_tensors),
                            bool(is_causal), int(window_size_left), int(window_size_right), float(softcap), bool(return_softmax),
-                           int(num_splits))
+                           gen_, int(num_splits))

@@ -190,6 +190,81 @@ def test_operator_layer_fails_loudly_without_gpu_tensors():
                                 rotary_sin=torch.zeros(8, 32, dtype=torch.bfloat16))
 
 
+def test_operator_layer_checks_every_shape_the_kernels_index_with():
+    """The kernels index v_cache and the scale caches with k_cache's page ids, rows and heads, and the table and the
+    lengths with the batch of q: a tensor that is smaller than that would be read out of bounds on the device, so it
+    is refused on the host, before the device check (these run without a GPU)."""
+    from flash_attn_npu import flash_attn_with_kvcache
+    from flash_attn_npu.flash_attn_npu import _C
+    q = torch.zeros(2, 1, 8, 128, dtype=torch.bfloat16)
+    kc = torch.zeros(4, 256, 2, 128, dtype=torch.bfloat16)
+    bt = torch.zeros(2, 2, dtype=torch.int32)
+    lens = torch.tensor([5, 6], dtype=torch.int32)
+    for bad_v in (kc[:3], kc[:, :128], kc[:, :, :1]):
+        with pytest.raises(RuntimeError, match="vcache must have the num_blocks, page_block_size and nheads_k of kcache"):
+            flash_attn_with_kvcache(q, kc, bad_v, cache_seqlens=lens, block_table=bt)
+    with pytest.raises(RuntimeError, match=r"block_table must be \(batch_size, max_num_blocks_per_seq\)"):
+        flash_attn_with_kvcache(q, kc, kc, cache_seqlens=lens, block_table=bt.view(-1))
+    with pytest.raises(RuntimeError, match="block_table / cache_seqlens batch mismatch"):
+        flash_attn_with_kvcache(q, kc, kc, cache_seqlens=lens, block_table=bt[:1])
+    with pytest.raises(RuntimeError, match=r"seqlens_k must be \(batch_size,\)"):
+        flash_attn_with_kvcache(q, kc, kc, cache_seqlens=lens.view(2, 1), block_table=bt)
+    # int8 latent cache: scale caches must cover every (block, row, head) of the code cache
+    q8 = torch.zeros(2, 1, 128, 576, dtype=torch.bfloat16)
+    codes = torch.zeros(4, 256, 1, 576, dtype=torch.int8)
+    scales = torch.ones(4, 256, 1)
+    for bad_s in (scales[:3], scales[:, :64], scales.double(), scales.view(4, 256)):
+        with pytest.raises(RuntimeError, match="k_scale_cache must be fp32"):
+            flash_attn_with_kvcache(q8, codes, codes[..., :512], cache_seqlens=lens, block_table=bt, k_scale_cache=bad_s,
+                                    v_scale_cache=scales)
+    with pytest.raises(RuntimeError, match="v_scale_cache must match"):
+        flash_attn_with_kvcache(q8, codes, codes[..., :512], cache_seqlens=lens, block_table=bt, k_scale_cache=scales,
+                                v_scale_cache=scales[:2])
+    # varlen: paged v against paged k, table and lengths against the batch
+    cu = torch.tensor([0, 4, 8], dtype=torch.int32)
+    x = torch.zeros(8, 8, 128, dtype=torch.bfloat16)
+    ext = _C()
+    tail = (4, 4, 0.0, 0.1, False, True, -1, -1, 0.0, False, None)
+    with pytest.raises(RuntimeError, match="paged v must have"):
+        ext.varlen_fwd(x, kc, kc[:3], None, cu, None, lens, None, bt, None, *tail)
+    with pytest.raises(RuntimeError, match=r"block_table must be \(batch_size"):
+        ext.varlen_fwd(x, kc, kc, None, cu, None, lens, None, bt[:1], None, *tail)
+    with pytest.raises(RuntimeError, match=r"seqused_k must be \(batch_size,\)"):
+        ext.varlen_fwd(x, kc, kc, None, cu, None, lens[:1], None, bt, None, *tail)
+    with pytest.raises(RuntimeError, match="v must have the total_k and nheads_k of k"):
+        ext.varlen_fwd(x, x, x[:4], None, cu, cu, None, None, None, None, *tail)
+    with pytest.raises(RuntimeError, match=r"cu_seqlens_k must have batch_size \+ 1 entries"):
+        ext.varlen_fwd(x, x, x, None, cu, cu[:2], None, None, None, None, *tail)
+
+
+def test_extension_module_takes_the_reference_argument_lists():
+    """flash_attn_npu.varlen_fwd is called by the reference's Python with 21 positional arguments, the last one the
+    random generator, passed as None (flash_attn_npu_interface.py:160-185; flash_api.cpp:848-869); fwd_kvcache with 20
+    (flash_attn_npu_interface.py:1556-1577).  Both argument lists must bind; num_splits of varlen_fwd is a trailing
+    extra with a default."""
+    from flash_attn_npu.flash_attn_npu import _C
+    ext = _C()
+    cu = torch.tensor([0, 4], dtype=torch.int32)
+    x = torch.zeros(4, 8, 128, dtype=torch.bfloat16)
+    ref_args = (x, x, x, None, cu, cu, None, None, None, None, 4, 4, 0.0, 0.1, False, True, -1, -1, 0.0, False, None)
+    assert len(ref_args) == 21
+    with pytest.raises(RuntimeError, match="ROCm device"):      # bound, checked, refused only for want of a GPU
+        ext.varlen_fwd(*ref_args)
+    with pytest.raises(RuntimeError, match="ROCm device"):
+        ext.varlen_fwd(*ref_args, 2)
+    with pytest.raises(RuntimeError, match="ROCm device"):
+        ext.varlen_fwd(*ref_args[:20], torch.Generator())
+    with pytest.raises(RuntimeError, match="ROCm device"):
+        ext.varlen_fwd(*ref_args[:20], num_splits=1)
+    q = torch.zeros(1, 1, 8, 128, dtype=torch.bfloat16)
+    kc = torch.zeros(4, 256, 2, 128, dtype=torch.bfloat16)
+    kv_args = (q, kc, kc, None, None, torch.tensor([5], dtype=torch.int32), None, None, None, None,
+               torch.zeros(1, 2, dtype=torch.int32), None, None, 0.1, True, -1, -1, 0.0, True, 0)
+    assert len(kv_args) == 20
+    with pytest.raises(RuntimeError, match="ROCm device"):
+        ext.fwd_kvcache(*kv_args)
+
+
 def test_even_cu_seqlens_of_empty_sequences():
     from flash_attn_npu.flash_attn_npu_interface import _even_cu_seqlens
     assert _even_cu_seqlens(3, 0, "cpu").tolist() == [0, 0, 0, 0]
