@@ -5,8 +5,8 @@
 
 A step is one call of the hot path (append + rotary + attention + split combine for the decode
 configs, one varlen forward for c5) on synthetic inputs that are resident in HBM before the
-timed region.  Two input sets are alternated so that no step finds its K/V in the 256 MB
-last-level cache.  Prints ONE JSON line: whole-call throughput (`value`, K steps between two device
+timed region.  Several input sets (distinct physical pools) are rotated so that no step finds its K/V in the
+256 MB last-level cache: as many as it takes for one rotation to read 512 MB.  Prints ONE JSON line: whole-call throughput (`value`, K steps between two device
 synchronisations), the median of the per-step durations taken with HIP events, the roofline record of
 the dominant kernel (its duration measured with HIP events the library records around it on the
 launch stream) and the CPU golden path timed on the host cores of this box.  The default (`all`) is
@@ -30,6 +30,7 @@ for _p in (os.path.join(ROOT, "flash-attention-npu_amd"), os.path.join(ROOT, "or
 
 HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
+COLD_BYTES = 512 << 20      # bytes the rotated pools of a decode config must add up to: twice the last-level cache
 
 # HBM bytes per launch of the dominant kernel are not something a timing run can see: they come from the
 # FETCH_SIZE / WRITE_SIZE counter passes whose summaries are tracked under profiles/ (a line
@@ -267,38 +268,45 @@ def run_decode(args, name, cpu_budget=(20.0, 10.0)):
     import torch
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    if name == "c4":
-        sets = [mla_workload(dev, seed=s) for s in (0, 0)]
-    else:
-        sets = [decode_workload(name, dev, seed=s, kv_layout=args.kv_layout) for s in (0, 0)]
-    # same seed -> same lengths and table, but two distinct physical pools, so that alternating
-    # them evicts the last-level cache between steps
+    # same seed -> same lengths and table, but distinct physical pools, rotated so that no step finds its K/V in the
+    # 256 MB last-level cache: as many pools as it takes for the bytes a step reads, times the pools, to reach 512 MB
+    first = mla_workload(dev, seed=0) if name == "c4" else decode_workload(name, dev, seed=0, kv_layout=args.kv_layout)
+    attn_bytes, append_bytes = decode_algorithmic_bytes(first)
+    total_bytes = attn_bytes + append_bytes
+    npools = max(2, math.ceil(COLD_BYTES / attn_bytes))
+    sets = [first] + [mla_workload(dev, seed=0) if name == "c4" else decode_workload(name, dev, seed=0, kv_layout=args.kv_layout)
+                      for _ in range(npools - 1)]
     calls = [bind_decode(w, args.num_splits) for w in sets]
     w = sets[0]
-    attn_bytes, append_bytes = decode_algorithmic_bytes(w)
-    total_bytes = attn_bytes + append_bytes
 
     for i in range(args.warmup):
-        calls[i % 2].run()
+        calls[i % npools].run()
     torch.cuda.synchronize()
+    # the timed pass: K calls between two device synchronisations, with one event on the launch stream between
+    # consecutive calls, so that the wall mean and the per-call median describe the same launches
+    stream = C.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+    marks = HipEvents(args.steps + 1)
     t0 = time.perf_counter()
+    marks.record(0, stream)
     for i in range(args.steps):
-        calls[i % 2].run()
+        calls[i % npools].run()
+        marks.record(i + 1, stream)
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     ms_per_step = wall / args.steps * 1e3
+    call_ms = [marks.elapsed_ms(i, i + 1) for i in range(args.steps)]
+    marks.close()
 
-    # second timed pass with the library's phase events: duration of the attention kernel alone
+    # a second pass with the library's phase events, for the duration of the attention kernel alone (the events
+    # between the kernels of a call would widen the call, so they stay out of the timed pass)
     ev = HipEvents(4 * args.steps)
     for i in range(args.steps):
-        calls[i % 2].run(events=ev.group(i))
+        calls[i % npools].run(events=ev.group(i))
     torch.cuda.synchronize()
     k_ms = [ev.elapsed_ms(4 * i + 1, 4 * i + 2) for i in range(args.steps)]
     a_ms = [ev.elapsed_ms(4 * i + 0, 4 * i + 1) for i in range(args.steps)]
     c_ms = [ev.elapsed_ms(4 * i + 2, 4 * i + 3) for i in range(args.steps)]
-    t_ms = [ev.elapsed_ms(4 * i + 0, 4 * i + 3) for i in range(args.steps)]
     ev.close()
-    call_ms = [ev_ms for ev_ms in t_ms]
     kern_ms = median(k_ms)
     achieved = attn_bytes / (kern_ms * 1e-3) / 1e9
     traffic, traffic_file = traffic_from_profile(name) if args.kv_layout == "nhd" and args.num_splits == 0 else (None, None)
@@ -321,9 +329,9 @@ def run_decode(args, name, cpu_budget=(20.0, 10.0)):
         "config": {"workload": f"{name}: {w['desc']}", "batch": w["B"], "q_heads": w["hq"], "kv_heads": w["hk"],
                    "headdim": w["d"], "page_block_size": w["page"], "sum_keys": int(w["lens"].sum()) + w["B"] * w["snew"],
                    "split_mode": "balanced" if plan.mode == 1 else "grid", "workgroups": plan.num_wgs, "workers": plan.num_workers,
-                   "kv_splits": plan.nsplits, "split_keys": plan.split_keys, "cold_cache": "two pools alternated", "kv_layout": args.kv_layout},
+                   "kv_splits": plan.nsplits, "split_keys": plan.split_keys, "cold_cache": f"{npools} pools rotated, {npools * attn_bytes / 2**20:.0f} MiB read per rotation (last-level cache 256 MiB)", "kv_layout": args.kv_layout},
         "us_per_call": ms_per_step * 1e3,
-        "us_per_call_median": median(call_ms) * 1e3,     # per-step HIP events on the launch stream, whole call
+        "us_per_call_median": median(call_ms) * 1e3,     # HIP events between the calls of the same timed pass
         "pct_of_hbm_peak": 100.0 * total_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,
         "algorithmic_bytes": total_bytes,
         "roofline": {"bound": "hbm", "kernel": kernel_name, "achieved": achieved, "peak": HBM_PEAK_GBPS,
@@ -386,20 +394,18 @@ def run_prefill(args, cpu_budget_s: float = 20.0):
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
+    # one timed pass: K calls between two device synchronisations; the call is a single kernel, so the events
+    # between the calls give its duration as well
+    ev = HipEvents(args.steps + 1)
+    stream = C.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    ev.record(0, stream)
+    for i in range(args.steps):
         step()
+        ev.record(i + 1, stream)
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) / args.steps * 1e3
-    # kernel duration: one kernel per call, bracketed by events on the launch stream
-    ev = HipEvents(2 * args.steps)
-    stream = C.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
-    for i in range(args.steps):
-        ev.record(2 * i, stream)
-        step()
-        ev.record(2 * i + 1, stream)
-    torch.cuda.synchronize()
-    kern_ms = median([ev.elapsed_ms(2 * i, 2 * i + 1) for i in range(args.steps)])
+    kern_ms = median([ev.elapsed_ms(i, i + 1) for i in range(args.steps)])
     ev.close()
     achieved = flops / (kern_ms * 1e-3) / 1e12
     traffic, traffic_file = traffic_from_profile("c5")
@@ -524,6 +530,8 @@ def sub_record(r):
             "roofline_mfma", "cpu_baseline", "algorithmic_bytes", "algorithmic_flops")
     d = {k: r[k] for k in keep if k in r}
     d["workload"] = r["config"]["workload"]
+    if "cold_cache" in r["config"]:
+        d["cold_cache"] = r["config"]["cold_cache"]
     return d
 
 

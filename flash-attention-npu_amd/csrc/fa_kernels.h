@@ -122,7 +122,7 @@ struct PrefillParams {
     float *lse;
     const int32_t *cu_seqlens_q;   // NULL: fixed seqlen_q per batch row (kvcache layout)
     const int32_t *cu_seqlens_k;   // dense K/V only
-    const int32_t *seqused_k;      // paged: keys per row (cache_seqlens)
+    const int32_t *seqused_k;      // paged: keys per row (cache_seqlens); dense: optional, the keys used of each sequence
     const int32_t *block_table;    // NULL: dense K/V
     int32_t batch, nheads, nheads_k, group;
     int32_t headdim;               // columns of a q / k / v / out row, a multiple of 8; the kernel is compiled for tile_headdim() of it

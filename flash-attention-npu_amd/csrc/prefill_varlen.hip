@@ -120,6 +120,7 @@ __device__ __forceinline__ void prefill_block(const PrefillParams &p, const unsi
     } else {
         k0 = p.cu_seqlens_k[b];
         Sk = p.cu_seqlens_k[b + 1] - k0;
+        if (p.seqused_k) Sk = max(0, min(Sk, p.seqused_k[b]));   // only the first seqused_k[b] keys of the sequence are used
     }
     // window normalisation: the varlen host passes max_seqlen_k as the reference does
     // (flash_api.cpp:938-943); the kvcache layout has the lengths on the device only, so the batch

@@ -266,9 +266,9 @@ std::vector<at::Tensor> varlen_fwd(const at::Tensor &q, const at::Tensor &k, con
     // flash_api.cpp:890 (the outputs are written in full either way, nothing is left to clear)
     TORCH_CHECK(!zero_tensors, "NPU FlashAttention does not support zero_tensors.");
     const bool paged = block_table_.has_value();
-    // flash_api.cpp:886 rejects seqused_k always; here it is the length array of paged K/V and has no meaning for
-    // packed keys, whose lengths are the differences of cu_seqlens_k
-    TORCH_CHECK(paged || !seqused_k_.has_value(), "NPU FlashAttention does not support seqused_k.");
+    // flash_api.cpp:886 rejects seqused_k always (the Python layer of that generation keeps doing so for packed keys);
+    // here it is the length array of paged K/V, and with packed keys the number of keys used of each sequence
+    // (flash_attn_npu_3/flash_api.cpp:143-147)
     const int64_t total_q = q.size(0), hq = q.size(1), d = q.size(2);
     const int64_t B = cu_seqlens_q.numel() - 1;
     TORCH_CHECK(B > 0, "batch size must be positive");
@@ -303,6 +303,13 @@ std::vector<at::Tensor> varlen_fwd(const at::Tensor &q, const at::Tensor &k, con
         TORCH_CHECK(k.dim() == 3 && v.dim() == 3, "k / v must be (total_k, nheads_k, headdim)");
         TORCH_CHECK(v.size(0) == k.size(0) && v.size(1) == k.size(1), "v must have the total_k and nheads_k of k");
         TORCH_CHECK(cu_seqlens_k->numel() == B + 1, "cu_seqlens_k must have batch_size + 1 entries");
+        if (seqused_k_.has_value()) {
+            seqused_k = seqused_k_.value();
+            TORCH_CHECK(seqused_k.scalar_type() == at::kInt, "seqused_k must have dtype int32");
+            TORCH_CHECK(seqused_k.dim() == 1 && seqused_k.size(0) == B, "seqused_k must be (batch_size,)");
+            seqused_k = seqused_k.contiguous();
+            a.seqused_k = seqused_k.data_ptr<int32_t>();
+        }
         hk = k.size(1);
         a.k_stride_t = k.stride(0), a.k_stride_h = k.stride(1);
         a.v_stride_t = v.stride(0), a.v_stride_h = v.stride(1);

@@ -306,6 +306,18 @@ def varlen_fwd(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k_, leftpad_k_
     """mha_varlen_fwd (flash_api.cpp:848-1089).  Returns [out, softmax_lse (Hq, total_q), p, rng_state].
     num_splits (paged K/V only; not an argument of the reference's function): 0 cuts every sequence's keys into
     as many ranges as it takes to fill the device when the query tiles alone cannot, 1 never, n at most n."""
+    # flash_api.cpp:886 (this generation's host takes seqused_k only as the lengths of paged K/V)
+    _require(block_table_ is not None or seqused_k_ is None, "NPU FlashAttention does not support seqused_k.")
+    return _varlen_fwd(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k_, leftpad_k_, block_table_, alibi_slopes_,
+                       max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale, zero_tensors, is_causal, window_size_left,
+                       window_size_right, softcap, return_softmax, gen_, num_splits=num_splits)
+
+
+def _varlen_fwd(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k_, leftpad_k_, block_table_, alibi_slopes_,
+                max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale, zero_tensors, is_causal, window_size_left,
+                window_size_right, softcap, return_softmax, gen_, *, num_splits: int = 0) -> List[torch.Tensor]:
+    """varlen_fwd without that generation's rejection of seqused_k for packed keys: with them, sequence b uses only
+    its first seqused_k[b] keys (the third-generation surface, flash_attn_npu_3/flash_api.cpp:143-147)."""
     if (isinstance(q, torch.Tensor) and q.dim() == 3 and q.shape[-1] % 8 != 0 and q.shape[-1] <= 256 and q.is_cuda
             and k.shape[-1] == q.shape[-1] and v.shape[-1] == q.shape[-1]):
         # rows that are not 16-byte pieces: zero-padded copies to the next multiple of 8, as the reference's front end
@@ -313,7 +325,7 @@ def varlen_fwd(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k_, leftpad_k_
         import torch.nn.functional as F
         d = q.shape[-1]
         extra = (d + 7) // 8 * 8 - d
-        res = varlen_fwd(F.pad(q, (0, extra)), F.pad(k, (0, extra)), F.pad(v, (0, extra)), None, cu_seqlens_q, cu_seqlens_k,
+        res = _varlen_fwd(F.pad(q, (0, extra)), F.pad(k, (0, extra)), F.pad(v, (0, extra)), None, cu_seqlens_q, cu_seqlens_k,
                          seqused_k_, leftpad_k_, block_table_, alibi_slopes_, max_seqlen_q, max_seqlen_k, p_dropout,
                          softmax_scale, zero_tensors, is_causal, window_size_left, window_size_right, softcap, return_softmax,
                          gen_, num_splits=num_splits)

@@ -250,11 +250,15 @@ def flash_attn_varlen_func(
     """Variable-length attention forward over packed sequences (reference
     flash_attn_npu_interface.py:911-958; forward only).  q: (total_q, nheads, headdim); k, v:
     (total_k, nheads_k, headdim); cu_seqlens_*: (batch+1,) int32.  Returns out, or (out, softmax_lse
-    (nheads, total_q) fp32) when return_attn_probs=True.  seqused_q / seqused_k are not supported."""
+    (nheads, total_q) fp32) when return_attn_probs=True.  seqused_k (batch,) int32: sequence b uses only the first
+    seqused_k[b] of its cu_seqlens_k[b+1] - cu_seqlens_k[b] keys (the length vector of the reference's host,
+    csrc/ascend910/flash_attn_npu_3/flash_api.cpp:143-147); the mask is aligned to that length.  seqused_q is not
+    supported (the reference's host accepts and ignores it, flash_api.cpp:71)."""
     _check_unsupported(qv, None, None, q_descale, k_descale, v_descale, attention_chunk, pack_gqa, softcap)
     _no_grad_inputs(q, k, v)
     _require(seqused_q is None, "NPU FlashAttention (MI355X build) does not support seqused_q")
-    _require(seqused_k is None, "NPU FlashAttention (MI355X build) does not support seqused_k with packed keys")
+    if seqused_k is not None:
+        _require(seqused_k.dtype == torch.int32, "seqused_k must have dtype int32")   # flash_api.cpp:146
     _require(cu_seqlens_q is not None and cu_seqlens_q.dtype == torch.int32, "cu_seqlens_q must have dtype int32")
     _require(cu_seqlens_k is not None and cu_seqlens_k.dtype == torch.int32, "cu_seqlens_k must have dtype int32")
     _require(max_seqlen_q is not None, "max_seqlen_q must be provided if cu_seqlens_q is provided")
@@ -267,8 +271,8 @@ def flash_attn_varlen_func(
     if softmax_scale is None:
         softmax_scale = q.shape[-1] ** (-0.5)
     q, k, v = [maybe_contiguous(x) for x in (q, k, v)]
-    out, lse, _, _ = _op.varlen_fwd(
-        q, k, v, None, cu_seqlens_q, cu_seqlens_k, None, None, None, None, int(max_seqlen_q), int(max_seqlen_k), 0.0,
+    out, lse, _, _ = _op._varlen_fwd(
+        q, k, v, None, cu_seqlens_q, cu_seqlens_k, seqused_k, None, None, None, int(max_seqlen_q), int(max_seqlen_k), 0.0,
         float(softmax_scale), False, bool(causal), int(window_size[0]), int(window_size[1]), float(softcap), False, None)
     return (out, lse) if return_attn_probs else out
 

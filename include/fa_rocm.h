@@ -102,7 +102,9 @@ typedef struct fa_kvcache_args {
 /*
  * Arguments of one flash_attn_varlen_func forward (token-major "TND" layout).
  * K/V are either dense (total_k, Hk, D) addressed through cu_seqlens_k, or paged
- * (block_table != NULL) with per-sequence lengths in seqused_k.
+ * (block_table != NULL) with per-sequence lengths in seqused_k.  With dense K/V seqused_k is
+ * optional: when given, sequence b uses only its first seqused_k[b] keys (the argument of that name of
+ * the reference's third-generation host, csrc/ascend910/flash_attn_npu_3/flash_api.cpp:72,143-147).
  */
 typedef struct fa_varlen_args {
     const void *q;               /* (total_q, Hq, D) */
@@ -112,7 +114,7 @@ typedef struct fa_varlen_args {
     float *softmax_lse;          /* (Hq, total_q) fp32 */
     const int32_t *cu_seqlens_q; /* (B+1,) */
     const int32_t *cu_seqlens_k; /* (B+1,) ; ignored when paged */
-    const int32_t *seqused_k;    /* (B,) ; paged only */
+    const int32_t *seqused_k;    /* (B,) ; paged: the lengths ; dense: NULL or the keys used per sequence */
     const int32_t *block_table;  /* (B, max_blocks_per_seq) or NULL */
     int32_t batch, total_q, nheads, nheads_k, headdim;
     int32_t max_seqlen_q, max_seqlen_k;
