@@ -26,7 +26,7 @@ __device__ __forceinline__ int window_norm_m(const DecodeParams &p) {
 // Rows of batch row b's query block that nobody reads (padding in front of the real query tokens): the
 // kernels compute them with the others but skip their stores and their merge.
 __device__ __forceinline__ int dead_rows(const DecodeParams &p, int b) {
-    return p.q_live ? max(p.seqlen_q - p.q_live[b], 0) * p.group : 0;
+    return (p.q_live && p.row_tiles <= 1) ? max(p.seqlen_q - p.q_live[b], 0) * p.group : 0;
 }
 
 struct UnitRange {
@@ -111,13 +111,21 @@ __device__ __forceinline__ bool batch_chunk_prefix(const DecodeParams &p, int *s
 
 // Query token and query head of row `row` of unit `kvh` of a batch row.  Ordinary caches: the unit
 // is a kv head, its rows are (query token, head of the group).  Latent int8 cache
-// (p.units_per_token > 0): the unit is (query token, 64-head group) and its rows are heads.
+// (p.units_per_token > 0): the unit is (query token, 64-head group) and its rows are heads.  Query blocks cut
+// into 16-row tiles (p.row_tiles > 1): the unit is (kv head, tile) and its rows are rows 16 * tile .. of the block;
+// rows behind the block's last get head = p.nheads, which every caller treats as "no such row".
 struct RowId { int qi, head; };
 __device__ __forceinline__ RowId row_id(const DecodeParams &p, int kvh, int row) {
     RowId r;
     if (p.units_per_token > 0) {
         r.qi = kvh / p.units_per_token;
         r.head = (kvh - r.qi * p.units_per_token) * p.group + row;
+    } else if (p.row_tiles > 1) {
+        const int kv = kvh / p.row_tiles;
+        const int full = (kvh - kv * p.row_tiles) * 16 + row;
+        r.qi = full / p.group;
+        r.head = full < p.rows_total ? kv * p.group + (full - r.qi * p.group) : p.nheads;
+        if (full >= p.rows_total) r.qi = 0;
     } else {
         r.qi = row / p.group;
         r.head = kvh * p.group + (row - r.qi * p.group);

@@ -37,6 +37,13 @@
 
 #include "decode_common.h"
 
+// This file keeps its output accumulators in a0..a255 behind the compiler's back (see below).  Whether the compiler
+// left those registers alone can only be read off the assembly it produced: build.py does that for every build
+// (_check_acc_registers) and defines this macro; a build that does not run the check must not produce this kernel.
+#ifndef FA_ROCM_ACC_REGISTERS_CHECKED
+#error "decode_mla_i8.hip must be compiled by flash-attention-npu_amd/build.py, which checks the accumulation registers in the device assembly"
+#endif
+
 namespace fa {
 
 constexpr int kMlaDqk = 576;

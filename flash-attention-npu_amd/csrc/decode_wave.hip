@@ -30,7 +30,7 @@ template <int D> struct WaveCfg {
 // Work item = one 16-byte piece of one row; in the non-interleaved rotary region the item of a
 // first-half piece also produces its partner piece rot/2 elements further on.
 template <typename T, int D, bool PART>
-__device__ __forceinline__ void stage_q_wave(const DecodeParams &p, int b, int kvh, int len_cache, uint16_t *sq) {
+__device__ __forceinline__ void stage_q_wave(const DecodeParams &p, int b, int kvh, int row0, int n_rows, int len_cache, uint16_t *sq) {
     using Cfg = WaveCfg<D>;
     const int lane = threadIdx.x & 63;
     const uint16_t *qbase = reinterpret_cast<const uint16_t *>(p.q) + (int64_t)b * p.q_stride_b;
@@ -39,11 +39,12 @@ __device__ __forceinline__ void stage_q_wave(const DecodeParams &p, int b, int k
     const int rot = (cosT != nullptr) ? p.rotary_dim : 0;
     const int half = rot >> 1;
     for (int item = lane; item < 16 * Cfg::kPiecesPerRow; item += 64) {
-        const int row = item / Cfg::kPiecesPerRow;
-        const int ci = item - row * Cfg::kPiecesPerRow;
+        const int trow = item / Cfg::kPiecesPerRow;          // row of the tile; row0 + trow of the query block
+        const int ci = item - trow * Cfg::kPiecesPerRow;
         const int d0 = ci * 8;
-        uint16_t *dst = sq + row * D + d0;
-        if (row >= p.rows || (PART && d0 >= p.headdim)) {   // padding rows, and the columns behind a head dimension below D
+        uint16_t *dst = sq + trow * D + d0;
+        const int row = row0 + trow;
+        if (row >= n_rows || (PART && d0 >= p.headdim)) {   // padding rows, and the columns behind a head dimension below D
             *reinterpret_cast<u32x4_t *>(dst) = u32x4_t{0, 0, 0, 0};
             continue;
         }
@@ -155,9 +156,13 @@ __device__ __forceinline__ void append_rows_wave(const DecodeParams &p, int b, i
 // PART: the head dimension p.headdim is below D (a multiple of 8 above D/2, or below 64 for D = 64).  The lanes whose
 // 16-byte pieces of a K / V row lie behind it load nothing and hold zeros, the k-steps and output tiles that only
 // see such pieces are skipped, and the stores stop at the head dimension.
+// A query block of more than 16 rows (p.row_tiles > 1) is cut into 16-row tiles and every (kv head, tile) is a unit of
+// its own: `row0` is the tile's first row, `n_rows` the rows of the block.  The tiles of a kv head are neighbouring
+// units, i.e. neighbouring waves of one workgroup that walk the same keys at the same time: the second one finds
+// them in the cache hierarchy, not in HBM.
 template <typename T, int D, bool SOFTCAP, bool PART>
-__device__ __forceinline__ void wave_piece(const DecodeParams &p, const int b, const int kvh, const UnitRange &ur,
-                                           const int range_lo, const int range_hi, const bool write_final,
+__device__ __forceinline__ void wave_piece(const DecodeParams &p, const int b, const int kvh, const int row0, const int n_rows,
+                                           const UnitRange &ur, const int range_lo, const int range_hi, const bool write_final,
                                            const int64_t slot, uint8_t *ktile, uint16_t *sq) {
     using Cfg = WaveCfg<D>;
     const int lane = threadIdx.x & 63;
@@ -261,6 +266,7 @@ __device__ __forceinline__ void wave_piece(const DecodeParams &p, const int b, c
         }
     };
 
+    // (with row tiles several waves read a chunk, so the host does not fuse the append then)
     if (p.k_new != nullptr && range_hi > ur.len_cache) append_rows_wave<T, D>(p, b, kvh, ur.len_cache, range_lo, range_hi);
 
     // first chunk in flight while Q is staged
@@ -275,7 +281,7 @@ __device__ __forceinline__ void wave_piece(const DecodeParams &p, const int b, c
         if (c < c_end) issue_loads(c, use_blk(blk0));
     }
 
-    stage_q_wave<T, D, PART>(p, b, kvh, ur.len_cache, sq);
+    stage_q_wave<T, D, PART>(p, b, kvh, row0, n_rows, ur.len_cache, sq);
     __builtin_amdgcn_wave_barrier();
     u32x4_t qreg[Cfg::kKSteps];
 #pragma unroll
@@ -284,10 +290,10 @@ __device__ __forceinline__ void wave_piece(const DecodeParams &p, const int b, c
     // visible key interval of query row ln, clipped to this piece
     int row_lo = range_lo, row_hi = range_hi - 1;
     {
-        const int qi = ln / p.group;
+        const int qi = (row0 + ln) / p.group;
         if (ur.wl >= 0) row_lo = max(row_lo, qi + off - ur.wl);
         if (ur.wr >= 0) row_hi = min(row_hi, qi + off + ur.wr);
-        if (ln >= p.rows) row_hi = -1;
+        if (row0 + ln >= n_rows) row_hi = -1;
     }
 
     float m_run = -INFINITY, l_run = 0.f;
@@ -400,10 +406,10 @@ __device__ __forceinline__ void wave_piece(const DecodeParams &p, const int b, c
     // ---- write.  Register i of column tile t = hh*kVW + w is column hh*128 + (lq*4 + i)*kVW + w
     //      of query row ln: kVW consecutive columns per (hh, i).
     l_run = quad_rows_sum(l_run);
-    if (ln < p.rows && ln >= dead_rows(p, b)) {
+    if (row0 + ln < n_rows && ln >= dead_rows(p, b)) {
         const float inv = (l_run > 0.f) ? 1.f / l_run : 0.f;
-        const int qi = ln / p.group;
-        const int head = kvh * p.group + (ln - qi * p.group);
+        const int qi = (row0 + ln) / p.group;
+        const int head = kvh * p.group + (row0 + ln - qi * p.group);
         if (write_final) {
             uint16_t *dst = reinterpret_cast<uint16_t *>(p.out) + (int64_t)b * p.o_stride_b + (int64_t)qi * p.o_stride_s +
                             (int64_t)head * p.o_stride_h;
@@ -449,8 +455,14 @@ __global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) decode_wave_kernel(co
     publish_partition(p, pt, s_pref);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     walk_share(p, pt, s_pref, (int64_t)blockIdx.x * 4 + wave,
-               [&](int b, int kvh, const UnitRange &ur, int range_lo, int range_hi, bool whole, int64_t slot) {
-                   wave_piece<T, D, SOFTCAP, PART>(p, b, kvh, ur, range_lo, range_hi, whole, slot, s_k[wave], s_q[wave]);
+               [&](int b, int unit, const UnitRange &ur, int range_lo, int range_hi, bool whole, int64_t slot) {
+                   int kvh = unit, row0 = 0, n_rows = p.rows;
+                   if (p.row_tiles > 1) {
+                       kvh = unit / p.row_tiles;
+                       row0 = (unit - kvh * p.row_tiles) * 16;
+                       n_rows = p.rows_total;
+                   }
+                   wave_piece<T, D, SOFTCAP, PART>(p, b, kvh, row0, n_rows, ur, range_lo, range_hi, whole, slot, s_k[wave], s_q[wave]);
                });
     init_empty_units<D>(p, pt);
 }
@@ -484,6 +496,9 @@ template <typename T> static hipError_t launch_wave_t(const DecodeParams &p, int
 
 hipError_t launch_decode_wave(const DecodeParams &p, int dtype, int headdim, hipStream_t stream) {
     if (p.rows > 16 || !p.balanced || !p.wave_workers || p.num_workers != p.num_wgs * 4) return hipErrorInvalidValue;
+    if (p.row_tiles > 1 && (p.rows != 16 || p.k_new != nullptr || p.q_live != nullptr || p.rows_total > 16 * p.row_tiles ||
+                            p.nheads_k % p.row_tiles != 0))
+        return hipErrorInvalidValue;
     return dtype == 0 ? launch_wave_t<BF16>(p, headdim, stream) : launch_wave_t<FP16>(p, headdim, stream);
 }
 

@@ -55,6 +55,10 @@ struct DecodeParams {
     int32_t piece_cost;            // balanced mode: list length charged for starting on a unit, in chunks (decode_common.h)
     int32_t split_adaptive;        // grid mode: keys per split = adaptive_split_keys(longest sequence, nsplits), not split_keys
     int32_t units_per_token;       // latent int8 cache: 64-head groups per query token (nheads_k = seqlen_q * this); else 0
+    int32_t row_tiles;             // > 1: a query block of 17 .. 16 * row_tiles rows is cut into 16-row tiles, each a unit of
+                                   // its own for the wave-level kernel: nheads_k = kv heads * row_tiles units per batch row (unit =
+                                   // kv head * row_tiles + tile), rows = 16 per unit, rows_total = seqlen_q * group; else 0 or 1
+    int32_t rows_total;            // seqlen_q * group when row_tiles > 1
 };
 
 struct AppendParams {
@@ -160,7 +164,9 @@ struct PrefillParams {
 // The partial rows of the 512-column kernel (the int8 latent cache: 128 heads x 512 columns per piece) are kept as
 // fp16: they are normalised outputs, i.e. averages of dequantised cache rows (11 significant bits against the 8 or 11
 // of the final rounding), and halving them halves what the split costs in writes and in the merge's reads.  Their
-// writer clamps to the fp16 range.  Every other width keeps fp32 partials.
+// writer clamps to the fp16 range: outputs of magnitude 6e-5 .. 65504 are independent of the partition up to the
+// rounding of the I/O type, smaller ones lose bits (zero below 6e-8) and larger ones saturate, for bf16 I/O as well.
+// Every other width keeps fp32 partials.
 constexpr bool partials_are_half(int dv) { return dv == 512; }
 
 // Balanced mode: the partition of a launch (share size, list length, prefix of the rows' chunk counts) as the decode
@@ -219,11 +225,23 @@ hipError_t launch_scatter_short_blocks(const ShortBlocksParams &p, hipStream_t s
 // Resident decode workgroups per compute unit for a head dimension / query-block height.
 inline int decode_wgs_per_cu(int headdim, int rows) { return (headdim <= 128 && rows <= 32) ? 2 : 1; }
 
-// Largest query block (seqlen_q * group) that runs on the decode kernels: one or two 16-row MFMA
-// tiles.  Taller blocks run on the tiled kernel with the GQA heads packed into its 128-row tiles, which
-// measures faster from 33 rows on for every head dimension and batch shape tried (a four-tile decode
-// variant existed: 64 rows x 8 K keys x 64 sequences 552 vs 468 us, ragged 256 x 2 K 712 vs 351 us,
-// D = 256 2131 vs 937 us).
+// Which kernel takes a query block of rows = seqlen_q * group rows (balanced partition), by measurement (64 sequences x
+// 8 K keys unless stated; us of the workgroup-level decode kernel with two row tiles / the wave-level kernel with the
+// block cut into two 16-row units / the tiled kernel with the GQA heads packed into its 128-row tiles):
+//   D = 128, 32 rows: 64q/8kv x 4 tokens 413 / 521 / 391; 32q/8kv x 8 tokens 413 / 522 / 383; MQA 32q/1kv 76 / 79 / 61;
+//            256 ragged sequences of <= 2 K keys 407 / 421 / 302; 4 sequences x 32 K 132 / 141 / 115; 18 rows 409 / 535 / 390
+//   D = 64,  32 rows: 213 / 268 / 232
+//   D = 256, 32 rows: MQA 32q/1kv 254 / 177 / 252; 64q/8kv x 4 tokens x 32 sequences 833 / 596 / 935
+// Up to 16 rows the wave-level kernel is far ahead everywhere; from 33 rows on the tiled kernel is (a four-tile decode
+// variant existed: 64 rows 552 vs 468 us, ragged 256 x 2 K 712 vs 351 us, D = 256 2131 vs 937 us; row tiles as units: 64
+// rows 842 vs 409 us).  In between the tiles of the wave-level kernel read the keys once per tile (the second read
+// comes from the cache hierarchy, but it takes a place among the loads in flight), which pays where the alternatives
+// are weakest, at D = 256.
+// Tallest block for the workgroup-level decode kernels (decode_balanced_kernel; decode_paged_kernel for explicit
+// num_splits); kDecodeMaxRows is what those kernels can take at all (two 16-row tiles).
 constexpr int kDecodeMaxRows = 32;
+inline int block_decode_max_rows(int tile_headdim) { return tile_headdim == 64 ? 32 : 16; }
+// Tallest block the wave-level kernel takes, as 16-row tiles that are units of their own.
+inline int wave_max_rows(int tile_headdim) { return tile_headdim == 256 ? 32 : 16; }
 
 }  // namespace fa

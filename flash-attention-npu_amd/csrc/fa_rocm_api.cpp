@@ -64,6 +64,7 @@ size_t partial_row_bytes(const fa_kvcache_args *a) {
 // needs them (or again when fa_rocm_reload_env() is called): nothing on the call path touches the environment.
 struct EnvKnobs {
     int decode_max_rows = 0;       // FA_ROCM_DECODE_MAX_ROWS: 16 or 32, else the built-in rule
+    int wave_max_rows = 0;         // FA_ROCM_WAVE_MAX_ROWS: 16, 32, 48 or 64: tallest block cut into 16-row tiles for the wave-level kernel
     int decode_wgs = 0;            // FA_ROCM_DECODE_WGS: workgroups of the balanced partition
     bool block_workers = false;    // FA_ROCM_DECODE_BLOCK_WORKERS
     int min_share = 0;             // FA_ROCM_MIN_SHARE
@@ -85,6 +86,7 @@ void load_env() {
         return v != nullptr && std::strcmp(v, "0") != 0;
     };
     e.decode_max_rows = num("FA_ROCM_DECODE_MAX_ROWS", 0);
+    e.wave_max_rows = num("FA_ROCM_WAVE_MAX_ROWS", 0);
     e.decode_wgs = num("FA_ROCM_DECODE_WGS", 0);
     e.block_workers = flag("FA_ROCM_DECODE_BLOCK_WORKERS");
     e.min_share = num("FA_ROCM_MIN_SHARE", 0);
@@ -134,6 +136,10 @@ __global__ void check_paged_rows_kernel(const int32_t *__restrict__ lens, const 
 int check_paged_rows(const char *what, const int32_t *lens, const int32_t *block_table, int64_t bt_stride_b, int batch, int add,
                      int page_size, int max_blocks, int num_blocks, int seqlen_ro, hipStream_t stream) {
     if (batch <= 0) return FA_OK;
+    // one set of result words per process: calls that validate (a debugging mode) take their turn, whatever their
+    // threads and streams; each waits for its own check before it returns, so the lock is held for one round trip
+    static std::mutex validate_mutex;
+    std::lock_guard<std::mutex> validate_lock(validate_mutex);
     int *result = nullptr;
     if (hipGetSymbolAddress((void **)&result, HIP_SYMBOL(g_check_result)) != hipSuccess || !result)
         return fail(FA_ERR_LAUNCH, "FA_ROCM_VALIDATE: the result words of the check kernel have no device address");
@@ -171,13 +177,27 @@ size_t tall_q_bytes(const fa_kvcache_args *a) {
     return (n + 255) / 256 * 256;
 }
 
-// Tallest query block (rows = seqlen_q * group) that runs on the decode kernels.
+// Tallest query block (rows = seqlen_q * group) that the wave-level kernel takes, cut into 16-row tiles that are units
+// of their own (fa::kWaveMaxRows; FA_ROCM_WAVE_MAX_ROWS = 16, 32, 48 or 64 overrides it for experiments).
+int wave_max_rows(const fa_kvcache_args *a) {
+    const int v = env().wave_max_rows;
+    return (v == 16 || v == 32 || v == 48 || v == 64) ? v : fa::wave_max_rows(fa::tile_headdim(a->headdim_qk));
+}
+
+// Tallest query block (rows = seqlen_q * group) that runs on the decode kernels: the workgroup-level ones up to
+// fa::block_decode_max_rows (FA_ROCM_DECODE_MAX_ROWS = 16 or 32 overrides it), the wave-level one, which runs the
+// balanced partition only, up to wave_max_rows().
 int decode_max_rows(const fa_kvcache_args *a) {
-    // tuning aid: FA_ROCM_DECODE_MAX_ROWS (16 or 32) overrides the rule
     const int v = env().decode_max_rows;
-    if (v == 16 || v == 32) return v;
-    (void)a;
-    return fa::kDecodeMaxRows;
+    const int block_level = (v == 16 || v == 32) ? v : fa::block_decode_max_rows(fa::tile_headdim(a->headdim_qk));
+    const bool wave_level = a->num_splits == 0 && !is_mla_i8(a) && !env().block_workers;
+    return wave_level ? std::max(block_level, wave_max_rows(a)) : block_level;
+}
+
+// 16-row tiles of a query block on the wave-level kernel (1: the block is one tile; 0: not that kernel's)
+int wave_row_tiles(const fa_kvcache_args *a, size_t rows) {
+    if (is_mla_i8(a) || env().block_workers || rows > (size_t)wave_max_rows(a)) return 0;
+    return (int)((rows + 15) / 16);
 }
 
 int64_t live_keys_bound(const fa_kvcache_args *a) {
@@ -301,7 +321,7 @@ int fa_rocm_plan_kvcache(const fa_kvcache_args *a, int num_cus, fa_split_plan *p
     const int group = a->nheads / a->nheads_k;
     // the int8 latent kernel works on units of 128 query heads and always uses the balanced partition
     const size_t rows = is_mla_i8(a) ? 128 : (size_t)a->seqlen_q * group;
-    const size_t slot_bytes = rows * partial_row_bytes(a);
+    size_t slot_bytes = rows * partial_row_bytes(a);
     if (!is_mla_i8(a) && rows > (size_t)decode_max_rows(a)) {
         // Query block too tall for the decode kernels: the tiled forward.  When its tiles alone
         // cannot fill the device (few sequences, short blocks) the keys of every unit are cut into
@@ -330,17 +350,19 @@ int fa_rocm_plan_kvcache(const fa_kvcache_args *a, int num_cus, fa_split_plan *p
     if (a->num_splits == 0 || is_mla_i8(a)) {
         plan->mode = FA_SPLIT_BALANCED;
         plan->nsplits = 1;
-        const int per_cu = is_mla_i8(a) ? 1 : fa::decode_wgs_per_cu(a->headdim_qk, (int)rows);
+        // Query blocks of up to wave_max_rows() rows: every wave is a worker with its own contiguous share (no
+        // workgroup barrier anywhere in the stream), blocks of more than 16 rows as 16-row tiles that are units of
+        // their own; taller blocks and the latent kernel: the workgroup is the worker.
+        const int tiles = wave_row_tiles(a, rows);
+        const bool wave_workers = tiles >= 1;
+        if (tiles > 1) slot_bytes = 16 * partial_row_bytes(a);
+        const int per_cu = is_mla_i8(a) ? 1 : fa::decode_wgs_per_cu(a->headdim_qk, wave_workers ? 16 : (int)rows);
         plan->num_wgs = num_cus * per_cu;
         // latent kernel: a piece costs ~15 us of pipeline fill and a 131 KB partial, so tiny launches are
         // not cut below 4 chunks per workgroup (1 sequence x 8 K tokens: 46 -> 37 us)
         plan->min_share = is_mla_i8(a) ? 4 : 1;
         // tuning aid: FA_ROCM_DECODE_WGS overrides the workgroup count of the balanced partition
         if (env().decode_wgs > 0) plan->num_wgs = env().decode_wgs;
-        // Query blocks of one 16-row tile: every wave is a worker with its own contiguous share (no
-        // workgroup barrier anywhere in the stream); taller blocks and the latent kernel: the
-        // workgroup is the worker.
-        const bool wave_workers = !is_mla_i8(a) && rows <= 16 && !env().block_workers;
         plan->num_workers = wave_workers ? plan->num_wgs * 4 : plan->num_wgs;
         if (wave_workers) plan->min_share = 2;   // short shares: the pipeline fill dominates tiny contexts otherwise
         if (env().min_share > 0) plan->min_share = env().min_share;
@@ -664,7 +686,15 @@ static int fwd_kvcache_impl(const fa_kvcache_args *a, void *stream_, void *const
     // charging 1-3 chunks measured within +-1 %, so it is not charged.
     p.piece_cost = is_mla_i8(a) ? 7 : 0;
     if (env().piece_cost >= 0) p.piece_cost = env().piece_cost;
-    p.head_interleave = p.wave_workers && a->nheads_k > 1 && plan.num_workers % a->nheads_k == 0 &&
+    const int row_tiles = p.wave_workers ? wave_row_tiles(a, rows) : 0;
+    if (row_tiles > 1) {
+        // (kv head, 16-row tile) units: the tiles of a kv head are neighbouring units
+        p.row_tiles = row_tiles;
+        p.rows_total = (int32_t)rows;
+        p.rows = 16;
+        p.nheads_k = a->nheads_k * row_tiles;
+    }
+    p.head_interleave = p.wave_workers && p.nheads_k > 1 && plan.num_workers % p.nheads_k == 0 &&
                         !env().no_head_interleave;
     const bool needs_combine = need > 0;
     if (needs_combine) {
@@ -678,7 +708,8 @@ static int fwd_kvcache_impl(const fa_kvcache_args *a, void *stream_, void *const
     // The wave-level kernel appends on the fly when every new position is certain to be visible
     // (and so owned by exactly one wave): causal or no right bound, and no left bound that could
     // exclude the oldest new key.  Otherwise the rows are written by their own kernel first.
-    const bool fuse_append = a->k_new && p.balanced && p.wave_workers && (a->causal || a->window_right < 0) &&
+    // With row tiles several waves read every chunk and only one of them would write the row: no fusion.
+    const bool fuse_append = a->k_new && p.balanced && p.wave_workers && row_tiles <= 1 && (a->causal || a->window_right < 0) &&
                              (a->window_left < 0 || (int64_t)a->seqlen_q + a->window_left >= a->seqlen_new) &&
                              !env().separate_append;
     if (fuse_append) {

@@ -12,6 +12,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(os.path.dirname(_HERE), "csrc", "libfa_rocm.so")
 
 FA_BF16, FA_FP16, FA_INT8 = 0, 1, 2
+ABI_VERSION = 2     # FA_ROCM_ABI_VERSION of include/fa_rocm.h this binding was written against
 
 _i32, _i64, _f32, _vp, _sz = C.c_int32, C.c_int64, C.c_float, C.c_void_p, C.c_size_t
 
@@ -91,7 +92,7 @@ def load() -> C.CDLL:
             fn = getattr(lib, name)
             fn.restype = res
             fn.argtypes = args
-        if lib.fa_rocm_abi_version() != 1:
+        if lib.fa_rocm_abi_version() != ABI_VERSION:
             raise RuntimeError("libfa_rocm.so ABI version mismatch")
         if (lib.fa_rocm_sizeof_kvcache_args() != C.sizeof(KvcacheArgs)
                 or lib.fa_rocm_sizeof_varlen_args() != C.sizeof(VarlenArgs)

