@@ -89,6 +89,23 @@ def fwd_kvcache(q, kcache, vcache, k_, v_, seqlens_k_, rotary_cos_, rotary_sin_,
                             softcap, is_rotary_interleaved, num_splits, k_scale_cache_, v_scale_cache_)
 
 
+# Head dimensions that are not multiples of 8 are served through zero-padded COPIES (rows of such widths are not made of
+# 16-byte pieces).  For q, k, v of a packed batch that is what the reference's front end does as well
+# (flash_attn_npu_interface.py:897-901); for a KV cache it means copying the cache on every call, which is only
+# acceptable while the cache is small (the reference's own test shapes with D = 1, 4, 111 are a few MB).  Beyond this many
+# bytes (K and V caches together) the call is refused with a message that says what to do instead.
+PADDED_CACHE_COPY_LIMIT = 256 << 20
+
+
+def _check_padded_cache_copy(kcache, vcache) -> None:
+    nbytes = kcache.numel() * kcache.element_size() + vcache.numel() * vcache.element_size()
+    _require(nbytes <= PADDED_CACHE_COPY_LIMIT,
+             f"head dimension {kcache.shape[-1]} is not a multiple of 8: this build serves such a KV cache through a zero-padded copy "
+             f"of the whole cache on every call, and refuses to do that for {nbytes} bytes of cache (limit {PADDED_CACHE_COPY_LIMIT}). "
+             "Allocate the cache with the head dimension rounded up to a multiple of 8 and zero columns behind the real ones "
+             "(they change neither the scores nor the kept output columns), and pass q / k / v padded the same way")
+
+
 def _fwd_kvcache_padded(q, kcache, vcache, k_, v_, seqlens_k_, rotary_cos_, rotary_sin_, cache_batch_idx_, leftpad_k_,
                         block_table_, alibi_slopes_, out_, softmax_scale, is_causal, window_size_left,
                         window_size_right, softcap, is_rotary_interleaved, num_splits) -> List[torch.Tensor]:
@@ -102,6 +119,7 @@ def _fwd_kvcache_padded(q, kcache, vcache, k_, v_, seqlens_k_, rotary_cos_, rota
     dp = (max(d, dv) + 7) // 8 * 8
     _require(kcache.dim() == 4 and vcache.dim() == 4, "q, kcache and vcache must be 4-D")
     _require(dv == d, "k and v head dimensions must match")
+    _check_padded_cache_copy(kcache, vcache)
 
     def pad(x):
         return None if x is None else F.pad(x, (0, dp - x.shape[-1]))
@@ -325,6 +343,8 @@ def _varlen_fwd(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, seqused_k_, leftpad_k
         import torch.nn.functional as F
         d = q.shape[-1]
         extra = (d + 7) // 8 * 8 - d
+        if block_table_ is not None:
+            _check_padded_cache_copy(k, v)
         res = _varlen_fwd(F.pad(q, (0, extra)), F.pad(k, (0, extra)), F.pad(v, (0, extra)), None, cu_seqlens_q, cu_seqlens_k,
                          seqused_k_, leftpad_k_, block_table_, alibi_slopes_, max_seqlen_q, max_seqlen_k, p_dropout,
                          softmax_scale, zero_tensors, is_causal, window_size_left, window_size_right, softcap, return_softmax,

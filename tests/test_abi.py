@@ -274,6 +274,17 @@ def test_extension_module_takes_the_reference_argument_lists():
         ext.fwd_kvcache(*kv_args)
 
 
+def test_padded_copy_of_a_cache_is_bounded():
+    """Head dimensions that are not multiples of 8 run through a padded copy of the cache; that is refused, with a
+    message, once the cache is large (meta tensors: no memory is touched)."""
+    from flash_attn_npu import flash_attn_npu as ops
+    small = torch.empty(64, 128, 16, 111, dtype=torch.bfloat16, device="meta")
+    ops._check_padded_cache_copy(small, small)
+    big = torch.empty(4096, 256, 8, 111, dtype=torch.bfloat16, device="meta")     # 1.9 GB per cache
+    with pytest.raises(RuntimeError, match="not a multiple of 8.*refuses.*rounded up to a multiple of 8"):
+        ops._check_padded_cache_copy(big, big)
+
+
 def test_even_cu_seqlens_of_empty_sequences():
     from flash_attn_npu.flash_attn_npu_interface import _even_cu_seqlens
     assert _even_cu_seqlens(3, 0, "cpu").tolist() == [0, 0, 0, 0]
