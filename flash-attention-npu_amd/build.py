@@ -53,17 +53,46 @@ def _check_acc_registers(src: str) -> None:
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"hipcc -S failed for {src}:\n{r.stdout}\n{r.stderr}")
+    with open(asm) as f:
+        scan_assembly(src, asm, f)
+
+
+def scan_assembly(src: str, asm: str, lines) -> None:
+    """The two checks on the device assembly of a source that pins accumulation registers (lines: its text, line by line)."""
     inside = False
-    for n, line in enumerate(open(asm), 1):
+    prev = ""          # the instruction in front of the current one
+    for n, line in enumerate(lines, 1):
+        code = line.split(";")[0].strip()
         if "ASMSTART" in line:
             inside = True
         elif "ASMEND" in line:
             inside = False
         elif not inside:
-            code = line.split(";")[0]
-            if not code.strip().startswith(".") and re.search(r"\ba\d+\b|\ba\[\d+:\d+\]", code):
+            if not code.startswith(".") and re.search(r"\ba\d+\b|\ba\[\d+:\d+\]", code):
                 raise RuntimeError(f"{src}: the compiler used an accumulation register on its own ({asm}:{n}: {line.strip()}); "
                                    "the kernel's accumulators would be overwritten")
+        if not code or code.startswith(".") or code.endswith(":"):
+            continue
+        # A hand-written matrix instruction is opaque to the compiler's hazard handling: an operand that the vector
+        # instruction right in front of it wrote is read before it has arrived (seen with v_mov_b64 in front of the
+        # instruction that zeroes the first accumulator tile).  One instruction in between is enough.
+        if inside and code.startswith("v_mfma") and prev.startswith("v_") and not prev.startswith("v_mfma"):
+            written = _vregs(prev.split(None, 1)[1].split(",")[0])
+            read = set().union(*[_vregs(t) for t in code.split(None, 1)[1].split(",")[1:]])
+            if written & read:
+                raise RuntimeError(f"{src}: a matrix instruction reads what the vector instruction in front of it wrote "
+                                   f"({asm}:{n}: {prev}  ->  {code}); put wait states in front of it")
+        prev = code
+
+
+def _vregs(tok: str) -> set:
+    """vector registers named by an assembly operand (v7, v[4:7])"""
+    tok = tok.strip()
+    m = re.match(r"v\[(\d+):(\d+)\]$", tok)
+    if m:
+        return set(range(int(m.group(1)), int(m.group(2)) + 1))
+    m = re.match(r"v(\d+)$", tok)
+    return {int(m.group(1))} if m else set()
 
 
 def _compile(src: str) -> str:

@@ -126,10 +126,11 @@ template <typename T, int BASE> __device__ __forceinline__ void acc_mfma(const u
                          : MLA_ALL_ACC);
     }
 }
-// a[BASE : BASE+15] = 0 (z must hold zeros)
+// a[BASE : BASE+15] = 0 (z must hold zeros).  The wait states in front of the first one stand for those the compiler
+// would put between the vector instruction that writes z and a matrix instruction it knows.
 template <typename T, int BASE> __device__ __forceinline__ void acc_mfma_zero(const u32x4_t &z) {
     if constexpr (BASE == 0)
-        asm volatile("v_mfma_f32_32x32x16_bf16 a[0:15], %0, %0, 0" ::"v"(z) : MLA_ALL_ACC);
+        asm volatile("s_nop 3\n\tv_mfma_f32_32x32x16_bf16 a[0:15], %0, %0, 0" ::"v"(z) : MLA_ALL_ACC);
     else
         asm volatile("v_mfma_f32_32x32x16_bf16 a[%1%2:%3%4], %0, %0, 0" ::"v"(z), "n"(BASE / 10), "n"(BASE % 10),
                      "n"((BASE + 15) / 10), "n"((BASE + 15) % 10)
@@ -377,11 +378,13 @@ __device__ __forceinline__ void mla_piece(const DecodeParams &p, const int b, co
     // vector registers (the softmax reads it there), and the products stand in the instruction stream exactly where
     // the vector work beside them is written (the wave issues in order: a product, then the few vector instructions
     // that run in its shadow).
+    // (the result of the first product is written while the operands are still being read: it may share no register
+    // with them, hence the early-clobber constraint; the accumulating form reads and writes the same registers)
     auto mfma_first = [&](float16_t &d, const u32x4_t &a, const u32x4_t &bq) {
         if constexpr (__is_same(T, BF16))
-            asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=v"(d) : "v"(a), "v"(bq));
+            asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "v"(bq));
         else
-            asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=v"(d) : "v"(a), "v"(bq));
+            asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "v"(bq));
     };
     auto mfma_v = [&](float16_t &d, const u32x4_t &a, const u32x4_t &bq) {
         if constexpr (__is_same(T, BF16))

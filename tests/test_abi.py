@@ -305,3 +305,26 @@ def test_package_exports_reference_names():
     for name in ("flash_attn_func", "flash_attn_kvpacked_func", "flash_attn_qkvpacked_func", "flash_attn_varlen_func",
                  "flash_attn_varlen_kvpacked_func", "flash_attn_varlen_qkvpacked_func", "flash_attn_with_kvcache"):
         assert callable(getattr(flash_attn_npu, name)), name
+
+
+def test_build_scans_the_assembly_of_hand_written_matrix_instructions():
+    """The build reads the device assembly of the latent kernel: the compiler may not use an accumulation register
+    of its own, and no hand-written matrix instruction may read what the vector instruction right in front of it
+    wrote (the compiler inserts no wait states for instructions it does not know)."""
+    import importlib.util
+    import os
+    spec = importlib.util.spec_from_file_location(
+        "fa_build", os.path.join(os.path.dirname(__file__), "..", "flash-attention-npu_amd", "build.py"))
+    build = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(build)
+    good = ["\tv_mov_b32_e32 v4, 0", "\t;;#ASMSTART", "\tv_mfma_f32_32x32x16_bf16 a[0:15], v[8:11], v[12:15], a[0:15]", "\t;;#ASMEND",
+            "\tv_add_f32_e32 v1, v2, v3"]
+    build.scan_assembly("k.hip", "k.s", good)
+    stray = good + ["\tv_accvgpr_write_b32 a7, v1"]
+    with pytest.raises(RuntimeError, match="accumulation register"):
+        build.scan_assembly("k.hip", "k.s", stray)
+    hazard = ["\tv_mov_b64_e32 v[8:9], s[0:1]", "\t;;#ASMSTART", "\tv_mfma_f32_32x32x16_bf16 a[0:15], v[8:11], v[8:11], 0", "\t;;#ASMEND"]
+    with pytest.raises(RuntimeError, match="matrix instruction reads"):
+        build.scan_assembly("k.hip", "k.s", hazard)
+    spaced = ["\tv_mov_b64_e32 v[8:9], s[0:1]", "\t;;#ASMSTART", "\ts_nop 3", "\tv_mfma_f32_32x32x16_bf16 a[0:15], v[8:11], v[8:11], 0", "\t;;#ASMEND"]
+    build.scan_assembly("k.hip", "k.s", spaced)
