@@ -10,8 +10,11 @@
 //     blocks under GQA are packed instead (p.pack = group): the 128 rows are (query, head of the
 //     group) pairs of one kv head, query-major, so a 16-token block of an 8-head group fills a tile
 //     and K/V are read once per kv head (the reference packs heads the same way, flash_api.cpp:33-95);
-//   * K/V tiles of 64 keys are fetched once per workgroup with 16-byte coalesced loads and
-//     double-buffered in LDS (K rows XOR-swizzled so MFMA operand reads are conflict free);
+//   * K/V tiles of 64 keys are fetched once per workgroup, 16 bytes per lane, straight from global memory
+//     into LDS (no register holds them and no LDS store instruction moves them: such a store keeps the
+//     wave from issuing anything else for ~50 cycles, and the tile stores were a tenth of the kernel's
+//     time), double-buffered (K rows XOR-swizzled so MFMA operand reads are conflict free: the lane that
+//     fills a piece's place in LDS fetches the piece that belongs there);
 //   * S^T = K Q^T and O^T = V^T P^T on the 32x32x16 MFMA: a query row is one lane column in both
 //     products, so the running max / sum / rescale never leave the lane (one xor-32 exchange);
 //   * V^T operands come straight from the transposing LDS read (ds_read_b64_tr_b16);
@@ -37,7 +40,13 @@ template <int D> struct PrefillCfg {
     static constexpr int kTileBytes = kBN * D * 2;
     static constexpr int kVRowBytes = D * 2 + 64;        // padded V rows: transposing reads spread over all banks
     static constexpr int kVTileBytes = kBN * kVRowBytes;
-    static constexpr int kPieces = kBN * kChunks / 256;  // 16-byte pieces per thread per tile
+    // A tile is filled by loads that go from global memory straight to LDS (global_load_lds_dwordx4): one instruction
+    // of a wave fills 64 consecutive 16-byte pieces, lane l the piece at the instruction's LDS base + 16 l, from
+    // whatever address the lane names.  The four waves share the pieces of a tile, instruction by instruction.
+    static constexpr int kKLoads = kBN * kChunks / 256;            // per wave and K tile
+    static constexpr int kVRowPieces = kVRowBytes / 16;            // data pieces and padding
+    static constexpr int kVLoads = kBN * kVRowPieces / 256;        // per wave and V tile
+    static_assert(kBN * kChunks % 256 == 0 && kBN * kVRowPieces % 256 == 0, "whole instructions per wave");
 };
 
 // EXT: packed heads and / or a split of the keys (p.pack, p.nsplits); without it both are compiled out
@@ -225,47 +234,67 @@ __device__ __forceinline__ void prefill_block(const PrefillParams &p, const unsi
         }
     }
 
-    // ---- K/V tile fetch: 256 threads x kPieces 16-byte pieces each --------------------------
+    // ---- K/V tile fetch ---------------------------------------------------------------------
     const uint16_t *kbase = reinterpret_cast<const uint16_t *>(p.k) + (int64_t)hk * p.k_stride_h;
     const uint16_t *vbase = reinterpret_cast<const uint16_t *>(p.v) + (int64_t)hk * p.v_stride_h;
     const int32_t *bt_row = PAGED ? p.block_table + (int64_t)b * p.bt_stride_b : nullptr;
 
-    u32x4_t kst[Cfg::kPieces], vst[Cfg::kPieces];
-    if constexpr (PART) {
+    // Load i of this wave covers the LDS pieces 64 (wave + 4i) .. + 63 of the tile, piece = (row, place in the row);
+    // a K row's place c' holds the row's piece c' ^ (row & kSwz), a V row is followed by its padding (nobody loads it).
+    // Rows past the last key re-read the last key (never memory nobody wrote; they are masked); with PART the pieces
+    // behind the head dimension are not loaded: their places hold the zeros written when the block started.
+    int k_row[Cfg::kKLoads], v_row[Cfg::kVLoads];
+    uint32_t k_col[Cfg::kKLoads], v_col[Cfg::kVLoads];          // byte offset of the lane's piece inside its row
+    bool k_on[Cfg::kKLoads], v_on[Cfg::kVLoads];
 #pragma unroll
-        for (int i = 0; i < Cfg::kPieces; ++i) kst[i] = vst[i] = u32x4_t{0, 0, 0, 0};
+    for (int i = 0; i < Cfg::kKLoads; ++i) {
+        const int piece = 64 * (wave + 4 * i) + lane;
+        k_row[i] = piece / Cfg::kChunks;
+        const int c = (piece % Cfg::kChunks) ^ (k_row[i] & Cfg::kSwz);
+        k_col[i] = c * 16;
+        k_on[i] = !PART || c * 8 < hd;
     }
-    // A thread's pieces of one tile sit 256/kChunks rows apart and tiles kBN rows apart, so one small
-    // per-thread byte offset plus wave-uniform (scalar) terms addresses every load of an interior
-    // tile of dense K/V, and one per-thread LDS offset plus constants every store.
-    constexpr int kRowsPerPass = 256 / Cfg::kChunks;
-    const int t_row = tid / Cfg::kChunks;
-    const int t_ch = tid % Cfg::kChunks;
-    const bool piece_live = !PART || t_ch * 8 < hd;
-    const uint32_t k_thread_off = (uint32_t)t_row * (uint32_t)p.k_stride_t * 2u + t_ch * 16;
-    const uint32_t v_thread_off = (uint32_t)t_row * (uint32_t)p.v_stride_t * 2u + t_ch * 16;
-    const uint32_t k_lds_off = t_row * (D * 2) + ((t_ch ^ (t_row & Cfg::kSwz)) << 4);   // row + 16*i keeps row & 15
-    const uint32_t v_lds_off = t_row * Cfg::kVRowBytes + (t_ch << 4);
-    static_assert(kRowsPerPass % (Cfg::kSwz + 1) == 0 && Cfg::kSwz < Cfg::kChunks, "swizzle must survive the row step");
-    auto fetch_tile = [&](int kt) {
-        if (!piece_live) return;
+#pragma unroll
+    for (int i = 0; i < Cfg::kVLoads; ++i) {
+        const int piece = 64 * (wave + 4 * i) + lane;
+        v_row[i] = piece / Cfg::kVRowPieces;
+        const int c = piece % Cfg::kVRowPieces;
+        v_col[i] = c * 16;
+        v_on[i] = c < Cfg::kChunks && (!PART || c * 8 < hd);
+    }
+    // per-lane offsets of an interior tile of dense K/V (one wave-uniform base per tile serves all its loads)
+    uint32_t k_off[Cfg::kKLoads], v_off[Cfg::kVLoads];
+#pragma unroll
+    for (int i = 0; i < Cfg::kKLoads; ++i) k_off[i] = (uint32_t)k_row[i] * (uint32_t)p.k_stride_t * 2u + k_col[i];
+#pragma unroll
+    for (int i = 0; i < Cfg::kVLoads; ++i) v_off[i] = (uint32_t)v_row[i] * (uint32_t)p.v_stride_t * 2u + v_col[i];
+    auto lds_of = [](const void *ptr) -> uint32_t { return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void *)ptr; };
+    // The loads are written out: the compiler would wait for such a load in front of every LDS read that follows (it
+    // cannot tell the two buffers apart).  tiles_landed() is the wait that orders them.
+    auto load_lds_base = [&](uint32_t lds, uint32_t off, const uint8_t *base) {
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds), "v"(off), "s"(base) : "memory", "m0");
+    };
+    auto load_lds_addr = [&](uint32_t lds, const void *addr) {
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds), "v"(addr) : "memory", "m0");
+    };
+    auto tiles_landed = [&]() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); };
+    auto fetch_tile = [&](int kt, int buf) {
+        const uint32_t k_lds = lds_of(&s_k[buf][0]) + (uint32_t)wave * 1024u, v_lds = lds_of(&s_v[buf][0]) + (uint32_t)wave * 1024u;
         if constexpr (!PAGED) {
             if (kt * kBN + kBN <= Sk) {
                 const uint8_t *kb = reinterpret_cast<const uint8_t *>(kbase) + (int64_t)(k0 + kt * kBN) * p.k_stride_t * 2;
                 const uint8_t *vb = reinterpret_cast<const uint8_t *>(vbase) + (int64_t)(k0 + kt * kBN) * p.v_stride_t * 2;
 #pragma unroll
-                for (int i = 0; i < Cfg::kPieces; ++i) {
-                    kst[i] = load16(kb + (int64_t)i * kRowsPerPass * p.k_stride_t * 2 + k_thread_off);
-                    vst[i] = load16(vb + (int64_t)i * kRowsPerPass * p.v_stride_t * 2 + v_thread_off);
-                }
+                for (int i = 0; i < Cfg::kKLoads; ++i)
+                    if (k_on[i]) load_lds_base(k_lds + i * 4096u, k_off[i], kb);
+#pragma unroll
+                for (int i = 0; i < Cfg::kVLoads; ++i)
+                    if (v_on[i]) load_lds_base(v_lds + i * 4096u, v_off[i], vb);
                 return;
             }
         }
-#pragma unroll
-        for (int i = 0; i < Cfg::kPieces; ++i) {
-            const int row = t_row + kRowsPerPass * i;
+        auto row_offsets = [&](int row, int64_t &koff, int64_t &voff) {
             const int key = min(kt * kBN + row, Sk - 1);
-            int64_t koff, voff;
             if constexpr (PAGED) {
                 const int page = key / p.page_size;
                 int blk = bt_row[page];
@@ -277,17 +306,26 @@ __device__ __forceinline__ void prefill_block(const PrefillParams &p, const unsi
                 koff = (int64_t)(k0 + key) * p.k_stride_t;
                 voff = (int64_t)(k0 + key) * p.v_stride_t;
             }
-            kst[i] = load16(kbase + koff + t_ch * 8);
-            vst[i] = load16(vbase + voff + t_ch * 8);
-        }
-    };
-    auto stash_tile = [&](int buf) {
+        };
 #pragma unroll
-        for (int i = 0; i < Cfg::kPieces; ++i) {
-            *reinterpret_cast<u32x4_t *>(&s_k[buf][k_lds_off + i * kRowsPerPass * (D * 2)]) = kst[i];
-            *reinterpret_cast<u32x4_t *>(&s_v[buf][v_lds_off + i * kRowsPerPass * Cfg::kVRowBytes]) = vst[i];
+        for (int i = 0; i < Cfg::kKLoads; ++i) {
+            int64_t koff, voff;
+            row_offsets(k_row[i], koff, voff);
+            if (k_on[i]) load_lds_addr(k_lds + i * 4096u, reinterpret_cast<const uint8_t *>(kbase + koff) + k_col[i]);
+        }
+#pragma unroll
+        for (int i = 0; i < Cfg::kVLoads; ++i) {
+            int64_t koff, voff;
+            row_offsets(v_row[i], koff, voff);
+            if (v_on[i]) load_lds_addr(v_lds + i * 4096u, reinterpret_cast<const uint8_t *>(vbase + voff) + v_col[i]);
         }
     };
+    if constexpr (PART) {
+        // the places of the pieces that nobody loads
+        for (int i = tid * 16; i < 2 * Cfg::kTileBytes; i += 256 * 16) *reinterpret_cast<u32x4_t *>(&s_k[0][0] + i) = u32x4_t{0, 0, 0, 0};
+        for (int i = tid * 16; i < 2 * Cfg::kVTileBytes; i += 256 * 16) *reinterpret_cast<u32x4_t *>(&s_v[0][0] + i) = u32x4_t{0, 0, 0, 0};
+        __syncthreads();
+    }
 
     float m_run = -INFINITY, l_run = 0.f;
     float16_t o_acc[Cfg::kMT];
@@ -299,14 +337,14 @@ __device__ __forceinline__ void prefill_block(const PrefillParams &p, const unsi
     const int kt_begin = k_lo / kBN;
     const int kt_end = (k_hi + kBN - 1) / kBN;
     const bool wave_live = __builtin_amdgcn_readfirstlane(R0 + wave * 32 < n_rows);
-    fetch_tile(kt_begin);
-    stash_tile(0);
+    fetch_tile(kt_begin, 0);
+    tiles_landed();
     __syncthreads();
 
     int cur = 0;
     for (int kt = kt_begin; kt < kt_end; ++kt) {
         const bool more = kt + 1 < kt_end;
-        if (more) fetch_tile(kt + 1);
+        if (more) fetch_tile(kt + 1, cur ^ 1);   // the other buffer: its readers passed the barrier that ended the last step
         __builtin_amdgcn_sched_barrier(0);
 
         // a wave whose 32 rows all lie past the block's end (short blocks: a decode row among prompt chunks
@@ -481,7 +519,7 @@ __device__ __forceinline__ void prefill_block(const PrefillParams &p, const unsi
         __builtin_amdgcn_s_setprio(0);
         }   // wave_live
 
-        if (more) stash_tile(cur ^ 1);
+        tiles_landed();
         __syncthreads();
         cur ^= 1;
     }
