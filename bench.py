@@ -37,7 +37,8 @@ COLD_BYTES = 512 << 20      # bytes the rotated pools of a decode config must ad
 # "traffic_bytes_per_launch: N" in the summary of that kernel and workload).  The workloads are seeded, so the
 # figure belongs to the kernel as it was when the summary was made; the record names the file it was read from.
 PROFILE_OF = {"c2": "decode_wave_kernel_c2.txt", "c2_8k": "decode_wave_kernel_c2_8k.txt", "c3a": "decode_wave_kernel_c3a.txt", "c3b": "decode_wave_kernel_c3b.txt",
-              "c4": "decode_mla_i8_kernel_c4.txt", "c5": "prefill_kernel_c5.txt"}
+              "c4": "decode_mla_i8_kernel_c4.txt", "c5": "prefill_kernel_c5.txt",
+              "mqa32": "prefill_kernel_mqa32.txt", "mqa32_d256": "decode_wave_kernel_mqa32_d256.txt"}
 
 
 def traffic_from_profile(name: str):
@@ -121,6 +122,14 @@ def decode_workload(name: str, device, seed: int = 0, kv_layout: str = "nhd"):
         snew, rotary, spare = 0, False, 0
         window = (-1, -1) if name == "c3a" else (4095, 0)
         desc = f"long-context split-KV decode bf16 B=4 64q/8kv d=128 Lk=131072 window={window} causal"
+    elif name in ("mqa32", "mqa32_d256", "mqa32_d64", "g32k8", "g32k8_d64", "g32k8_d256"):
+        # query blocks of 17..32 rows (one token x 32 q heads of one kv head): past the 16 rows of one decode tile
+        B, hq, hk, d = 64, 32, 1, (128 if name in ("mqa32", "g32k8") else int(name[7:]))
+        if name.startswith("g32k8"):
+            hq, hk = 256, 8
+        lens = torch.full((B,), 8192)
+        snew, rotary, window, spare = 0, False, (-1, -1), 16
+        desc = f"multi-query paged decode bf16 B=64 32q/1kv d={d} page=256 all rows 8192 keys causal (32-row query blocks)"
     else:
         raise ValueError(name)
     pages = [math.ceil((int(l) + snew) / page) for l in lens]
@@ -318,6 +327,8 @@ def run_decode(args, name, cpu_budget=(20.0, 10.0)):
 
     if name == "c4":
         kernel_name = "decode_mla_i8_kernel"
+    elif plan.mode != 1 and w["hq"] // w["hk"] > 16 and w["d"] >= 128:
+        kernel_name = "prefill_kernel"        # a query block too tall for the decode kernels of this head dimension: the tiled forward
     elif plan.mode == 1:
         kernel_name = "decode_wave_kernel" if plan.num_workers > plan.num_wgs else "decode_balanced_kernel"
     else:
@@ -561,7 +572,7 @@ def main():
             subs[name] = sub_record(r)
         subs["c5"] = sub_record(run_prefill(args, cpu_budget_s=3.0))
         out["configs"] = subs
-    elif args.config in ("c2", "c2_8k", "c3a", "c3b", "c4") or args.config.startswith("c2_u"):
+    elif args.config in ("c2", "c2_8k", "c3a", "c3b", "c4", "mqa32", "mqa32_d256", "mqa32_d64", "g32k8", "g32k8_d64", "g32k8_d256") or args.config.startswith("c2_u"):
         out = run_decode(args, args.config)
     elif args.config == "c5":
         out = run_prefill(args)

@@ -6,9 +6,12 @@
 //
 // Same arithmetic as decode_paged.hip (the reference's hot loop, csrc/ascend910/flash_attn_npu/
 // mha_fwd_kvcache.cpp:632-969): S^T = K Q^T and O^T = V^T P^T on the 16x16x32 MFMA with the query
-// row in lane column lane%16; K rows through a wave-private swizzled LDS tile, V rows loaded in
-// operand order and transposed with v_perm; P rounded to the I/O dtype before PV.  Used when the
-// query block (seqlen_q * group rows) fits one 16-row tile.
+// row in lane column lane%16; K rows through a wave-private swizzled LDS tile, which they reach
+// straight from global memory (global_load_lds_dwordx4: no register holds them and no LDS store
+// instruction moves them; two tiles per wave, the chunk being read and the chunk on its way); V rows
+// loaded in operand order and transposed with v_perm; P rounded to the I/O dtype before PV.  Used
+// when the query block (seqlen_q * group rows) fits one 16-row tile, or two where a wave's registers
+// hold two sets of accumulators.
 #include "decode_common.h"
 
 namespace fa {
@@ -160,10 +163,17 @@ __device__ __forceinline__ void append_rows_wave(const DecodeParams &p, int b, i
 // its own: `row0` is the tile's first row, `n_rows` the rows of the block.  The tiles of a kv head are neighbouring
 // units, i.e. neighbouring waves of one workgroup that walk the same keys at the same time: the second one finds
 // them in the cache hierarchy, not in HBM.
-template <typename T, int D, bool SOFTCAP, bool PART>
+// RT = 2: the wave carries TWO 16-row tiles (rows row0 .. row0 + 31) through one pass over the keys: every K operand it
+// reads from its LDS tile and every V operand it builds feeds two matrix instructions, and the chunk in flight - what
+// bounds a stream like this one - serves 32 rows.  The registers that the second set of accumulators takes are those
+// that staged K: with RT = 2 the K rows of a chunk go from global memory straight to LDS (global_load_lds_dwordx4: lane
+// l's 16 bytes land at the instruction's LDS base + 16 l, so the lane that fills a place of the swizzled tile fetches
+// the piece that belongs there), into the one of the wave's two tiles that is not being read; `ktile` then points at
+// both (2 * kTileBytes), and the second doubles as the staging area of the q rows before the first chunk uses it.
+template <typename T, int D, bool SOFTCAP, bool PART, int RT>
 __device__ __forceinline__ void wave_piece(const DecodeParams &p, const int b, const int kvh, const int row0, const int n_rows,
                                            const UnitRange &ur, const int range_lo, const int range_hi, const bool write_final,
-                                           const int64_t slot, uint8_t *ktile, uint16_t *sq) {
+                                           const int64_t slot, uint8_t *ktile) {
     using Cfg = WaveCfg<D>;
     const int lane = threadIdx.x & 63;
     const int lq = lane >> 4;
@@ -178,16 +188,12 @@ __device__ __forceinline__ void wave_piece(const DecodeParams &p, const int b, c
     const int c_begin = range_lo / kChunk;
     const int c_end = (range_hi + kChunk - 1) / kChunk;
 
-    u32x4_t kreg[Cfg::kKLoads];
     uint32_t vreg[8][Cfg::kVH][Cfg::kVW / 2];
     const int hd = PART ? p.headdim : D;
-    const bool k_live = !PART || (lane % Cfg::kLanesPerRow) * 8 < hd;
     bool v_live[Cfg::kVH];
 #pragma unroll
     for (int hh = 0; hh < Cfg::kVH; ++hh) v_live[hh] = !PART || hh * 128 + ln * Cfg::kVW < hd;
     if constexpr (PART) {
-#pragma unroll
-        for (int j = 0; j < Cfg::kKLoads; ++j) kreg[j] = u32x4_t{0, 0, 0, 0};
 #pragma unroll
         for (int e = 0; e < 8; ++e)
 #pragma unroll
@@ -198,9 +204,24 @@ __device__ __forceinline__ void wave_piece(const DecodeParams &p, const int b, c
     const uint32_t k_row_bytes = (uint32_t)p.k_stride_row * 2u;
     const uint32_t v_row_bytes = (uint32_t)p.v_stride_row * 2u;
     const int k_lane_row = lane / Cfg::kLanesPerRow;
-    const uint32_t k_lane_col = (uint32_t)(lane % Cfg::kLanesPerRow) * 16u;
     const uint32_t v_lane_col = (uint32_t)(ln * Cfg::kVW) * 2u;
-    const uint32_t k_lane_off = (uint32_t)k_lane_row * k_row_bytes + k_lane_col;
+    // direct loads: load j fills the LDS pieces 64j .. 64j+63 of the tile = rows j * kRowsPerLoad .., the lane's place c' of
+    // row r holds the row's piece c' ^ (r & kSwzMask); kd_col[j % kSwzRows]: that piece's byte offset in its row
+    constexpr int kSwzRows = (Cfg::kSwzMask + 1 + Cfg::kRowsPerLoad - 1) / Cfg::kRowsPerLoad;   // loads after which the pattern repeats
+    uint32_t kd_col[kSwzRows], kd_off[kSwzRows];   // ... and with the lane's row inside a load added (chunks inside the sequence)
+    bool kd_live[kSwzRows];
+#pragma unroll
+    for (int j = 0; j < kSwzRows; ++j) {
+        const int c = (lane % Cfg::kLanesPerRow) ^ ((j * Cfg::kRowsPerLoad + k_lane_row) & Cfg::kSwzMask);
+        kd_col[j] = (uint32_t)c * 16u;
+        kd_off[j] = (uint32_t)k_lane_row * k_row_bytes + kd_col[j];
+        kd_live[j] = !PART || c * 8 < hd;
+    }
+    auto lds_of = [](const void *ptr) -> uint32_t { return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void *)ptr; };
+    // (written out: the compiler would wait for such a load in front of every LDS read that follows)
+    auto load_k_direct = [&](uint32_t lds, uint32_t off, const uint8_t *base) {
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(lds), "v"(off), "s"(base) : "memory", "m0");
+    };
     const uint32_t v_lane_off = (uint32_t)(lq * 4) * v_row_bytes + v_lane_col;
 
     auto load_blk = [&](int c) -> int {   // the table entry as loaded (every lane the same address); not waited for
@@ -226,18 +247,18 @@ __device__ __forceinline__ void wave_piece(const DecodeParams &p, const int b, c
             vreg[e][hh][0] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(s2));
         }
     };
-    auto issue_loads = [&](int c, int blk) {
+    auto issue_loads = [&](int c, int blk, int kbuf) {
         const int key0 = c * kChunk;
         const int inpage0 = key0 % p.page_size;
         const int last = Lk - 1 - key0;  // last written key relative to the chunk (>= 0)
         const uint8_t *kb = kc_base + (int64_t)blk * p.k_stride_block * 2 + (int64_t)inpage0 * k_row_bytes;
         const uint8_t *vb = vc_base + (int64_t)blk * p.v_stride_block * 2 + (int64_t)inpage0 * v_row_bytes;
+        const uint32_t lds = lds_of(ktile + kbuf * Cfg::kTileBytes);
         if (last >= kChunk - 1) {
-            if (k_live) {
 #pragma unroll
-                for (int j = 0; j < Cfg::kKLoads; ++j)
-                    kreg[j] = load16_stream(kb + (size_t)(j * Cfg::kRowsPerLoad) * k_row_bytes + k_lane_off);
-            }
+            for (int j = 0; j < Cfg::kKLoads; ++j)
+                if (kd_live[j % kSwzRows])
+                    load_k_direct(lds + j * 1024u, kd_off[j % kSwzRows], kb + (size_t)(j * Cfg::kRowsPerLoad) * k_row_bytes);
 #pragma unroll
             for (int hh = 0; hh < Cfg::kVH; ++hh)
                 if (v_live[hh]) {
@@ -247,12 +268,10 @@ __device__ __forceinline__ void wave_piece(const DecodeParams &p, const int b, c
                 }
         } else {
             // tail chunk: rows past the last written key re-read that key (their scores are masked)
-            if (k_live) {
 #pragma unroll
-                for (int j = 0; j < Cfg::kKLoads; ++j) {
-                    const int row = min(j * Cfg::kRowsPerLoad + k_lane_row, last);
-                    kreg[j] = load16(kb + (uint32_t)row * k_row_bytes + k_lane_col);
-                }
+            for (int j = 0; j < Cfg::kKLoads; ++j) {
+                const int row = min(j * Cfg::kRowsPerLoad + k_lane_row, last);
+                if (kd_live[j % kSwzRows]) load_k_direct(lds + j * 1024u, (uint32_t)row * k_row_bytes + kd_col[j % kSwzRows], kb);
             }
 #pragma unroll
             for (int hh = 0; hh < Cfg::kVH; ++hh)
@@ -269,6 +288,11 @@ __device__ __forceinline__ void wave_piece(const DecodeParams &p, const int b, c
     // (with row tiles several waves read a chunk, so the host does not fuse the append then)
     if (p.k_new != nullptr && range_hi > ur.len_cache) append_rows_wave<T, D>(p, b, kvh, ur.len_cache, range_lo, range_hi);
 
+    if constexpr (PART) {
+        // the places of the K pieces that nobody loads hold zeros: the first tile here, the second once the q rows have left it
+        for (int i = lane * 16; i < Cfg::kTileBytes; i += 64 * 16) *reinterpret_cast<u32x4_t *>(ktile + i) = u32x4_t{0, 0, 0, 0};
+        __builtin_amdgcn_wave_barrier();
+    }
     // first chunk in flight while Q is staged
     int c = c_begin;
     int blk_next;
@@ -278,28 +302,49 @@ __device__ __forceinline__ void wave_piece(const DecodeParams &p, const int b, c
         // memory latency later than they need be.
         const int blk0 = load_blk(c);
         blk_next = load_blk(c + 1);
-        if (c < c_end) issue_loads(c, use_blk(blk0));
+        if (c < c_end) issue_loads(c, use_blk(blk0), 0);
     }
+    // the q rows are staged in the wave's second tile: the first chunk that lands there leaves after they have been read
+    uint16_t *sq = reinterpret_cast<uint16_t *>(ktile + Cfg::kTileBytes);
+    static_assert(RT * 16 * D * 2 <= Cfg::kTileBytes, "the q rows fit a tile");
 
-    stage_q_wave<T, D, PART>(p, b, kvh, row0, n_rows, ur.len_cache, sq);
+#pragma unroll
+    for (int r = 0; r < RT; ++r) stage_q_wave<T, D, PART>(p, b, kvh, row0 + 16 * r, n_rows, ur.len_cache, sq + r * 16 * D);
     __builtin_amdgcn_wave_barrier();
-    u32x4_t qreg[Cfg::kKSteps];
+    u32x4_t qreg[RT][Cfg::kKSteps];
 #pragma unroll
-    for (int t = 0; t < Cfg::kKSteps; ++t) qreg[t] = *reinterpret_cast<const u32x4_t *>(&sq[ln * D + t * 32 + lq * 8]);
+    for (int r = 0; r < RT; ++r)
+#pragma unroll
+        for (int t = 0; t < Cfg::kKSteps; ++t) qreg[r][t] = *reinterpret_cast<const u32x4_t *>(&sq[(r * 16 + ln) * D + t * 32 + lq * 8]);
 
-    // visible key interval of query row ln, clipped to this piece
-    int row_lo = range_lo, row_hi = range_hi - 1;
-    {
-        const int qi = (row0 + ln) / p.group;
-        if (ur.wl >= 0) row_lo = max(row_lo, qi + off - ur.wl);
-        if (ur.wr >= 0) row_hi = min(row_hi, qi + off + ur.wr);
-        if (row0 + ln >= n_rows) row_hi = -1;
+    if constexpr (PART) {
+        // the places of the K pieces that nobody loads hold zeros (the q rows lay elsewhere in this tile)
+        __builtin_amdgcn_wave_barrier();
+        for (int i = lane * 16; i < Cfg::kTileBytes; i += 64 * 16) *reinterpret_cast<u32x4_t *>(ktile + Cfg::kTileBytes + i) = u32x4_t{0, 0, 0, 0};
+        __builtin_amdgcn_wave_barrier();
+    }
+    // visible key interval of query row ln of every tile, clipped to this piece
+    int row_lo[RT], row_hi[RT];
+#pragma unroll
+    for (int r = 0; r < RT; ++r) {
+        row_lo[r] = range_lo;
+        row_hi[r] = range_hi - 1;
+        const int row = row0 + 16 * r + ln;
+        const int qi = row / p.group;
+        if (ur.wl >= 0) row_lo[r] = max(row_lo[r], qi + off - ur.wl);
+        if (ur.wr >= 0) row_hi[r] = min(row_hi[r], qi + off + ur.wr);
+        if (row >= n_rows) row_hi[r] = -1;
     }
 
-    float m_run = -INFINITY, l_run = 0.f;
-    float4_t o_acc[Cfg::kColTiles];
+    float m_run[RT], l_run[RT];
+    float4_t o_acc[RT][Cfg::kColTiles];
 #pragma unroll
-    for (int t = 0; t < Cfg::kColTiles; ++t) o_acc[t] = float4_t{0.f, 0.f, 0.f, 0.f};
+    for (int r = 0; r < RT; ++r) {
+        m_run[r] = -INFINITY;
+        l_run[r] = 0.f;
+#pragma unroll
+        for (int t = 0; t < Cfg::kColTiles; ++t) o_acc[r][t] = float4_t{0.f, 0.f, 0.f, 0.f};
+    }
 
     // The two waves of a SIMD belong to different workgroups and stream independent shares; with
     // equal priority the older one (wave slot 0) wins every arbitration and finishes ~10 % earlier,
@@ -313,12 +358,9 @@ __device__ __forceinline__ void wave_piece(const DecodeParams &p, const int b, c
         else
             __builtin_amdgcn_s_setprio(0);
         // staged chunk: K -> swizzled LDS tile, V -> transposed operand registers
-#pragma unroll
-        for (int j = 0; j < Cfg::kKLoads; ++j) {
-            const int row = j * Cfg::kRowsPerLoad + k_lane_row;
-            const int ch = lane % Cfg::kLanesPerRow;
-            *reinterpret_cast<u32x4_t *>(ktile + row * (D * 2) + ((ch ^ (row & Cfg::kSwzMask)) << 4)) = kreg[j];
-        }
+        const int kbuf = (c - c_begin) & 1;
+        const uint8_t *kt = ktile + kbuf * Cfg::kTileBytes;
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the chunk's K rows are in their tile (and its V rows in their registers)
         u32x4_t vt[Cfg::kColTiles];
 #pragma unroll
         for (int hh = 0; hh < Cfg::kVH; ++hh)
@@ -334,14 +376,16 @@ __device__ __forceinline__ void wave_piece(const DecodeParams &p, const int b, c
         __builtin_amdgcn_wave_barrier();
 
         const int cn = c + 1;
-        if (cn < c_end) issue_loads(cn, use_blk(blk_next));
+        if (cn < c_end) issue_loads(cn, use_blk(blk_next), kbuf ^ 1);
         // asked for behind the chunk's loads, the next table entry is there when they all are: the wave rests here
         // until chunk cn has landed and only then works on chunk c
         blk_next = __builtin_amdgcn_readfirstlane(load_blk(cn + 1));
         __builtin_amdgcn_sched_barrier(0);
 
-        // S^T = K Q^T, two 16-key tiles
-        float4_t s[2] = {float4_t{0.f, 0.f, 0.f, 0.f}, float4_t{0.f, 0.f, 0.f, 0.f}};
+        // S^T = K Q^T, two 16-key tiles (for every row tile)
+        float4_t s[RT][2];
+#pragma unroll
+        for (int r = 0; r < RT; ++r) s[r][0] = s[r][1] = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int t = 0; t < Cfg::kKSteps; ++t) {
             if (PART && t * 32 >= hd) continue;   // wave-uniform
@@ -349,140 +393,162 @@ __device__ __forceinline__ void wave_piece(const DecodeParams &p, const int b, c
             for (int tt = 0; tt < 2; ++tt) {
                 const int row = tt * 16 + ln;
                 const u32x4_t a = *reinterpret_cast<const u32x4_t *>(
-                    ktile + row * (D * 2) + (((t * 4 + lq) ^ (row & Cfg::kSwzMask)) << 4));
-                s[tt] = mfma16<T>(a, qreg[t], s[tt]);
+                    kt + row * (D * 2) + (((t * 4 + lq) ^ (row & Cfg::kSwzMask)) << 4));
+#pragma unroll
+                for (int r = 0; r < RT; ++r) s[r][tt] = mfma16<T>(a, qreg[r][t], s[r][tt]);
             }
         }
 
-        // online softmax of query row ln; register i of tile tt is key c*32 + tt*16 + lq*4 + i
+        // online softmax of query row ln of every tile; register i of key tile tt is key c*32 + tt*16 + lq*4 + i
         const int key_base = c * kChunk + lq * 4;
-        float x[8];
-        float mloc = -INFINITY;
+        u32x4_t pk[RT];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const int key = key_base + (e >> 2) * 16 + (e & 3);
-            float v = s[e >> 2][e & 3];
-            if constexpr (SOFTCAP) {
-                const float y = v * p.softcap_pre;
-                const float e2 = __expf(2.f * y);
-                v = p.softcap_post * (1.f - 2.f / (e2 + 1.f));
-            } else {
-                v *= p.scale_log2;
+        for (int r = 0; r < RT; ++r) {
+            float x[8];
+            float mloc = -INFINITY;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const int key = key_base + (e >> 2) * 16 + (e & 3);
+                float v = s[r][e >> 2][e & 3];
+                if constexpr (SOFTCAP) {
+                    const float y = v * p.softcap_pre;
+                    const float e2 = __expf(2.f * y);
+                    v = p.softcap_post * (1.f - 2.f / (e2 + 1.f));
+                } else {
+                    v *= p.scale_log2;
+                }
+                v = (key >= row_lo[r] && key <= row_hi[r]) ? v : -INFINITY;
+                x[e] = v;
+                mloc = fmaxf(mloc, v);
             }
-            v = (key >= row_lo && key <= row_hi) ? v : -INFINITY;
-            x[e] = v;
-            mloc = fmaxf(mloc, v);
-        }
-        mloc = quad_rows_max(mloc);
-        const float m_new = fmaxf(m_run, mloc);
-        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-        const float alpha = fast_exp2(m_run - m_use);
-        m_run = m_new;
-        float psum = 0.f;
+            mloc = quad_rows_max(mloc);
+            const float m_new = fmaxf(m_run[r], mloc);
+            const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+            const float alpha = fast_exp2(m_run[r] - m_use);
+            m_run[r] = m_new;
+            float psum = 0.f;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            x[e] = fast_exp2(x[e] - m_use);
-            psum += x[e];
-        }
-        l_run = l_run * alpha + psum;
-        u32x4_t pk;
-        pk[0] = pack2<T>(x[0], x[1]);
-        pk[1] = pack2<T>(x[2], x[3]);
-        pk[2] = pack2<T>(x[4], x[5]);
-        pk[3] = pack2<T>(x[6], x[7]);
+            for (int e = 0; e < 8; ++e) {
+                x[e] = fast_exp2(x[e] - m_use);
+                psum += x[e];
+            }
+            l_run[r] = l_run[r] * alpha + psum;
+            pk[r][0] = pack2<T>(x[0], x[1]);
+            pk[r][1] = pack2<T>(x[2], x[3]);
+            pk[r][2] = pack2<T>(x[4], x[5]);
+            pk[r][3] = pack2<T>(x[6], x[7]);
 #pragma unroll
-        for (int t = 0; t < Cfg::kColTiles; ++t) {
-            o_acc[t][0] *= alpha;
-            o_acc[t][1] *= alpha;
-            o_acc[t][2] *= alpha;
-            o_acc[t][3] *= alpha;
+            for (int t = 0; t < Cfg::kColTiles; ++t) {
+                o_acc[r][t][0] *= alpha;
+                o_acc[r][t][1] *= alpha;
+                o_acc[r][t][2] *= alpha;
+                o_acc[r][t][3] *= alpha;
+            }
         }
         // (every column tile interleaves columns of the whole 128-column pass, so none is dead as a whole)
 #pragma unroll
-        for (int t = 0; t < Cfg::kColTiles; ++t) o_acc[t] = mfma16<T>(vt[t], pk, o_acc[t]);
+        for (int t = 0; t < Cfg::kColTiles; ++t)
+#pragma unroll
+            for (int r = 0; r < RT; ++r) o_acc[r][t] = mfma16<T>(vt[t], pk[r], o_acc[r][t]);
         c = cn;
     }
 
     // ---- write.  Register i of column tile t = hh*kVW + w is column hh*128 + (lq*4 + i)*kVW + w
     //      of query row ln: kVW consecutive columns per (hh, i).
-    l_run = quad_rows_sum(l_run);
-    if (row0 + ln < n_rows && ln >= dead_rows(p, b)) {
-        const float inv = (l_run > 0.f) ? 1.f / l_run : 0.f;
-        const int qi = (row0 + ln) / p.group;
-        const int head = kvh * p.group + (row0 + ln - qi * p.group);
-        if (write_final) {
-            uint16_t *dst = reinterpret_cast<uint16_t *>(p.out) + (int64_t)b * p.o_stride_b + (int64_t)qi * p.o_stride_s +
-                            (int64_t)head * p.o_stride_h;
 #pragma unroll
-            for (int hh = 0; hh < Cfg::kVH; ++hh)
+    for (int r = 0; r < RT; ++r) {
+        const float lr = quad_rows_sum(l_run[r]);
+        const int trow = 16 * r + ln;                 // row of the unit
+        if (row0 + trow < n_rows && trow >= dead_rows(p, b)) {
+            const float inv = (lr > 0.f) ? 1.f / lr : 0.f;
+            const int qi = (row0 + trow) / p.group;
+            const int head = kvh * p.group + (row0 + trow - qi * p.group);
+            if (write_final) {
+                uint16_t *dst = reinterpret_cast<uint16_t *>(p.out) + (int64_t)b * p.o_stride_b + (int64_t)qi * p.o_stride_s +
+                                (int64_t)head * p.o_stride_h;
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    if (PART && hh * 128 + (lq * 4 + i) * Cfg::kVW >= hd) continue;
-                    uint16_t *d2 = dst + hh * 128 + (lq * 4 + i) * Cfg::kVW;
+                for (int hh = 0; hh < Cfg::kVH; ++hh)
 #pragma unroll
-                    for (int w = 0; w < Cfg::kVW; w += 2)
-                        *reinterpret_cast<uint32_t *>(d2 + w) =
-                            pack2<T>(o_acc[hh * Cfg::kVW + w][i] * inv, o_acc[hh * Cfg::kVW + w + 1][i] * inv);
-                }
-            if (lq == 0)
-                p.lse[((int64_t)b * p.nheads + head) * Sq + qi] = (l_run > 0.f) ? (m_run + fast_log2(l_run)) * kLn2 : INFINITY;
-        } else {
-            const int64_t srow = slot * p.rows + ln;
-            float *dst = p.o_partial + srow * D;
+                    for (int i = 0; i < 4; ++i) {
+                        if (PART && hh * 128 + (lq * 4 + i) * Cfg::kVW >= hd) continue;
+                        uint16_t *d2 = dst + hh * 128 + (lq * 4 + i) * Cfg::kVW;
 #pragma unroll
-            for (int hh = 0; hh < Cfg::kVH; ++hh)
+                        for (int w = 0; w < Cfg::kVW; w += 2)
+                            *reinterpret_cast<uint32_t *>(d2 + w) =
+                                pack2<T>(o_acc[r][hh * Cfg::kVW + w][i] * inv, o_acc[r][hh * Cfg::kVW + w + 1][i] * inv);
+                    }
+                if (lq == 0)
+                    p.lse[((int64_t)b * p.nheads + head) * Sq + qi] = (lr > 0.f) ? (m_run[r] + fast_log2(lr)) * kLn2 : INFINITY;
+            } else {
+                const int64_t srow = slot * p.rows + trow;
+                float *dst = p.o_partial + srow * D;
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    float *d2 = dst + hh * 128 + (lq * 4 + i) * Cfg::kVW;
+                for (int hh = 0; hh < Cfg::kVH; ++hh)
 #pragma unroll
-                    for (int w = 0; w < Cfg::kVW; w += 2)
-                        *reinterpret_cast<float2 *>(d2 + w) =
-                            make_float2(o_acc[hh * Cfg::kVW + w][i] * inv, o_acc[hh * Cfg::kVW + w + 1][i] * inv);
-                }
-            if (lq == 0) p.lse_partial[srow] = (l_run > 0.f) ? m_run + fast_log2(l_run) : -INFINITY;
+                    for (int i = 0; i < 4; ++i) {
+                        float *d2 = dst + hh * 128 + (lq * 4 + i) * Cfg::kVW;
+#pragma unroll
+                        for (int w = 0; w < Cfg::kVW; w += 2)
+                            *reinterpret_cast<float2 *>(d2 + w) =
+                                make_float2(o_acc[r][hh * Cfg::kVW + w][i] * inv, o_acc[r][hh * Cfg::kVW + w + 1][i] * inv);
+                    }
+                if (lq == 0) p.lse_partial[srow] = (lr > 0.f) ? m_run[r] + fast_log2(lr) : -INFINITY;
+            }
         }
     }
     __builtin_amdgcn_wave_barrier();   // the wave's LDS rows are reused by its next piece
 }
 
-template <typename T, int D, bool SOFTCAP, bool PART>
+template <typename T, int D, bool SOFTCAP, bool PART, int RT>
 __global__ void __launch_bounds__(256, (D <= 128) ? 2 : 1) decode_wave_kernel(const DecodeParams p) {
     using Cfg = WaveCfg<D>;
     __shared__ int s_pref[257];
-    __shared__ __attribute__((aligned(16))) uint8_t s_k[4][Cfg::kTileBytes];
-    __shared__ __attribute__((aligned(16))) uint16_t s_q[4][16 * D];
+    // two K tiles per wave: the chunk being read and the chunk on its way; the second also stages the q rows of a piece
+    __shared__ __attribute__((aligned(16))) uint8_t s_k[4][2 * Cfg::kTileBytes];
     const Partition pt = make_partition(p, s_pref);
     publish_partition(p, pt, s_pref);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     walk_share(p, pt, s_pref, (int64_t)blockIdx.x * 4 + wave,
                [&](int b, int unit, const UnitRange &ur, int range_lo, int range_hi, bool whole, int64_t slot) {
                    int kvh = unit, row0 = 0, n_rows = p.rows;
-                   if (p.row_tiles > 1) {
+                   if (RT == 1 && p.row_tiles > 1) {
                        kvh = unit / p.row_tiles;
                        row0 = (unit - kvh * p.row_tiles) * 16;
                        n_rows = p.rows_total;
                    }
-                   wave_piece<T, D, SOFTCAP, PART>(p, b, kvh, row0, n_rows, ur, range_lo, range_hi, whole, slot, s_k[wave], s_q[wave]);
+                   wave_piece<T, D, SOFTCAP, PART, RT>(p, b, kvh, row0, n_rows, ur, range_lo, range_hi, whole, slot, s_k[wave]);
                });
     init_empty_units<D>(p, pt);
 }
 
-template <typename T, int D> static hipError_t launch_wave_d(const DecodeParams &p, hipStream_t stream) {
+template <typename T, int D, int RT> static hipError_t launch_wave_rt(const DecodeParams &p, hipStream_t stream) {
     dim3 grid(p.num_wgs), block(256);
     if (p.headdim > D || p.headdim < 8 || p.headdim % 8 != 0) return hipErrorInvalidValue;
     const bool part = p.headdim < D;
     if (p.softcap_post != 0.f) {
         if (part)
-            hipLaunchKernelGGL((decode_wave_kernel<T, D, true, true>), grid, block, 0, stream, p);
+            hipLaunchKernelGGL((decode_wave_kernel<T, D, true, true, RT>), grid, block, 0, stream, p);
         else
-            hipLaunchKernelGGL((decode_wave_kernel<T, D, true, false>), grid, block, 0, stream, p);
+            hipLaunchKernelGGL((decode_wave_kernel<T, D, true, false, RT>), grid, block, 0, stream, p);
     } else {
         if (part)
-            hipLaunchKernelGGL((decode_wave_kernel<T, D, false, true>), grid, block, 0, stream, p);
+            hipLaunchKernelGGL((decode_wave_kernel<T, D, false, true, RT>), grid, block, 0, stream, p);
         else
-            hipLaunchKernelGGL((decode_wave_kernel<T, D, false, false>), grid, block, 0, stream, p);
+            hipLaunchKernelGGL((decode_wave_kernel<T, D, false, false, RT>), grid, block, 0, stream, p);
     }
     return hipGetLastError();
+}
+
+// Blocks of up to 16 rows: one tile per wave.  17 .. 32 rows: two tiles per wave where the registers allow it
+// (wave_rows_per_unit(D) = 32); otherwise the host has cut the block into 16-row units (p.row_tiles > 1).
+template <typename T, int D> static hipError_t launch_wave_d(const DecodeParams &p, hipStream_t stream) {
+    if (p.rows > 16) {
+        if constexpr (wave_rows_per_unit(D) >= 32)
+            return launch_wave_rt<T, D, 2>(p, stream);
+        else
+            return hipErrorInvalidValue;
+    }
+    return launch_wave_rt<T, D, 1>(p, stream);
 }
 
 template <typename T> static hipError_t launch_wave_t(const DecodeParams &p, int headdim, hipStream_t stream) {
@@ -495,7 +561,8 @@ template <typename T> static hipError_t launch_wave_t(const DecodeParams &p, int
 }
 
 hipError_t launch_decode_wave(const DecodeParams &p, int dtype, int headdim, hipStream_t stream) {
-    if (p.rows > 16 || !p.balanced || !p.wave_workers || p.num_workers != p.num_wgs * 4) return hipErrorInvalidValue;
+    if (p.rows > wave_rows_per_unit(headdim) || !p.balanced || !p.wave_workers || p.num_workers != p.num_wgs * 4) return hipErrorInvalidValue;
+    if (p.rows > 16 && p.row_tiles > 1) return hipErrorInvalidValue;
     if (p.row_tiles > 1 && (p.rows != 16 || p.k_new != nullptr || p.q_live != nullptr || p.rows_total > 16 * p.row_tiles ||
                             p.nheads_k % p.row_tiles != 0))
         return hipErrorInvalidValue;

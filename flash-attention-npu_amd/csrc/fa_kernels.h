@@ -225,23 +225,27 @@ hipError_t launch_scatter_short_blocks(const ShortBlocksParams &p, hipStream_t s
 // Resident decode workgroups per compute unit for a head dimension / query-block height.
 inline int decode_wgs_per_cu(int headdim, int rows) { return (headdim <= 128 && rows <= 32) ? 2 : 1; }
 
-// Which kernel takes a query block of rows = seqlen_q * group rows (balanced partition), by measurement (64 sequences x
-// 8 K keys unless stated; us of the workgroup-level decode kernel with two row tiles / the wave-level kernel with the
-// block cut into two 16-row units / the tiled kernel with the GQA heads packed into its 128-row tiles):
-//   D = 128, 32 rows: 64q/8kv x 4 tokens 413 / 521 / 391; 32q/8kv x 8 tokens 413 / 522 / 383; MQA 32q/1kv 76 / 79 / 61;
-//            256 ragged sequences of <= 2 K keys 407 / 421 / 302; 4 sequences x 32 K 132 / 141 / 115; 18 rows 409 / 535 / 390
-//   D = 64,  32 rows: 213 / 268 / 232
-//   D = 256, 32 rows: MQA 32q/1kv 254 / 177 / 252; 64q/8kv x 4 tokens x 32 sequences 833 / 596 / 935
-// Up to 16 rows the wave-level kernel is far ahead everywhere; from 33 rows on the tiled kernel is (a four-tile decode
-// variant existed: 64 rows 552 vs 468 us, ragged 256 x 2 K 712 vs 351 us, D = 256 2131 vs 937 us; row tiles as units: 64
-// rows 842 vs 409 us).  In between the tiles of the wave-level kernel read the keys once per tile (the second read
-// comes from the cache hierarchy, but it takes a place among the loads in flight), which pays where the alternatives
-// are weakest, at D = 256.
+// Which kernel takes a query block of rows = seqlen_q * group rows (balanced partition), by measurement with a cold
+// cache (the pools of a step rotated past the 256 MB last-level cache; 64 sequences x 8 K keys, one query token, 32 q
+// heads per kv head; whole call in us, tiled kernel or workgroup-level decode kernel -> wave-level kernel):
+//   D = 128: 8 kv heads (2.1 GB) 789 -> 363 (5.9 TB/s); 1 kv head (268 MB) 116 -> 87
+//   D = 64:  8 kv heads (1.1 GB) 212 -> 195 (5.5 TB/s); 1 kv head (134 MB, mostly resident) 44 -> 50
+//   D = 256: 8 kv heads (4.3 GB) 2901 -> 1051 (4.1 TB/s), the block cut into two 16-row units
+// A stream like this is bounded by the bytes it keeps in flight, and only the wave-level kernel keeps every wave's
+// chunk in flight for all the rows of a block: with two 16-row tiles in one wave (D <= 128, where the registers that
+// used to stage K now hold the second set of accumulators) one pass over the keys serves 32 rows; at D = 256 the
+// tiles are units of their own, i.e. neighbouring waves that read the same keys (the second read comes from the
+// cache hierarchy, but takes a place among the loads in flight).  Up to 16 rows the wave-level kernel is far ahead
+// everywhere; from 33 rows on the tiled kernel is (a four-tile decode variant existed: 64 rows 552 vs 468 us, ragged
+// 256 x 2 K 712 vs 351 us, D = 256 2131 vs 937 us; row tiles as units: 64 rows 842 vs 409 us).
 // Tallest block for the workgroup-level decode kernels (decode_balanced_kernel; decode_paged_kernel for explicit
 // num_splits); kDecodeMaxRows is what those kernels can take at all (two 16-row tiles).
 constexpr int kDecodeMaxRows = 32;
 inline int block_decode_max_rows(int tile_headdim) { return tile_headdim == 64 ? 32 : 16; }
-// Tallest block the wave-level kernel takes, as 16-row tiles that are units of their own.
-inline int wave_max_rows(int tile_headdim) { return tile_headdim == 256 ? 32 : 16; }
+// Rows of a unit of the wave-level kernel: one 16-row tile per wave, or two where the registers of a wave that shares
+// its SIMD with another hold two sets of accumulators (D <= 128).
+constexpr int wave_rows_per_unit(int tile_headdim) { return tile_headdim <= 128 ? 32 : 16; }
+// Tallest block the wave-level kernel takes: a unit's rows, or 16-row tiles that are units of their own (D = 256).
+inline int wave_max_rows(int tile_headdim) { return 32; }
 
 }  // namespace fa

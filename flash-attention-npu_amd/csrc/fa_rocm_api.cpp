@@ -194,9 +194,11 @@ int decode_max_rows(const fa_kvcache_args *a) {
     return wave_level ? std::max(block_level, wave_max_rows(a)) : block_level;
 }
 
-// 16-row tiles of a query block on the wave-level kernel (1: the block is one tile; 0: not that kernel's)
+// Units that a query block is cut into for the wave-level kernel (1: the block is one unit, of one or two 16-row tiles
+// that one wave carries; more: 16-row tiles that are units of their own; 0: not that kernel's)
 int wave_row_tiles(const fa_kvcache_args *a, size_t rows) {
     if (is_mla_i8(a) || env().block_workers || rows > (size_t)wave_max_rows(a)) return 0;
+    if (rows <= (size_t)fa::wave_rows_per_unit(fa::tile_headdim(a->headdim_qk)) && env().wave_max_rows == 0) return 1;
     return (int)((rows + 15) / 16);
 }
 

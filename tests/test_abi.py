@@ -134,14 +134,19 @@ def test_split_plan_invariants():
     assert plan.num_workers == 2048 and plan.min_share == 2            # one 16-row tile: every wave is a worker
     rows = 4
     assert plan.workspace_bytes == 2048 * 2 * rows * (128 + 1) * 4 + 2048 == lib.fa_rocm_kvcache_workspace_bytes(C.byref(a), 256)
-    # 20 rows (two 16-row tiles): which kernel takes them depends on the head dimension
+    # 20 rows (two 16-row tiles): every wave is a worker; how it carries the tiles depends on the head dimension
     a.seqlen_q = 5
-    lib.fa_rocm_plan_kvcache(C.byref(a), 256, C.byref(plan))           # d = 128: the tiled kernel, heads packed
-    assert plan.mode == 0 and plan.num_workers == 0
-    a.headdim_qk = a.headdim_v = 64                                     # d = 64: the workgroup is the worker
+    lib.fa_rocm_plan_kvcache(C.byref(a), 256, C.byref(plan))           # d = 128: both tiles in one wave, 20-row partial slots
+    assert plan.mode == 1 and plan.num_wgs == 512 and plan.num_workers == 2048
+    assert plan.workspace_bytes == 2048 * 2 * 20 * 129 * 4 + 2048
+    a.headdim_qk = a.headdim_v = 64                                     # d = 64: the same
     lib.fa_rocm_plan_kvcache(C.byref(a), 256, C.byref(plan))
-    assert plan.mode == 1 and plan.num_workers == plan.num_wgs == 512 and plan.workspace_bytes == 512 * 2 * 20 * 65 * 4 + 2048
-    a.headdim_qk = a.headdim_v = 256                                    # d = 256: every wave a worker, the tiles are units
+    assert plan.mode == 1 and plan.num_workers == 2048 and plan.workspace_bytes == 2048 * 2 * 20 * 65 * 4 + 2048
+    a.num_splits = 2                                                    # explicit splits: the workgroup-level kernel's grid
+    lib.fa_rocm_plan_kvcache(C.byref(a), 256, C.byref(plan))
+    assert plan.mode == 0 and plan.num_workers == 0
+    a.num_splits = 0
+    a.headdim_qk = a.headdim_v = 256                                    # d = 256: the tiles are units of their own
     lib.fa_rocm_plan_kvcache(C.byref(a), 256, C.byref(plan))
     assert plan.mode == 1 and plan.num_wgs == 256 and plan.num_workers == 1024
     assert plan.workspace_bytes == 1024 * 2 * 16 * 257 * 4 + 2048

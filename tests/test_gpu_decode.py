@@ -235,11 +235,12 @@ def test_decode_two_tile_blocks_on_every_kernel(kernel, d, sq, hq, hk, kw):
     assert torch.equal(dev["v_cache"].cpu().view(torch.int16), vc.view(torch.int16))
 
 
-def test_decode_two_tile_blocks_split_over_many_workers():
-    """One long sequence, 32 rows: every unit is cut over many workers and merged; the wave-level kernel with its
-    16-row units against the other two kernels and the oracle."""
+@pytest.mark.parametrize("d", [256, 128, 64])
+def test_decode_two_tile_blocks_split_over_many_workers(d):
+    """One long sequence, 32 rows: every unit is cut over many workers and merged; the wave-level kernel (two tiles in
+    one wave up to d = 128, 16-row units at d = 256) against the other kernels and the oracle."""
     from helpers import library_env
-    case = make_paged_case(1, 32, 1, 256, 256, [40000], seed=77)
+    case = make_paged_case(1, 32, 1, d, 256, [40000], seed=77)
     outs = {}
     for kernel, env in _TWO_TILE_KERNELS.items():
         with library_env(**env):
