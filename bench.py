@@ -38,7 +38,8 @@ COLD_BYTES = 512 << 20      # bytes the rotated pools of a decode config must ad
 # figure belongs to the kernel as it was when the summary was made; the record names the file it was read from.
 PROFILE_OF = {"c2": "decode_wave_kernel_c2.txt", "c2_8k": "decode_wave_kernel_c2_8k.txt", "c3a": "decode_wave_kernel_c3a.txt", "c3b": "decode_wave_kernel_c3b.txt",
               "c4": "decode_mla_i8_kernel_c4.txt", "c5": "prefill_kernel_c5.txt",
-              "mqa32": "prefill_kernel_mqa32.txt", "mqa32_d256": "decode_wave_kernel_mqa32_d256.txt"}
+              "mqa32": "decode_wave_kernel_mqa32.txt", "mqa32_d256": "decode_wave_kernel_mqa32_d256.txt",
+              "g32k8": "decode_wave_kernel_g32k8.txt"}
 
 
 def traffic_from_profile(name: str):
@@ -123,13 +124,14 @@ def decode_workload(name: str, device, seed: int = 0, kv_layout: str = "nhd"):
         window = (-1, -1) if name == "c3a" else (4095, 0)
         desc = f"long-context split-KV decode bf16 B=4 64q/8kv d=128 Lk=131072 window={window} causal"
     elif name in ("mqa32", "mqa32_d256", "mqa32_d64", "g32k8", "g32k8_d64", "g32k8_d256"):
-        # query blocks of 17..32 rows (one token x 32 q heads of one kv head): past the 16 rows of one decode tile
+        # query blocks of 17..32 rows (one token x 32 q heads of one kv head): past the 16 rows of one decode tile;
+        # mqa32*: one kv head; g32k8*: eight kv heads of 32 q heads each; the suffix _d<n> sets the head dimension
         B, hq, hk, d = 64, 32, 1, (128 if name in ("mqa32", "g32k8") else int(name[7:]))
         if name.startswith("g32k8"):
             hq, hk = 256, 8
         lens = torch.full((B,), 8192)
         snew, rotary, window, spare = 0, False, (-1, -1), 16
-        desc = f"multi-query paged decode bf16 B=64 32q/1kv d={d} page=256 all rows 8192 keys causal (32-row query blocks)"
+        desc = f"paged decode bf16 B=64 {hq}q/{hk}kv d={d} page=256 all rows 8192 keys causal (32-row query blocks)"
     else:
         raise ValueError(name)
     pages = [math.ceil((int(l) + snew) / page) for l in lens]

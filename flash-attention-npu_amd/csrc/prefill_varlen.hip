@@ -280,45 +280,57 @@ __device__ __forceinline__ void prefill_block(const PrefillParams &p, const unsi
     auto tiles_landed = [&]() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); };
     auto fetch_tile = [&](int kt, int buf) {
         const uint32_t k_lds = lds_of(&s_k[buf][0]) + (uint32_t)wave * 1024u, v_lds = lds_of(&s_v[buf][0]) + (uint32_t)wave * 1024u;
-        if constexpr (!PAGED) {
-            if (kt * kBN + kBN <= Sk) {
-                const uint8_t *kb = reinterpret_cast<const uint8_t *>(kbase) + (int64_t)(k0 + kt * kBN) * p.k_stride_t * 2;
-                const uint8_t *vb = reinterpret_cast<const uint8_t *>(vbase) + (int64_t)(k0 + kt * kBN) * p.v_stride_t * 2;
-#pragma unroll
-                for (int i = 0; i < Cfg::kKLoads; ++i)
-                    if (k_on[i]) load_lds_base(k_lds + i * 4096u, k_off[i], kb);
-#pragma unroll
-                for (int i = 0; i < Cfg::kVLoads; ++i)
-                    if (v_on[i]) load_lds_base(v_lds + i * 4096u, v_off[i], vb);
-                return;
+        // A tile inside the sequence, of dense K/V or inside one page: one wave-uniform base serves all its loads
+        if (kt * kBN + kBN <= Sk && (!PAGED || p.page_size % kBN == 0)) {
+            int64_t koff, voff;
+            if constexpr (PAGED) {
+                const int page = (kt * kBN) / p.page_size;
+                const int blk = min(max(__builtin_amdgcn_readfirstlane(bt_row[page]), 0), p.num_blocks - 1);
+                const int inpage = kt * kBN - page * p.page_size;
+                koff = (int64_t)blk * p.k_stride_block + (int64_t)inpage * p.k_stride_t;
+                voff = (int64_t)blk * p.v_stride_block + (int64_t)inpage * p.v_stride_t;
+            } else {
+                koff = (int64_t)(k0 + kt * kBN) * p.k_stride_t;
+                voff = (int64_t)(k0 + kt * kBN) * p.v_stride_t;
             }
+            const uint8_t *kb = reinterpret_cast<const uint8_t *>(kbase + koff);
+            const uint8_t *vb = reinterpret_cast<const uint8_t *>(vbase + voff);
+#pragma unroll
+            for (int i = 0; i < Cfg::kKLoads; ++i)
+                if (k_on[i]) load_lds_base(k_lds + i * 4096u, k_off[i], kb);
+#pragma unroll
+            for (int i = 0; i < Cfg::kVLoads; ++i)
+                if (v_on[i]) load_lds_base(v_lds + i * 4096u, v_off[i], vb);
+            return;
         }
-        auto row_offsets = [&](int row, int64_t &koff, int64_t &voff) {
+        // The ragged end of a sequence, or pages that a tile straddles: an address per row.  All addresses first (their
+        // page-table entries are then fetched together), the loads behind them.
+        auto row_addr = [&](int row, bool is_k) -> const uint8_t * {
             const int key = min(kt * kBN + row, Sk - 1);
+            int64_t off;
             if constexpr (PAGED) {
                 const int page = key / p.page_size;
                 int blk = bt_row[page];
                 blk = min(max(blk, 0), p.num_blocks - 1);
                 const int inpage = key - page * p.page_size;
-                koff = (int64_t)blk * p.k_stride_block + (int64_t)inpage * p.k_stride_t;
-                voff = (int64_t)blk * p.v_stride_block + (int64_t)inpage * p.v_stride_t;
+                off = is_k ? (int64_t)blk * p.k_stride_block + (int64_t)inpage * p.k_stride_t
+                           : (int64_t)blk * p.v_stride_block + (int64_t)inpage * p.v_stride_t;
             } else {
-                koff = (int64_t)(k0 + key) * p.k_stride_t;
-                voff = (int64_t)(k0 + key) * p.v_stride_t;
+                off = (int64_t)(k0 + key) * (is_k ? p.k_stride_t : p.v_stride_t);
             }
+            return reinterpret_cast<const uint8_t *>((is_k ? kbase : vbase) + off);
         };
+        const uint8_t *ka[Cfg::kKLoads], *va[Cfg::kVLoads];
 #pragma unroll
-        for (int i = 0; i < Cfg::kKLoads; ++i) {
-            int64_t koff, voff;
-            row_offsets(k_row[i], koff, voff);
-            if (k_on[i]) load_lds_addr(k_lds + i * 4096u, reinterpret_cast<const uint8_t *>(kbase + koff) + k_col[i]);
-        }
+        for (int i = 0; i < Cfg::kKLoads; ++i) ka[i] = row_addr(k_row[i], true) + k_col[i];
 #pragma unroll
-        for (int i = 0; i < Cfg::kVLoads; ++i) {
-            int64_t koff, voff;
-            row_offsets(v_row[i], koff, voff);
-            if (v_on[i]) load_lds_addr(v_lds + i * 4096u, reinterpret_cast<const uint8_t *>(vbase + voff) + v_col[i]);
-        }
+        for (int i = 0; i < Cfg::kVLoads; ++i) va[i] = row_addr(v_row[i], false) + v_col[i];
+#pragma unroll
+        for (int i = 0; i < Cfg::kKLoads; ++i)
+            if (k_on[i]) load_lds_addr(k_lds + i * 4096u, ka[i]);
+#pragma unroll
+        for (int i = 0; i < Cfg::kVLoads; ++i)
+            if (v_on[i]) load_lds_addr(v_lds + i * 4096u, va[i]);
     };
     if constexpr (PART) {
         // the places of the pieces that nobody loads
