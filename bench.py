@@ -38,7 +38,7 @@ COLD_BYTES = 512 << 20      # bytes the rotated pools of a decode config must ad
 # figure belongs to the kernel as it was when the summary was made; the record names the file it was read from.
 PROFILE_OF = {"c2": "decode_wave_kernel_c2.txt", "c2_8k": "decode_wave_kernel_c2_8k.txt", "c3a": "decode_wave_kernel_c3a.txt", "c3b": "decode_wave_kernel_c3b.txt",
               "c4": "decode_mla_i8_kernel_c4.txt", "c5": "prefill_kernel_c5.txt",
-              "mqa32": "decode_wave_kernel_mqa32.txt", "mqa32_d256": "decode_wave_kernel_mqa32_d256.txt",
+              "mqa32": "prefill_kernel_mqa32.txt", "mqa32_d256": "prefill_kernel_mqa32_d256.txt",
               "g32k8": "decode_wave_kernel_g32k8.txt"}
 
 
@@ -123,12 +123,17 @@ def decode_workload(name: str, device, seed: int = 0, kv_layout: str = "nhd"):
         snew, rotary, spare = 0, False, 0
         window = (-1, -1) if name == "c3a" else (4095, 0)
         desc = f"long-context split-KV decode bf16 B=4 64q/8kv d=128 Lk=131072 window={window} causal"
-    elif name in ("mqa32", "mqa32_d256", "mqa32_d64", "g32k8", "g32k8_d64", "g32k8_d256"):
+    elif name in ("mqa32", "mqa32_d256", "mqa32_d64", "g32k8", "g32k8_d64", "g32k8_d256", "g64k8", "g48k8", "g32k4", "g32k2"):
         # query blocks of 17..32 rows (one token x 32 q heads of one kv head): past the 16 rows of one decode tile;
         # mqa32*: one kv head; g32k8*: eight kv heads of 32 q heads each; the suffix _d<n> sets the head dimension
-        B, hq, hk, d = 64, 32, 1, (128 if name in ("mqa32", "g32k8") else int(name[7:]))
+        B, hq, hk, d = 64, 32, 1, (128 if name in ("mqa32", "g32k8", "g64k8", "g48k8", "g32k4", "g32k2") else int(name[7:]))
+        if name in ("g32k4", "g32k2"):
+            hk = int(name[4:])
+            hq = 32 * hk
         if name.startswith("g32k8"):
             hq, hk = 256, 8
+        if name in ("g64k8", "g48k8"):
+            hq, hk = 8 * int(name[1:3]), 8
         lens = torch.full((B,), 8192)
         snew, rotary, window, spare = 0, False, (-1, -1), 16
         desc = f"paged decode bf16 B=64 {hq}q/{hk}kv d={d} page=256 all rows 8192 keys causal (32-row query blocks)"
@@ -329,7 +334,7 @@ def run_decode(args, name, cpu_budget=(20.0, 10.0)):
 
     if name == "c4":
         kernel_name = "decode_mla_i8_kernel"
-    elif plan.mode != 1 and w["hq"] // w["hk"] > 16 and w["d"] >= 128:
+    elif plan.mode != 1 and w["hq"] // w["hk"] > 16:
         kernel_name = "prefill_kernel"        # a query block too tall for the decode kernels of this head dimension: the tiled forward
     elif plan.mode == 1:
         kernel_name = "decode_wave_kernel" if plan.num_workers > plan.num_wgs else "decode_balanced_kernel"
@@ -574,7 +579,7 @@ def main():
             subs[name] = sub_record(r)
         subs["c5"] = sub_record(run_prefill(args, cpu_budget_s=3.0))
         out["configs"] = subs
-    elif args.config in ("c2", "c2_8k", "c3a", "c3b", "c4", "mqa32", "mqa32_d256", "mqa32_d64", "g32k8", "g32k8_d64", "g32k8_d256") or args.config.startswith("c2_u"):
+    elif args.config in ("c2", "c2_8k", "c3a", "c3b", "c4", "mqa32", "mqa32_d256", "mqa32_d64", "g32k8", "g32k8_d64", "g32k8_d256", "g64k8", "g48k8", "g32k4", "g32k2") or args.config.startswith("c2_u"):
         out = run_decode(args, args.config)
     elif args.config == "c5":
         out = run_prefill(args)

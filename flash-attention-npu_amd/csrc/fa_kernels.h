@@ -227,17 +227,19 @@ inline int decode_wgs_per_cu(int headdim, int rows) { return (headdim <= 128 && 
 
 // Which kernel takes a query block of rows = seqlen_q * group rows (balanced partition), by measurement with a cold
 // cache (the pools of a step rotated past the 256 MB last-level cache; 64 sequences x 8 K keys, one query token, 32 q
-// heads per kv head; whole call in us, tiled kernel or workgroup-level decode kernel -> wave-level kernel):
-//   D = 128: 8 kv heads (2.1 GB) 789 -> 363 (5.9 TB/s); 1 kv head (268 MB) 116 -> 87
-//   D = 64:  8 kv heads (1.1 GB) 212 -> 195 (5.5 TB/s); 1 kv head (134 MB, mostly resident) 44 -> 50
-//   D = 256: 8 kv heads (4.3 GB) 2901 -> 1051 (4.1 TB/s), the block cut into two 16-row units
-// A stream like this is bounded by the bytes it keeps in flight, and only the wave-level kernel keeps every wave's
-// chunk in flight for all the rows of a block: with two 16-row tiles in one wave (D <= 128, where the registers that
-// used to stage K now hold the second set of accumulators) one pass over the keys serves 32 rows; at D = 256 the
-// tiles are units of their own, i.e. neighbouring waves that read the same keys (the second read comes from the
-// cache hierarchy, but takes a place among the loads in flight).  Up to 16 rows the wave-level kernel is far ahead
-// everywhere; from 33 rows on the tiled kernel is (a four-tile decode variant existed: 64 rows 552 vs 468 us, ragged
-// 256 x 2 K 712 vs 351 us, D = 256 2131 vs 937 us; row tiles as units: 64 rows 842 vs 409 us).
+// heads per kv head; whole call in us: wave-level kernel / tiled kernel, both filling their LDS tiles straight from
+// global memory):
+//   D = 128: 8 kv heads (2.1 GB) 364 (5.9 TB/s) / 392; 4 kv heads 204 / 217; 2 kv heads 127 / 113; 1 kv head 87 / 66
+//   D = 64:  8 kv heads (1.1 GB) 193 (5.6 TB/s) / workgroup-level decode kernel 212; 1 kv head (134 MB) 50 / 44
+//   D = 256: 8 kv heads (4.3 GB), the block as two 16-row units of the wave-level kernel 1050 / tiled 830 (5.2 TB/s)
+// A stream like this is bounded by the bytes it keeps in flight, and the wave-level kernel keeps every wave's chunk in
+// flight for all the rows of a block: with two 16-row tiles in one wave (D <= 128, where the registers that used to
+// stage K hold the second set of accumulators) one pass over the keys serves 32 rows.  That pays when the units are
+// cut into few pieces (at least as many units as compute units: the host's rule, wave_max_rows() in fa_rocm_api.cpp);
+// cut 16 or 32 ways, the fixed costs of the pieces and their merge outweigh it.  At D = 256 the accumulators of two
+// tiles do not fit a wave, and tiles as units of their own read the keys twice (1.7 x the traffic).  Up to 16 rows the
+// wave-level kernel is far ahead everywhere; from 33 rows on the tiled kernel runs (64 rows x 8 kv heads: 418 us,
+// 5.2 TB/s).
 // Tallest block for the workgroup-level decode kernels (decode_balanced_kernel; decode_paged_kernel for explicit
 // num_splits); kDecodeMaxRows is what those kernels can take at all (two 16-row tiles).
 constexpr int kDecodeMaxRows = 32;
@@ -245,7 +247,6 @@ inline int block_decode_max_rows(int tile_headdim) { return tile_headdim == 64 ?
 // Rows of a unit of the wave-level kernel: one 16-row tile per wave, or two where the registers of a wave that shares
 // its SIMD with another hold two sets of accumulators (D <= 128).
 constexpr int wave_rows_per_unit(int tile_headdim) { return tile_headdim <= 128 ? 32 : 16; }
-// Tallest block the wave-level kernel takes: a unit's rows, or 16-row tiles that are units of their own (D = 256).
-inline int wave_max_rows(int tile_headdim) { return 32; }
+
 
 }  // namespace fa

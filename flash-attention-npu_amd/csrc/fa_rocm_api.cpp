@@ -65,6 +65,7 @@ size_t partial_row_bytes(const fa_kvcache_args *a) {
 struct EnvKnobs {
     int decode_max_rows = 0;       // FA_ROCM_DECODE_MAX_ROWS: 16 or 32, else the built-in rule
     int wave_max_rows = 0;         // FA_ROCM_WAVE_MAX_ROWS: 16, 32, 48 or 64: tallest block cut into 16-row tiles for the wave-level kernel
+    int wave_two_tiles = 0;        // FA_ROCM_WAVE_TWO_TILES=1: 17-32-row blocks as two tiles in one wave whatever the number of units
     int decode_wgs = 0;            // FA_ROCM_DECODE_WGS: workgroups of the balanced partition
     bool block_workers = false;    // FA_ROCM_DECODE_BLOCK_WORKERS
     int min_share = 0;             // FA_ROCM_MIN_SHARE
@@ -87,6 +88,7 @@ void load_env() {
     };
     e.decode_max_rows = num("FA_ROCM_DECODE_MAX_ROWS", 0);
     e.wave_max_rows = num("FA_ROCM_WAVE_MAX_ROWS", 0);
+    e.wave_two_tiles = num("FA_ROCM_WAVE_TWO_TILES", 0);
     e.decode_wgs = num("FA_ROCM_DECODE_WGS", 0);
     e.block_workers = flag("FA_ROCM_DECODE_BLOCK_WORKERS");
     e.min_share = num("FA_ROCM_MIN_SHARE", 0);
@@ -177,27 +179,36 @@ size_t tall_q_bytes(const fa_kvcache_args *a) {
     return (n + 255) / 256 * 256;
 }
 
-// Tallest query block (rows = seqlen_q * group) that the wave-level kernel takes, cut into 16-row tiles that are units
-// of their own (fa::kWaveMaxRows; FA_ROCM_WAVE_MAX_ROWS = 16, 32, 48 or 64 overrides it for experiments).
-int wave_max_rows(const fa_kvcache_args *a) {
+// Tallest query block (rows = seqlen_q * group) that the wave-level kernel takes.  Blocks of 17-32 rows run there as
+// two 16-row tiles in one wave (fa::wave_rows_per_unit) when the call has at least as many units (batch rows x kv
+// heads) as the device has compute units: then a unit is cut into few pieces and the stream is bounded by the bytes
+// in flight, which that kernel keeps highest; with fewer units the fixed costs of the many pieces and their merge
+// weigh more than that, and the tiled kernel (or, at d = 64, the workgroup-level decode kernel) is ahead (measured at
+// 64 sequences x 8 K keys, d = 128, whole call, wave-level / tiled: 8 kv heads 364 / 392 us, 4 heads 204 / 217,
+// 2 heads 127 / 113, 1 head 87 / 66).  FA_ROCM_WAVE_MAX_ROWS = 16, 32, 48 or 64 overrides the rule for experiments: the
+// block is then cut into 16-row tiles that are units of their own; FA_ROCM_WAVE_TWO_TILES = 1 drops the unit count from
+// the rule (tests).
+int wave_max_rows(const fa_kvcache_args *a, int num_cus) {
     const int v = env().wave_max_rows;
-    return (v == 16 || v == 32 || v == 48 || v == 64) ? v : fa::wave_max_rows(fa::tile_headdim(a->headdim_qk));
+    if (v == 16 || v == 32 || v == 48 || v == 64) return v;
+    const int per_unit = fa::wave_rows_per_unit(fa::tile_headdim(a->headdim_qk));
+    return (per_unit > 16 && ((int64_t)a->batch * a->nheads_k >= num_cus || env().wave_two_tiles > 0)) ? per_unit : 16;
 }
 
 // Tallest query block (rows = seqlen_q * group) that runs on the decode kernels: the workgroup-level ones up to
 // fa::block_decode_max_rows (FA_ROCM_DECODE_MAX_ROWS = 16 or 32 overrides it), the wave-level one, which runs the
 // balanced partition only, up to wave_max_rows().
-int decode_max_rows(const fa_kvcache_args *a) {
+int decode_max_rows(const fa_kvcache_args *a, int num_cus) {
     const int v = env().decode_max_rows;
     const int block_level = (v == 16 || v == 32) ? v : fa::block_decode_max_rows(fa::tile_headdim(a->headdim_qk));
     const bool wave_level = a->num_splits == 0 && !is_mla_i8(a) && !env().block_workers;
-    return wave_level ? std::max(block_level, wave_max_rows(a)) : block_level;
+    return wave_level ? std::max(block_level, wave_max_rows(a, num_cus)) : block_level;
 }
 
 // Units that a query block is cut into for the wave-level kernel (1: the block is one unit, of one or two 16-row tiles
 // that one wave carries; more: 16-row tiles that are units of their own; 0: not that kernel's)
-int wave_row_tiles(const fa_kvcache_args *a, size_t rows) {
-    if (is_mla_i8(a) || env().block_workers || rows > (size_t)wave_max_rows(a)) return 0;
+int wave_row_tiles(const fa_kvcache_args *a, size_t rows, int num_cus) {
+    if (is_mla_i8(a) || env().block_workers || rows > (size_t)wave_max_rows(a, num_cus)) return 0;
     if (rows <= (size_t)fa::wave_rows_per_unit(fa::tile_headdim(a->headdim_qk)) && env().wave_max_rows == 0) return 1;
     return (int)((rows + 15) / 16);
 }
@@ -324,7 +335,7 @@ int fa_rocm_plan_kvcache(const fa_kvcache_args *a, int num_cus, fa_split_plan *p
     // the int8 latent kernel works on units of 128 query heads and always uses the balanced partition
     const size_t rows = is_mla_i8(a) ? 128 : (size_t)a->seqlen_q * group;
     size_t slot_bytes = rows * partial_row_bytes(a);
-    if (!is_mla_i8(a) && rows > (size_t)decode_max_rows(a)) {
+    if (!is_mla_i8(a) && rows > (size_t)decode_max_rows(a, num_cus)) {
         // Query block too tall for the decode kernels: the tiled forward.  When its tiles alone
         // cannot fill the device (few sequences, short blocks) the keys of every unit are cut into
         // ranges as well; the range length is sized on the device from the longest sequence, so only
@@ -355,7 +366,7 @@ int fa_rocm_plan_kvcache(const fa_kvcache_args *a, int num_cus, fa_split_plan *p
         // Query blocks of up to wave_max_rows() rows: every wave is a worker with its own contiguous share (no
         // workgroup barrier anywhere in the stream), blocks of more than 16 rows as 16-row tiles that are units of
         // their own; taller blocks and the latent kernel: the workgroup is the worker.
-        const int tiles = wave_row_tiles(a, rows);
+        const int tiles = wave_row_tiles(a, rows, num_cus);
         const bool wave_workers = tiles >= 1;
         if (tiles > 1) slot_bytes = 16 * partial_row_bytes(a);
         const int per_cu = is_mla_i8(a) ? 1 : fa::decode_wgs_per_cu(a->headdim_qk, wave_workers ? 16 : (int)rows);
@@ -480,10 +491,10 @@ static int fwd_kvcache_impl(const fa_kvcache_args *a, void *stream_, void *const
 
     const bool local = a->window_left >= 0 || a->window_right >= 0;
 
-    if (!is_mla_i8(a) && rows > decode_max_rows(a)) {
+    int cus_t = device_cus();
+    if (cus_t <= 0) cus_t = 256;
+    if (!is_mla_i8(a) && rows > decode_max_rows(a, cus_t)) {
         // query block too tall for the decode kernel: tiled forward over the paged cache
-        int cus_t = device_cus();
-        if (cus_t <= 0) cus_t = 256;
         fa_split_plan tplan;
         rc = fa_rocm_plan_kvcache(a, cus_t, &tplan);
         if (rc != FA_OK) return rc;
@@ -688,7 +699,7 @@ static int fwd_kvcache_impl(const fa_kvcache_args *a, void *stream_, void *const
     // charging 1-3 chunks measured within +-1 %, so it is not charged.
     p.piece_cost = is_mla_i8(a) ? 7 : 0;
     if (env().piece_cost >= 0) p.piece_cost = env().piece_cost;
-    const int row_tiles = p.wave_workers ? wave_row_tiles(a, rows) : 0;
+    const int row_tiles = p.wave_workers ? wave_row_tiles(a, rows, cus) : 0;
     if (row_tiles > 1) {
         // (kv head, 16-row tile) units: the tiles of a kv head are neighbouring units
         p.row_tiles = row_tiles;

@@ -146,10 +146,16 @@ def test_split_plan_invariants():
     lib.fa_rocm_plan_kvcache(C.byref(a), 256, C.byref(plan))
     assert plan.mode == 0 and plan.num_workers == 0
     a.num_splits = 0
-    a.headdim_qk = a.headdim_v = 256                                    # d = 256: the tiles are units of their own
+    a.headdim_qk = a.headdim_v = 256                                    # d = 256: two tiles do not fit a wave: the tiled kernel
     lib.fa_rocm_plan_kvcache(C.byref(a), 256, C.byref(plan))
-    assert plan.mode == 1 and plan.num_wgs == 256 and plan.num_workers == 1024
-    assert plan.workspace_bytes == 1024 * 2 * 16 * 257 * 4 + 2048
+    assert plan.mode == 0 and plan.num_workers == 0
+    a.headdim_qk = a.headdim_v = 128
+    a.batch = 16                                                        # fewer units (16 x 8) than compute units: the tiled kernel
+    lib.fa_rocm_plan_kvcache(C.byref(a), 256, C.byref(plan))
+    assert plan.mode == 0 and plan.num_workers == 0
+    lib.fa_rocm_plan_kvcache(C.byref(a), 128, C.byref(plan))            # ... on a device of 128 compute units they fill it
+    assert plan.mode == 1 and plan.num_workers == 128 * 2 * 4
+    a.batch = 64
     a.headdim_qk = a.headdim_v = 128
     a.seqlen_q = 1
     a.num_splits = 1

@@ -207,6 +207,7 @@ def test_decode_batch_larger_than_prefix_segments(B, num_splits):
 # experiment settings force each of them in turn so that none goes untested whatever the rule is.
 _TWO_TILE_KERNELS = {
     "rule": {},
+    "wave-level, two tiles in a wave": dict(FA_ROCM_WAVE_TWO_TILES=1),
     "wave-level, tiles as units": dict(FA_ROCM_WAVE_MAX_ROWS=32),
     "workgroup-level, two tiles": dict(FA_ROCM_WAVE_MAX_ROWS=16, FA_ROCM_DECODE_MAX_ROWS=32),
     "tiled, heads packed": dict(FA_ROCM_WAVE_MAX_ROWS=16, FA_ROCM_DECODE_MAX_ROWS=16),

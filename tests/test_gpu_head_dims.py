@@ -54,6 +54,17 @@ def test_wave_decode(d):
     run_kvcache(d, 3, 0, causal=False, dtype=torch.float16, seed=1)
 
 
+@pytest.mark.parametrize("d", [d for d in DIMS if d <= 128])
+def test_wave_decode_with_two_tiles_in_a_wave(d):
+    """28 and 24 rows as two 16-row tiles carried by one wave (the rule takes that path when the call has at least as
+    many units as the device has compute units; the knob takes it for these small cases)."""
+    from helpers import library_env
+    print("head dim: wave decode, two tiles", d, flush=True)
+    with library_env(FA_ROCM_WAVE_TWO_TILES=1):
+        run_kvcache(d, 7, 2, causal=True, nan_other_head=True)
+        run_kvcache(d, 6, 0, causal=False, window_size=(300, 10), dtype=torch.float16, seed=5)
+
+
 @pytest.mark.parametrize("d", DIMS)
 def test_block_decode_and_fixed_splits(d):
     print("head dim: block decode", d, flush=True)
