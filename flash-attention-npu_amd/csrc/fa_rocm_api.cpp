@@ -50,6 +50,7 @@ int device_cus() {
 }
 
 bool is_mla_i8(const fa_kvcache_args *a) { return a->kv_dtype == FA_INT8; }
+bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 // columns of a row of fp32 partials: the width the kernels are compiled for
 int partial_width(const fa_kvcache_args *a) { return is_mla_i8(a) ? a->headdim_v : fa::tile_headdim(a->headdim_v); }
@@ -308,6 +309,10 @@ int fa_rocm_kvcache_validate(const fa_kvcache_args *a) {
         if (!is_mla_i8(a)) return fail(FA_ERR_SHAPE, "tensor strides must be multiples of 8 elements (16 bytes)");
     if ((int64_t)a->page_size * a->k_stride_row * 2 >= (1ll << 31) || (int64_t)a->page_size * a->v_stride_row * 2 >= (1ll << 31))
         return fail(FA_ERR_SHAPE, "a cache page must span less than 2 GiB");
+    // every row is moved 16 bytes at a time (K/V rows straight into LDS)
+    if (!aligned16(a->q) || !aligned16(a->out) || !aligned16(a->k_cache) || !aligned16(a->v_cache) || !aligned16(a->k_new) ||
+        !aligned16(a->v_new))
+        return fail(FA_ERR_SHAPE, "tensor data must be 16-byte aligned");
     return FA_OK;
 }
 
@@ -319,7 +324,8 @@ int fa_rocm_plan_kvcache(const fa_kvcache_args *a, int num_cus, fa_split_plan *p
         // The plan is defined for exactly the shapes the call accepts.  A caller that only plans may leave the tensor
         // pointers NULL: they are stood in for here, so that the dimension checks of the validator decide alone.
         fa_kvcache_args c = *a;
-        void *const some = &c;
+        alignas(16) static char placeholder[16];
+        void *const some = placeholder;
         if (!c.q) c.q = some;
         if (!c.out) c.out = some;
         if (!c.softmax_lse) c.softmax_lse = static_cast<float *>(some);
@@ -843,6 +849,8 @@ int fa_rocm_varlen_validate(const fa_varlen_args *a) {
     if (a->q_stride_t % 8 || a->q_stride_h % 8 || a->k_stride_t % 8 || a->k_stride_h % 8 || a->v_stride_t % 8 ||
         a->v_stride_h % 8 || a->o_stride_t % 8 || a->o_stride_h % 8)
         return fail(FA_ERR_SHAPE, "tensor strides must be multiples of 8 elements (16 bytes)");
+    if (!aligned16(a->q) || !aligned16(a->k) || !aligned16(a->v) || !aligned16(a->out))
+        return fail(FA_ERR_SHAPE, "tensor data must be 16-byte aligned");
     return FA_OK;
 }
 

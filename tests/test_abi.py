@@ -98,6 +98,8 @@ def test_grid_extent_limits_are_rejected_with_a_message():
     expect_error(a, "batch size must be at most 65535")
     a = good_args(); a.nheads = a.nheads_k = 65536
     expect_error(a, "too many units per batch row")
+    a = good_args(); a.k_cache = 0x1008
+    expect_error(a, "tensor data must be 16-byte aligned")
     plan = _lib.SplitPlan()
     a = good_args(); a.batch = 1 << 20
     assert lib.fa_rocm_plan_kvcache(C.byref(a), 256, C.byref(plan)) == -3     # the planner accepts what the call accepts
