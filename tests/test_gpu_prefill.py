@@ -379,3 +379,21 @@ def test_varlen_paged_small_mixed_batch():
     torch.cuda.synchronize()
     ref, ref_lse = O.flash_attn_varlen(q, kl, vl, cu_q, cu_k, max(lens_q), max(lens_k), causal=True, mode="fp32")
     check_paged(out, ref, lse, ref_lse, "small mixed batch")
+
+
+@pytest.mark.parametrize("page", [32, 96, 160])
+@pytest.mark.parametrize("d,dtype", [(128, torch.bfloat16), (64, torch.float16), (256, torch.bfloat16)])
+def test_tall_query_block_over_pages_that_a_tile_straddles(page, d, dtype):
+    """Pages that are no multiple of the 64-key tile: a tile then lies in two or three pages and every row of it takes
+    its own page-table entry (the path of the ragged end of a sequence); pages of 64 keys and more give a whole tile
+    one base address.  Lengths that end inside a tile, on a tile and on a page."""
+    from flash_attn_npu import flash_attn_with_kvcache
+    lens = [5 * page + 7, 64, page, 1000]
+    case = make_paged_case(len(lens), 8, 2, d, page, lens, seqlen_q=40, seqlen_new=0, dtype=dtype, seed=60 + page)
+    dev = to_dev(case)
+    out, lse = flash_attn_with_kvcache(dev["q"], dev["k_cache"], dev["v_cache"], cache_seqlens=dev["cache_seqlens"],
+                                       block_table=dev["block_table"], causal=True, return_softmax_lse=True)
+    torch.cuda.synchronize()
+    ref, ref_lse = O.flash_attn_with_kvcache(case["q"], case["k_cache"], case["v_cache"], cache_seqlens=case["cache_seqlens"],
+                                             block_table=case["block_table"], causal=True, mode="fp32")
+    check_out(out, ref, lse, ref_lse, f"page {page} d {d}")
