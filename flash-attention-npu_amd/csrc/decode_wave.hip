@@ -316,6 +316,8 @@ __device__ __forceinline__ void wave_piece(const DecodeParams &p, const int b, c
     for (int r = 0; r < RT; ++r)
 #pragma unroll
         for (int t = 0; t < Cfg::kKSteps; ++t) qreg[r][t] = *reinterpret_cast<const u32x4_t *>(&sq[(r * 16 + ln) * D + t * 32 + lq * 8]);
+    // the q rows have left the second tile before the first load into it is issued
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 
     if constexpr (PART) {
         // the places of the K pieces that nobody loads hold zeros (the q rows lay elsewhere in this tile)
