@@ -7,10 +7,13 @@ A step is one call of the hot path (append + rotary + attention + split combine 
 configs, one varlen forward for c5) on synthetic inputs that are resident in HBM before the
 timed region.  Several input sets (distinct physical pools) are rotated so that no step finds its K/V in the
 256 MB last-level cache: as many as it takes for one rotation to read 512 MB.  Prints ONE JSON line: whole-call throughput (`value`, K steps between two device
-synchronisations), the median of the per-step durations taken with HIP events, the roofline record of
+synchronisations after W untimed ones; without --warmup, at least 10 calls and at least 0.1 s of them, which is
+what the device's clocks take to settle), the median of the per-call durations taken with HIP events in the same
+pass (an event every K/10 calls for the decode configs, where one between every two calls would cost each call
+≈ 3 µs), the roofline record of
 the dominant kernel (its duration measured with HIP events the library records around it on the
 launch stream) and the CPU golden path timed on the host cores of this box.  The default (`all`) is
-the headline config c2 plus a `configs` object with the same measurements, on the same K and W, for
+the headline config c2 plus a `configs` object with the same measurements, on the same K, for
 every other configuration of the baseline (c2_8k, c3a, c3b, c4, c5), each with a short CPU sample.
 """
 from __future__ import annotations
@@ -279,6 +282,33 @@ def cpu_decode_baseline(w, budget_s: float = 20.0, min_s: float = 10.0):
                 ms_per_call_extrapolated=secs / rows_done * B * 1e3)
 
 
+# ----------------------------------------------------------------------------- warm-up
+WARM_SECONDS = 0.1
+
+
+def warm_up(args, run_one) -> int:
+    """The untimed calls in front of a timed pass; returns how many were made.
+
+    --warmup W makes exactly W.  Without it: at least 10 calls and at least WARM_SECONDS of them.  The device needs
+    tens of milliseconds of work before its clocks have settled, and a matrix-bound call of 0.1 ms feels that: timed
+    after 10 / 100 / 400 untimed calls, the latent decode config takes 130 / 121 / 111 us per call and its kernel
+    105 / 104 / 98 us, where the memory-bound configs move by less than 1 %."""
+    import torch
+    if args.warmup is not None:
+        for i in range(args.warmup):
+            run_one(i)
+        torch.cuda.synchronize()
+        return args.warmup
+    n, t0 = 0, time.perf_counter()
+    while n < 10 or time.perf_counter() - t0 < WARM_SECONDS:
+        run_one(n)
+        n += 1
+        if n % 8 == 0:
+            torch.cuda.synchronize()   # the queue stays short, so the wall clock follows the device
+    torch.cuda.synchronize()
+    return n
+
+
 # ----------------------------------------------------------------------------- main
 def run_decode(args, name, cpu_budget=(20.0, 10.0)):
     import torch
@@ -295,22 +325,26 @@ def run_decode(args, name, cpu_budget=(20.0, 10.0)):
     calls = [bind_decode(w, args.num_splits) for w in sets]
     w = sets[0]
 
-    for i in range(args.warmup):
-        calls[i % npools].run()
-    torch.cuda.synchronize()
-    # the timed pass: K calls between two device synchronisations, with one event on the launch stream between
-    # consecutive calls, so that the wall mean and the per-call median describe the same launches
+    warmup = warm_up(args, lambda i: calls[i % npools].run())
+    # the timed pass: K calls between two device synchronisations, with an event on the launch stream after every
+    # `every`-th call, so that the wall mean and the median (of the groups' per-call durations) describe the same
+    # launches.  An event between every two calls would cost each call 2.5-3 us (c2 204.7 -> 201.9 us, c3b 29.6 ->
+    # 27.0 us, the same box with the marks 1 and 10 calls apart; no marks at all: 201.3 and 26.9 us): the kernel
+    # behind a mark starts only when the one in front has drained, which no caller's loop would impose.
     stream = C.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
-    marks = HipEvents(args.steps + 1)
+    every = max(1, args.steps // 10)
+    groups = args.steps // every
+    marks = HipEvents(groups + 1)
     t0 = time.perf_counter()
     marks.record(0, stream)
     for i in range(args.steps):
         calls[i % npools].run()
-        marks.record(i + 1, stream)
+        if (i + 1) % every == 0:
+            marks.record((i + 1) // every, stream)
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     ms_per_step = wall / args.steps * 1e3
-    call_ms = [marks.elapsed_ms(i, i + 1) for i in range(args.steps)]
+    call_ms = [marks.elapsed_ms(i, i + 1) / every for i in range(groups)]
     marks.close()
 
     # a second pass with the library's phase events, for the duration of the attention kernel alone (the events
@@ -342,14 +376,15 @@ def run_decode(args, name, cpu_budget=(20.0, 10.0)):
         kernel_name = "decode_paged_kernel"
     out = {
         "metric": "paged_decode_hbm_bandwidth", "value": total_bytes / (ms_per_step * 1e-3) / 1e9, "unit": "GB/s",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
+        "n_gpus": 1, "steps": args.steps, "warmup": warmup, "ms_per_step": ms_per_step,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"{name}: {w['desc']}", "batch": w["B"], "q_heads": w["hq"], "kv_heads": w["hk"],
                    "headdim": w["d"], "page_block_size": w["page"], "sum_keys": int(w["lens"].sum()) + w["B"] * w["snew"],
                    "split_mode": "balanced" if plan.mode == 1 else "grid", "workgroups": plan.num_wgs, "workers": plan.num_workers,
                    "kv_splits": plan.nsplits, "split_keys": plan.split_keys, "cold_cache": f"{npools} pools rotated, {npools * attn_bytes / 2**20:.0f} MiB read per rotation (last-level cache 256 MiB)", "kv_layout": args.kv_layout},
         "us_per_call": ms_per_step * 1e3,
-        "us_per_call_median": median(call_ms) * 1e3,     # HIP events between the calls of the same timed pass
+        "us_per_call_median": median(call_ms) * 1e3,     # HIP events in the same timed pass, `marks_every` calls apart
+        "marks_every": every,
         "pct_of_hbm_peak": 100.0 * total_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,
         "algorithmic_bytes": total_bytes,
         "roofline": {"bound": "hbm", "kernel": kernel_name, "achieved": achieved, "peak": HBM_PEAK_GBPS,
@@ -409,9 +444,7 @@ def run_prefill(args, cpu_budget_s: float = 20.0):
         return ops.varlen_fwd(w["q"], w["k"], w["v"], out, w["cu"], w["cu"], None, None, None, None, w["max_len"],
                               w["max_len"], 0.0, scale, False, True, -1, -1, 0.0, False, None)
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
+    warmup = warm_up(args, lambda i: step())
     # one timed pass: K calls between two device synchronisations; the call is a single kernel, so the events
     # between the calls give its duration as well
     ev = HipEvents(args.steps + 1)
@@ -429,7 +462,7 @@ def run_prefill(args, cpu_budget_s: float = 20.0):
     traffic, traffic_file = traffic_from_profile("c5")
     res = {
         "metric": "varlen_prefill_fwd_tflops", "value": flops / (ms_per_step * 1e-3) / 1e12, "unit": "TFLOP/s",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
+        "n_gpus": 1, "steps": args.steps, "warmup": warmup, "ms_per_step": ms_per_step,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "c5: varlen prefill forward bf16, 16 sequences (lengths U[512,4096] rescaled to 32768 "
                                "tokens), 32q/8kv heads, d=128, causal", "seq_lens": [int(x) for x in w["lens"]],
@@ -502,9 +535,7 @@ def run_mixed(args):
         return ops.varlen_fwd(q, kc, vc, out, cu_q, None, used, None, table, None, max(lens_q), max(lens_k), 0.0, scale,
                               False, True, -1, -1, 0.0, False, None)
 
-    for i in range(args.warmup):
-        step(i)
-    torch.cuda.synchronize()
+    warmup = warm_up(args, step)
     t0 = time.perf_counter()
     for i in range(args.steps):
         step(i)
@@ -514,7 +545,7 @@ def run_mixed(args):
     chunk_flops = 4.0 * 1024 * (16384 - 1024 + 1024 / 2.0) * d * hq
     at_roofs_us = decode_bytes / (HBM_PEAK_GBPS * 1e9) * 1e6 + chunk_flops / (MFMA_BF16_PEAK_TFLOPS * 1e12) * 1e6
     return {"metric": "mixed_batch_step_us", "value": ms * 1e3, "unit": "us", "n_gpus": 1, "steps": args.steps,
-            "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+            "warmup": warmup, "ms_per_step": ms, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
             "dtype": "bf16", "data": "synthetic",
             "config": {"workload": "mixed: token-major step over a paged cache, 63 decode rows (contexts U[1024,8191]) + one "
                                    "1024-token chunk ending a 16384-key context, 32q/8kv d=128 page=256 causal",
@@ -529,22 +560,20 @@ def run_copy(args):
     n = 1 << 30
     src = torch.empty(n, dtype=torch.uint8, device="cuda:0").random_(0, 255)
     dst = torch.empty_like(src)
-    for _ in range(args.warmup):
-        dst.copy_(src)
-    torch.cuda.synchronize()
+    warmup = warm_up(args, lambda i: dst.copy_(src))
     t0 = time.perf_counter()
     for _ in range(args.steps):
         dst.copy_(src)
     torch.cuda.synchronize()
     ms = (time.perf_counter() - t0) / args.steps * 1e3
     return {"metric": "device_copy_bandwidth", "value": 2 * n / (ms * 1e-3) / 1e9, "unit": "GB/s", "n_gpus": 1,
-            "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True,
+            "steps": args.steps, "warmup": warmup, "ms_per_step": ms, "higher_is_better": True,
             "config": {"workload": "copy: 1 GiB torch copy_ (read 1 GiB + write 1 GiB per step)"}}
 
 
 def sub_record(r):
     """What a sub-record of the default line keeps of a config's own line."""
-    keep = ("metric", "value", "unit", "ms_per_step", "us_per_call", "us_per_call_median", "dtype", "roofline",
+    keep = ("metric", "value", "unit", "warmup", "ms_per_step", "us_per_call", "us_per_call_median", "marks_every", "dtype", "roofline",
             "roofline_mfma", "cpu_baseline", "algorithmic_bytes", "algorithmic_flops")
     d = {k: r[k] for k in keep if k in r}
     d["workload"] = r["config"]["workload"]
@@ -557,7 +586,8 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=None,
+                    help="untimed calls in front of the timed ones; default: at least 10 and at least 0.1 s of them")
     ap.add_argument("--config", default="all", help="all = c2 headline plus sub-records of every other baseline config")
     ap.add_argument("--num-splits", type=int, default=0, help="0 = balanced partition (default), n >= 1 = fixed splits")
     ap.add_argument("--kv-layout", default="nhd", choices=["nhd", "hnd"], help="memory layout of the paged caches")
