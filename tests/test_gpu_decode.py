@@ -236,6 +236,34 @@ def test_decode_two_tile_blocks_on_every_kernel(kernel, d, sq, hq, hk, kw):
     assert torch.equal(dev["v_cache"].cpu().view(torch.int16), vc.view(torch.int16))
 
 
+@pytest.mark.parametrize("kernel", list(_TWO_TILE_KERNELS))
+@pytest.mark.parametrize("interleaved", [False, True])
+def test_decode_two_tile_blocks_fp16_with_rotary(kernel, interleaved):
+    """24 rows (three tokens x eight heads of one group) in fp16 with the rotation applied to q and to the appended keys:
+    q rows of one tile belong to different tokens, i.e. different rotation angles and causal bounds."""
+    from helpers import library_env
+    from flash_attn_npu import flash_attn_with_kvcache
+    lens = [515, 64, 0, 1300]
+    case = make_paged_case(4, 16, 2, 128, 64, lens, seqlen_q=3, seqlen_new=3, dtype=torch.float16, seed=91)
+    cos, sin = rotary_tables(2048, 64)
+    cos, sin = cos.to(torch.float16), sin.to(torch.float16)
+    dev = to_dev(case)
+    print("case", kernel, interleaved, flush=True)
+    with library_env(**_TWO_TILE_KERNELS[kernel]):
+        out, lse = flash_attn_with_kvcache(dev["q"], dev["k_cache"], dev["v_cache"], dev["k"], dev["v"],
+                                           rotary_cos=cos.cuda(), rotary_sin=sin.cuda(), cache_seqlens=dev["cache_seqlens"],
+                                           block_table=dev["block_table"], causal=True, rotary_interleaved=interleaved,
+                                           return_softmax_lse=True)
+        torch.cuda.synchronize()
+    kc, vc = case["k_cache"].clone(), case["v_cache"].clone()
+    ref, ref_lse = O.flash_attn_with_kvcache(case["q"], kc, vc, case["k"], case["v"], rotary_cos=cos, rotary_sin=sin,
+                                             cache_seqlens=case["cache_seqlens"], block_table=case["block_table"],
+                                             causal=True, rotary_interleaved=interleaved, mode="fp32")
+    check_out(out, ref, lse, ref_lse, f"{kernel} fp16 rotary")
+    assert torch.equal(dev["k_cache"].cpu().view(torch.int16), kc.view(torch.int16))
+    assert torch.equal(dev["v_cache"].cpu().view(torch.int16), vc.view(torch.int16))
+
+
 @pytest.mark.parametrize("d", [256, 128, 64])
 def test_decode_two_tile_blocks_split_over_many_workers(d):
     """One long sequence, 32 rows: every unit is cut over many workers and merged; the wave-level kernel (two tiles in
